@@ -1,0 +1,78 @@
+"""Build libarhip.so (HIP kernels + C ABI) for gfx950 with hipcc.
+
+    python -m autorust_amd.build          # rebuild if sources are newer
+    python -m autorust_amd.build --force
+
+hipcc cross-compiles without a GPU.  The library lands in-tree
+(autorust_amd/libarhip.so) so that it travels with the source tree.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libarhip.so")
+PROBES = os.path.join(HERE, "probes.hsaco")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+SOURCES = ["device.hip", "flash.hip", "sage_quant.hip"]
+HEADERS = ["arhip_internal.h", "attn_fwd.h", "flash_f32.h", os.path.join("..", "..", "include", "arhip.h")]
+
+# -packed-fp32-ops off: packed fp32 VALU instructions are not used by this build.
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wall", "-Wno-unused-function"]
+
+
+def _newer(target, deps):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        sys.stderr.write(" ".join(cmd) + "\n" + r.stdout + r.stderr)
+        raise RuntimeError("hipcc failed")
+    # the host pass does not know the packed-fp32 feature and says so; that is harmless
+    noise = "is not a recognized feature for this target"
+    out = "\n".join(l for l in (r.stdout + r.stderr).splitlines() if noise not in l)
+    if out.strip():
+        sys.stderr.write(out + "\n")
+
+
+def build(force=False, verbose=False):
+    srcs = [os.path.join(CSRC, s) for s in SOURCES]
+    deps = srcs + [os.path.join(CSRC, h) for h in HEADERS] + [os.path.abspath(__file__)]
+    if force or _newer(LIB, deps):
+        objs = []
+        procs = []
+        for s in srcs:
+            o = s[:-4] + ".o"
+            objs.append(o)
+            cmd = [HIPCC] + FLAGS + ["-c", s, "-o", o]
+            if verbose:
+                print(" ".join(cmd))
+            procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        noise = "is not a recognized feature for this target"
+        for cmd, p in procs:
+            out, _ = p.communicate()
+            out = "\n".join(l for l in out.splitlines() if noise not in l)
+            if p.returncode != 0:
+                sys.stderr.write(" ".join(cmd) + "\n" + out + "\n")
+                raise RuntimeError("hipcc failed")
+            if out.strip():
+                sys.stderr.write(out + "\n")
+        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    probe_src = os.path.join(CSRC, "probes.hip")
+    if os.path.exists(probe_src) and (force or _newer(PROBES, [probe_src])):
+        _run([HIPCC] + FLAGS + ["--genco", probe_src, "-o", PROBES])
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv, verbose=True)
+    print(LIB)

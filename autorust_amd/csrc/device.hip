@@ -1,0 +1,389 @@
+// Device handle, memory, timing and the generic host-kernel launch of libarhip.
+//
+// Stands in for the reference's CUDA device (src/runtime/ops_cuda.rs): context
+// and stream (:140-174), allocator (:595-685), module load and argument
+// encoding (:888-1019).  One stream per handle, default priority.
+#include "arhip_internal.h"
+
+#include <atomic>
+#include <cstring>
+
+static thread_local std::string g_last_error;
+
+int arhip_fail(int code, const char *fmt, ...)
+{
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+extern "C" const char *arhip_last_error(void) { return g_last_error.c_str(); }
+
+static std::atomic<uint64_t> g_selected[ARHIP_K_COUNT];
+
+void arhip_note_selected(int kernel)
+{
+    if (kernel >= 0 && kernel < ARHIP_K_COUNT) g_selected[kernel].fetch_add(1, std::memory_order_relaxed);
+}
+
+extern "C" uint64_t arhip_selections(int kernel)
+{
+    if (kernel < 0 || kernel >= ARHIP_K_COUNT) return 0;
+    return g_selected[kernel].load(std::memory_order_relaxed);
+}
+
+static int prof_event(arhip_device *dev, hipEvent_t *e)
+{
+    if (!dev->prof_pool.empty()) {
+        *e = dev->prof_pool.back();
+        dev->prof_pool.pop_back();
+        return ARHIP_OK;
+    }
+    ARHIP_HIP(hipEventCreate(e));
+    return ARHIP_OK;
+}
+
+int arhip_call_timer::begin()
+{
+    if (dev->prof && kernel >= 0) {
+        if (int rc = prof_event(dev, &p0)) return rc;
+        if (int rc = prof_event(dev, &p1)) return rc;
+        ARHIP_HIP(hipEventRecord(p0, dev->stream));
+    }
+    if (wait) ARHIP_HIP(hipEventRecord(dev->ev0, dev->stream));
+    return ARHIP_OK;
+}
+
+int arhip_call_timer::end()
+{
+    ARHIP_HIP(hipGetLastError());
+    if (p0) {
+        ARHIP_HIP(hipEventRecord(p1, dev->stream));
+        dev->prof_log.push_back({kernel, p0, p1});
+    }
+    if (wait) {
+        ARHIP_HIP(hipEventRecord(dev->ev1, dev->stream));
+        ARHIP_HIP(hipEventSynchronize(dev->ev1));
+        float ms = 0.f;
+        ARHIP_HIP(hipEventElapsedTime(&ms, dev->ev0, dev->ev1));
+        if (secs) *secs = (double)ms * 1e-3;
+    }
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_device_count(int *count)
+{
+    ARHIP_REQUIRE(count, "arhip_device_count: null out pointer");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        n = 0;
+    }
+    *count = n;
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_open(int ordinal, arhip_device **out)
+{
+    ARHIP_REQUIRE(out, "arhip_open: null out pointer");
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return arhip_fail(ARHIP_ENODEVICE, "arhip_open: no HIP device is visible");
+    }
+    if (ordinal < 0 || ordinal >= n)
+        return arhip_fail(ARHIP_ENODEVICE, "arhip_open: ordinal %d out of range (%d devices)", ordinal, n);
+    hipDeviceProp_t prop;
+    ARHIP_HIP(hipGetDeviceProperties(&prop, ordinal));
+    std::string arch = prop.gcnArchName;  // e.g. "gfx950:sramecc+:xnack-"
+    arch = arch.substr(0, arch.find(':'));
+    if (arch != "gfx950")
+        return arhip_fail(ARHIP_ENODEVICE, "arhip_open: device %d is %s; the kernels are built for gfx950 only",
+                          ordinal, arch.c_str());
+    ARHIP_HIP(hipSetDevice(ordinal));
+    arhip_device *d = new arhip_device();
+    d->ordinal = ordinal;
+    d->arch = arch;
+    d->cus = prop.multiProcessorCount;
+    hipError_t e = hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&d->ev0);
+    if (e == hipSuccess) e = hipEventCreate(&d->ev1);
+    if (e == hipSuccess) e = hipEventCreate(&d->tm0);
+    if (e == hipSuccess) e = hipEventCreate(&d->tm1);
+    if (e != hipSuccess) {
+        delete d;
+        return arhip_fail(ARHIP_EHIP, "arhip_open: stream/event creation failed: %s", hipGetErrorString(e));
+    }
+    *out = d;
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_close(arhip_device *dev)
+{
+    if (!dev) return ARHIP_OK;
+    (void)hipSetDevice(dev->ordinal);
+    (void)hipStreamSynchronize(dev->stream);
+    for (auto &kv : dev->modules) {
+        (void)hipModuleUnload(kv.second->mod);
+        delete kv.second;
+    }
+    for (auto &e : dev->prof_log) {
+        (void)hipEventDestroy(e.e0);
+        (void)hipEventDestroy(e.e1);
+    }
+    for (auto e : dev->prof_pool) (void)hipEventDestroy(e);
+    (void)hipEventDestroy(dev->ev0);
+    (void)hipEventDestroy(dev->ev1);
+    (void)hipEventDestroy(dev->tm0);
+    (void)hipEventDestroy(dev->tm1);
+    (void)hipStreamDestroy(dev->stream);
+    delete dev;
+    return ARHIP_OK;
+}
+
+extern "C" const char *arhip_arch(arhip_device *dev) { return dev ? dev->arch.c_str() : ""; }
+extern "C" int arhip_compute_units(arhip_device *dev) { return dev ? dev->cus : 0; }
+extern "C" void *arhip_stream(arhip_device *dev) { return dev ? (void *)dev->stream : nullptr; }
+
+#define ARHIP_DEV(dev)                                              \
+    do {                                                            \
+        ARHIP_REQUIRE((dev) != nullptr, "%s: null device", __func__); \
+        ARHIP_HIP(hipSetDevice((dev)->ordinal));                    \
+    } while (0)
+
+extern "C" int arhip_alloc(arhip_device *dev, size_t bytes, void **dptr)
+{
+    ARHIP_DEV(dev);
+    ARHIP_REQUIRE(dptr, "arhip_alloc: null out pointer");
+    *dptr = nullptr;
+    if (bytes == 0) return ARHIP_OK;  // zero-size buffers have no storage (src/runtime/device.rs:128-203)
+    ARHIP_HIP(hipMalloc(dptr, bytes));
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_free(arhip_device *dev, void *dptr)
+{
+    ARHIP_DEV(dev);
+    if (!dptr) return ARHIP_OK;
+    ARHIP_HIP(hipStreamSynchronize(dev->stream));
+    ARHIP_HIP(hipFree(dptr));
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_copyin(arhip_device *dev, void *dst, const void *host, size_t bytes)
+{
+    ARHIP_DEV(dev);
+    if (bytes == 0) return ARHIP_OK;
+    ARHIP_REQUIRE(dst && host, "arhip_copyin: null pointer");
+    ARHIP_HIP(hipMemcpyAsync(dst, host, bytes, hipMemcpyHostToDevice, dev->stream));
+    ARHIP_HIP(hipStreamSynchronize(dev->stream));  // the host buffer may be reused on return
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_copyout(arhip_device *dev, void *host, const void *src, size_t bytes)
+{
+    ARHIP_DEV(dev);
+    if (bytes == 0) return ARHIP_OK;
+    ARHIP_REQUIRE(host && src, "arhip_copyout: null pointer");
+    ARHIP_HIP(hipMemcpyAsync(host, src, bytes, hipMemcpyDeviceToHost, dev->stream));
+    ARHIP_HIP(hipStreamSynchronize(dev->stream));
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_copy_d2d(arhip_device *dev, void *dst, const void *src, size_t bytes)
+{
+    ARHIP_DEV(dev);
+    if (bytes == 0) return ARHIP_OK;
+    ARHIP_REQUIRE(dst && src, "arhip_copy_d2d: null pointer");
+    ARHIP_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, dev->stream));
+    return ARHIP_OK;
+}
+
+__global__ void __launch_bounds__(256) arhip_fill_zero_kernel(uint32_t *p, size_t words, uint8_t *tail, int tail_bytes)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += stride) p[i] = 0u;
+    if (blockIdx.x == 0 && (int)threadIdx.x < tail_bytes) tail[threadIdx.x] = 0;
+}
+
+extern "C" int arhip_fill_zero(arhip_device *dev, void *dst, size_t bytes)
+{
+    ARHIP_DEV(dev);
+    if (bytes == 0) return ARHIP_OK;
+    ARHIP_REQUIRE(dst && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0, "arhip_fill_zero: dst must be 4-byte aligned");
+    const size_t words = bytes / 4;
+    const int tail = (int)(bytes % 4);
+    size_t blocks = (words + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(arhip_fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, dev->stream,
+                       (uint32_t *)dst, words, (uint8_t *)dst + words * 4, tail);
+    ARHIP_HIP(hipGetLastError());
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_mem_info(arhip_device *dev, size_t *free_bytes, size_t *total_bytes)
+{
+    ARHIP_DEV(dev);
+    size_t f = 0, t = 0;
+    ARHIP_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_sync(arhip_device *dev)
+{
+    ARHIP_DEV(dev);
+    ARHIP_HIP(hipStreamSynchronize(dev->stream));
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_timer_start(arhip_device *dev)
+{
+    ARHIP_DEV(dev);
+    ARHIP_HIP(hipEventRecord(dev->tm0, dev->stream));
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_timer_stop(arhip_device *dev, double *secs)
+{
+    ARHIP_DEV(dev);
+    ARHIP_HIP(hipEventRecord(dev->tm1, dev->stream));
+    ARHIP_HIP(hipEventSynchronize(dev->tm1));
+    float ms = 0.f;
+    ARHIP_HIP(hipEventElapsedTime(&ms, dev->tm0, dev->tm1));
+    if (secs) *secs = (double)ms * 1e-3;
+    return ARHIP_OK;
+}
+
+// Per-kernel device time, the counterpart of the reference's AUTORUST_KPROF
+// (src/runtime/ops_cuda.rs:1004-1016), without a sync per launch: every typed
+// launch is bracketed by two events on the stream while profiling is on.
+extern "C" int arhip_kprof_enable(arhip_device *dev, int on)
+{
+    ARHIP_DEV(dev);
+    dev->prof = on != 0;
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_kprof_collect(arhip_device *dev, int kernel, double *total_secs, uint64_t *launches)
+{
+    ARHIP_DEV(dev);
+    ARHIP_HIP(hipStreamSynchronize(dev->stream));
+    double tot = 0.0;
+    uint64_t n = 0;
+    std::vector<arhip_device::prof_entry> keep;
+    for (auto &e : dev->prof_log) {
+        if (e.kernel != kernel) {
+            keep.push_back(e);
+            continue;
+        }
+        float ms = 0.f;
+        ARHIP_HIP(hipEventElapsedTime(&ms, e.e0, e.e1));
+        tot += (double)ms * 1e-3;
+        ++n;
+        dev->prof_pool.push_back(e.e0);
+        dev->prof_pool.push_back(e.e1);
+    }
+    dev->prof_log.swap(keep);
+    if (total_secs) *total_secs = tot;
+    if (launches) *launches = n;
+    return ARHIP_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Generic launch: the `run_host_kernel` seam (src/runtime/device.rs:383-402).
+
+static uint64_t fnv1a(const void *p, size_t n)
+{
+    const uint8_t *b = (const uint8_t *)p;
+    uint64_t h = 1469598103934665603ull;
+    for (size_t i = 0; i < n; ++i) {
+        h ^= b[i];
+        h *= 1099511628211ull;
+    }
+    return h ^ (uint64_t)n;
+}
+
+extern "C" int arhip_module_load(arhip_device *dev, const void *image, size_t len, void **module)
+{
+    ARHIP_DEV(dev);
+    ARHIP_REQUIRE(image && len > 0 && module, "arhip_module_load: null image or out pointer");
+    const uint64_t key = fnv1a(image, len);
+    auto it = dev->modules.find(key);
+    if (it != dev->modules.end()) {
+        *module = it->second;
+        return ARHIP_OK;
+    }
+    // Keep a private copy of the image alive for as long as the module is loaded.
+    arhip_module_entry *e = new arhip_module_entry();
+    e->image.assign((const char *)image, (const char *)image + len);
+    hipError_t err = hipModuleLoadData(&e->mod, e->image.data());
+    if (err != hipSuccess) {
+        delete e;
+        return arhip_fail(ARHIP_EHIP, "hipModuleLoadData failed: %s", hipGetErrorString(err));
+    }
+    dev->modules[key] = e;
+    *module = e;
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_launch(arhip_device *dev, void *module, const char *name,
+                            const unsigned grid[3], const unsigned block[3],
+                            void *const *bufs, int nbufs,
+                            const int64_t *vals, const int *val_bits, int nvals,
+                            int wait, double *secs)
+{
+    ARHIP_DEV(dev);
+    ARHIP_REQUIRE(module && name && grid && block, "arhip_launch: null argument");
+    ARHIP_REQUIRE(nbufs >= 0 && nvals >= 0 && nbufs + nvals <= 64, "arhip_launch: too many arguments");
+    ARHIP_REQUIRE(nvals == 0 || (vals && val_bits), "arhip_launch: scalar values without widths");
+    arhip_module_entry *m = (arhip_module_entry *)module;
+    hipFunction_t fn;
+    auto it = m->fns.find(name);
+    if (it == m->fns.end()) {
+        ARHIP_HIP(hipModuleGetFunction(&fn, m->mod, name));
+        m->fns[name] = fn;
+    } else {
+        fn = it->second;
+    }
+    // A zero-sized grid is a no-op (the reference clamps negatives to 0, session.rs:241-251).
+    if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) {
+        if (secs) *secs = 0.0;
+        return ARHIP_OK;
+    }
+    ARHIP_REQUIRE(block[0] * block[1] * block[2] >= 1 && block[0] * block[1] * block[2] <= 1024,
+                  "arhip_launch: block of %u threads", block[0] * block[1] * block[2]);
+    void *ptrs[64];
+    int32_t v32[64];
+    int64_t v64[64];
+    void *params[64];
+    int na = 0;
+    for (int i = 0; i < nbufs; ++i, ++na) {
+        ptrs[na] = bufs[i];
+        params[na] = &ptrs[na];
+    }
+    for (int i = 0; i < nvals; ++i, ++na) {
+        if (val_bits[i] == 32) {
+            v32[na] = (int32_t)vals[i];
+            params[na] = &v32[na];
+        } else if (val_bits[i] == 64) {
+            v64[na] = vals[i];
+            params[na] = &v64[na];
+        } else {
+            return arhip_fail(ARHIP_EINVAL, "arhip_launch: scalar %d has width %d (32 or 64)", i, val_bits[i]);
+        }
+    }
+    arhip_call_timer t{dev, wait, secs};
+    if (int rc = t.begin()) return rc;
+    ARHIP_HIP(hipModuleLaunchKernel(fn, grid[0], grid[1], grid[2], block[0], block[1], block[2], 0,
+                                    dev->stream, params, nullptr));
+    return t.end();
+}

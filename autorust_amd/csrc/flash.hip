@@ -1,0 +1,173 @@
+// arhip_flash_fwd / arhip_sage_fwd: argument checks, kernel selection, launch.
+//
+// Mirrors the reference's launch wrappers: cuda_flash::run_ex
+// (src/runtime/cuda_flash.rs:203-254), cuda_flash_bf16::run_ex
+// (src/runtime/cuda_flash_bf16.rs:495-548) and cuda_flash_sage::run_ex
+// (src/runtime/cuda_flash_sage.rs:452-485).
+#include "arhip_internal.h"
+#include "attn_fwd.h"
+#include "flash_f32.h"
+
+using namespace arhip;
+
+extern "C" int arhip_attn_supported(int kind, int64_t n, int64_t d, int dtype)
+{
+    if (n <= 0 || n > (int64_t)1 << 24) return 0;
+    if (d != 64 && d != 128) return 0;
+    switch (kind) {
+    case ARHIP_ATTN_FLASH: return dtype == ARHIP_F32 || dtype == ARHIP_BF16;
+    case ARHIP_ATTN_SAGE: return dtype == ARHIP_F32 || dtype == ARHIP_BF16;
+    default: return 0;  // SDPA is the caller's general path
+    }
+}
+
+static int check_common(const char *fn, arhip_device *dev, const void *q, const void *k, const void *v, const void *o,
+                        const float *mask, int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D)
+{
+    ARHIP_REQUIRE(dev != nullptr, "%s: null device", fn);
+    ARHIP_REQUIRE(q && k && v && o, "%s: null tensor pointer", fn);
+    ARHIP_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && N > 0, "%s: empty shape B=%lld Hq=%lld Hkv=%lld N=%lld", fn,
+                  (long long)B, (long long)Hq, (long long)Hkv, (long long)N);
+    ARHIP_REQUIRE(Hq % Hkv == 0, "%s: Hq=%lld is not a multiple of Hkv=%lld", fn, (long long)Hq, (long long)Hkv);
+    if (D != 64 && D != 128) return arhip_fail(ARHIP_EUNSUPPORTED, "%s: head_dim %lld (64 or 128)", fn, (long long)D);
+    if (N > ((int64_t)1 << 24) || B * Hq > ((int64_t)1 << 24))
+        return arhip_fail(ARHIP_EUNSUPPORTED, "%s: shape too large for 32-bit tile indices", fn);
+    ARHIP_REQUIRE(arhip_aligned16(q) && arhip_aligned16(k) && arhip_aligned16(v) && arhip_aligned16(o),
+                  "%s: q/k/v/o must be 16-byte aligned", fn);
+    ARHIP_REQUIRE(mask == nullptr || (reinterpret_cast<uintptr_t>(mask) & 3u) == 0, "%s: mask must be 4-byte aligned", fn);
+    return ARHIP_OK;
+}
+
+template <int D, int NW, int MODE, bool OUT_F32, bool DBG>
+static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bool has_mask)
+{
+    const dim3 grid((unsigned)p.total), block(NW * 64);
+    if (DBG) {  // debug export: never combined with an additive mask
+        if (causal) hipLaunchKernelGGL((attn_fwd_kernel<D, NW, true, false, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, false, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
+    } else if (causal) {
+        if (has_mask)
+            hipLaunchKernelGGL((attn_fwd_kernel<D, NW, true, true, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((attn_fwd_kernel<D, NW, true, false, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
+    } else {
+        if (has_mask)
+            hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, true, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, false, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
+    }
+}
+
+// Waves per workgroup: 4 (128 queries) when that still fills the chip, else 1
+// (32 queries) so that short sequences spread over more compute units.
+static int pick_nw(arhip_device *dev, int64_t heads, int64_t N)
+{
+    const int64_t wg4 = heads * ((N + 127) / 128);
+    return (wg4 >= 2 * (int64_t)dev->cus) ? 4 : 1;
+}
+
+extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, const void *v, void *o,
+                               const float *mask, const int32_t *kv_len,
+                               int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                               int causal, int dtype, float scale, int wait, double *secs)
+{
+    if (int rc = check_common("arhip_flash_fwd", dev, q, k, v, o, mask, B, Hq, Hkv, N, D)) return rc;
+    ARHIP_REQUIRE(dtype == ARHIP_F32 || dtype == ARHIP_BF16, "arhip_flash_fwd: dtype %d", dtype);
+    ARHIP_HIP(hipSetDevice(dev->ordinal));
+    arhip_call_timer t{dev, wait, secs};
+    t.kernel = (dtype == ARHIP_F32) ? ARHIP_K_FLASH_F32 : ARHIP_K_FLASH_BF16;
+
+    if (dtype == ARHIP_F32) {
+        FlashF32Params fp;
+        fp.q = (const float *)q; fp.k = (const float *)k; fp.v = (const float *)v; fp.o = (float *)o;
+        fp.mask = mask; fp.kv_len = kv_len;
+        fp.Hq = (int)Hq; fp.Hkv = (int)Hkv; fp.N = (int)N;
+        fp.nq = (int)((N + FLASH_F32_BQ - 1) / FLASH_F32_BQ);
+        fp.scale = scale;
+        if (int rc = t.begin()) return rc;
+        const dim3 grid((unsigned)(fp.nq * B * Hq)), block(FLASH_F32_THREADS);
+        if (D == 64) {
+            if (causal) hipLaunchKernelGGL((flash_f32_kernel<64, true>), grid, block, 0, dev->stream, fp);
+            else hipLaunchKernelGGL((flash_f32_kernel<64, false>), grid, block, 0, dev->stream, fp);
+        } else {
+            if (causal) hipLaunchKernelGGL((flash_f32_kernel<128, true>), grid, block, 0, dev->stream, fp);
+            else hipLaunchKernelGGL((flash_f32_kernel<128, false>), grid, block, 0, dev->stream, fp);
+        }
+        arhip_note_selected(ARHIP_K_FLASH_F32);
+        return t.end();
+    }
+
+    AttnParams p = {};
+    p.q = q; p.k = k; p.v = (const uint16_t *)v; p.o = o;
+    p.mask = mask; p.kv_len = kv_len;
+    p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
+    p.bq = p.bk = 1;
+    p.scale = scale;
+    const int nw = (D == 64) ? pick_nw(dev, B * Hq, N) : 4;
+    p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
+    p.total = (int)(p.nq * B * Hq);
+    if (int rc = t.begin()) return rc;
+    if (D == 64) {
+        if (nw == 4) launch_attn<64, 4, MODE_BF16, false, false>(dev->stream, p, causal != 0, mask != nullptr);
+        else launch_attn<64, 1, MODE_BF16, false, false>(dev->stream, p, causal != 0, mask != nullptr);
+    } else {
+        launch_attn<128, 4, MODE_BF16, false, false>(dev->stream, p, causal != 0, mask != nullptr);
+    }
+    arhip_note_selected(ARHIP_K_FLASH_BF16);
+    return t.end();
+}
+
+extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t *k8,
+                              const float *sq, const float *sk, const uint16_t *v, void *o,
+                              const float *mask, const int32_t *kv_len,
+                              int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                              int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
+                              int32_t *dbg_logits, const int32_t dbg_sel[3],
+                              int wait, double *secs)
+{
+    if (int rc = check_common("arhip_sage_fwd", dev, q8, k8, v, o, mask, B, Hq, Hkv, N, D)) return rc;
+    ARHIP_REQUIRE(sq && sk, "arhip_sage_fwd: null scale pointer");
+    ARHIP_REQUIRE(bq >= 1 && bk >= 1, "arhip_sage_fwd: block sizes bq=%lld bk=%lld", (long long)bq, (long long)bk);
+    ARHIP_REQUIRE(out_dtype == ARHIP_F32 || out_dtype == ARHIP_BF16, "arhip_sage_fwd: out_dtype %d", out_dtype);
+    ARHIP_REQUIRE(dbg_logits == nullptr || dbg_sel != nullptr, "arhip_sage_fwd: dbg_logits without dbg_sel");
+    ARHIP_REQUIRE(dbg_logits == nullptr || mask == nullptr, "arhip_sage_fwd: the logits export does not take a mask");
+    ARHIP_HIP(hipSetDevice(dev->ordinal));
+
+    AttnParams p = {};
+    p.q = q8; p.k = k8; p.v = v; p.o = o;
+    p.mask = mask; p.kv_len = kv_len;
+    p.sq = sq; p.sk = sk;
+    p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
+    p.bq = (int)bq; p.bk = (int)bk;
+    p.scale = scale;
+    const int nw = 4;
+    p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
+    p.total = (int)(p.nq * B * Hq);
+    const bool dbg = dbg_logits != nullptr;
+    if (dbg) {
+        p.dbg = dbg_logits;
+        p.dbg_bh = dbg_sel[0]; p.dbg_qt = dbg_sel[1]; p.dbg_kt = dbg_sel[2];
+        ARHIP_REQUIRE(p.dbg_bh >= 0 && p.dbg_bh < B * Hq && p.dbg_qt >= 0 && (int64_t)p.dbg_qt * 32 < N &&
+                          p.dbg_kt >= 0 && (int64_t)p.dbg_kt * 64 < N,
+                      "arhip_sage_fwd: debug tile selector out of range");
+    }
+    const bool c = causal != 0, hm = mask != nullptr, f32o = out_dtype == ARHIP_F32;
+    arhip_call_timer t{dev, wait, secs};
+    t.kernel = ARHIP_K_SAGE;
+    if (int rc = t.begin()) return rc;
+#define SAGE_LAUNCH(DD)                                                                              \
+    do {                                                                                             \
+        if (dbg) {                                                                                   \
+            if (f32o) launch_attn<DD, 4, MODE_I8, true, true>(dev->stream, p, c, hm);                \
+            else launch_attn<DD, 4, MODE_I8, false, true>(dev->stream, p, c, hm);                    \
+        } else {                                                                                     \
+            if (f32o) launch_attn<DD, 4, MODE_I8, true, false>(dev->stream, p, c, hm);               \
+            else launch_attn<DD, 4, MODE_I8, false, false>(dev->stream, p, c, hm);                   \
+        }                                                                                            \
+    } while (0)
+    if (D == 64) SAGE_LAUNCH(64);
+    else SAGE_LAUNCH(128);
+#undef SAGE_LAUNCH
+    arhip_note_selected(ARHIP_K_SAGE);
+    return t.end();
+}

@@ -1,0 +1,83 @@
+// MFMA lane-layout probes, launched through the generic host-kernel seam
+// (arhip_module_load + arhip_launch).  They are to this build what
+// tests/sage_layout_probe.rs is to the reference: a known-answer check that
+// pins the matrix-instruction operand/result layouts the attention kernel
+// relies on.
+//
+// Every probe multiplies A[M x K] (row-major) by B[K x N] (row-major) with ONE
+// MFMA, loading operands with the lane mapping the attention kernel assumes and
+// scattering the result with the assumed result layout.  If the assumed layouts
+// are right, C == A.B exactly (small integers).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+
+// A int8 [32 x 32], B int8 [32 x 32] (k rows), C int32 [32 x 32]
+extern "C" __global__ void probe_i8_32x32x32(const int8_t *A, const int8_t *B, int32_t *C)
+{
+    const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
+    int8_t a[16], b[16];
+    for (int t = 0; t < 16; ++t) {
+        a[t] = A[i * 32 + 16 * h + t];        // row i, k = 16h + t
+        b[t] = B[(16 * h + t) * 32 + i];      // k = 16h + t, column i
+    }
+    i32x4 av, bv;
+    __builtin_memcpy(&av, a, 16);
+    __builtin_memcpy(&bv, b, 16);
+    i32x16 acc;
+    for (int r = 0; r < 16; ++r) acc[r] = 0;
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, acc, 0, 0, 0);
+    for (int r = 0; r < 16; ++r) C[(8 * (r >> 2) + 4 * h + (r & 3)) * 32 + i] = acc[r];
+}
+
+// A bf16 bits [32 x 16], B bf16 bits [16 x 32], C f32 [32 x 32]
+extern "C" __global__ void probe_bf16_32x32x16(const uint16_t *A, const uint16_t *B, float *C)
+{
+    const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
+    uint16_t a[8], b[8];
+    for (int t = 0; t < 8; ++t) {
+        a[t] = A[i * 16 + 8 * h + t];
+        b[t] = B[(8 * h + t) * 32 + i];
+    }
+    bf16x8 av, bv;
+    __builtin_memcpy(&av, a, 16);
+    __builtin_memcpy(&bv, b, 16);
+    f32x16 acc;
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
+    for (int r = 0; r < 16; ++r) C[(8 * (r >> 2) + 4 * h + (r & 3)) * 32 + i] = acc[r];
+}
+
+// The reference's own known answer (tests/sage_layout_probe.rs:73-84):
+// A int8 [16 x 32], B int8 [32 x 8], C int32 [16 x 8], here computed with the
+// 32x32x32 instruction on zero-padded operands.
+extern "C" __global__ void probe_i8_16x8_padded(const int8_t *A, const int8_t *B, int32_t *C)
+{
+    const int lane = threadIdx.x, i = lane & 31, h = lane >> 5;
+    int8_t a[16], b[16];
+    for (int t = 0; t < 16; ++t) {
+        a[t] = (i < 16) ? A[i * 32 + 16 * h + t] : (int8_t)0;
+        b[t] = (i < 8) ? B[(16 * h + t) * 8 + i] : (int8_t)0;
+    }
+    i32x4 av, bv;
+    __builtin_memcpy(&av, a, 16);
+    __builtin_memcpy(&bv, b, 16);
+    i32x16 acc;
+    for (int r = 0; r < 16; ++r) acc[r] = 0;
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, acc, 0, 0, 0);
+    for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+        if (row < 16 && i < 8) C[row * 8 + i] = acc[r];
+    }
+}
+
+// The trivial kernel of tests/host_kernel.rs:28-61: y[i] = x[i] * 3 + 1.
+extern "C" __global__ void probe_axpb(const float *x, float *y, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = x[i] * 3.0f + 1.0f;
+}

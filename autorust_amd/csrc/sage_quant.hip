@@ -1,0 +1,190 @@
+// Sage pre-pass: K mean (smoothing), per-block symmetric int8 quantisation,
+// and the f32 -> bf16 cast of V.  All of it is HBM-bound streaming work.
+//
+// The quantisation rule is the reference's (src/runtime/cuda_flash_sage.rs):
+//   scale = absmax > 0 ? absmax / 127 : 1      (:209-213, :264-268)
+//   inv   = 1 / scale                          (:218, :273)
+//   x8    = clamp(rint(x * inv), -127, 127)    (:124-137), rint = nearest-even
+// hoisted out of the attention kernel (the reference re-quantises K for every
+// query block, :248-278) and applied to blocks of tokens instead of single
+// rows.  Every fp32 operation is a single IEEE operation in a fixed order, so
+// the int8 tensors and scales are bit-reproducible on the CPU.
+#include "arhip_internal.h"
+
+#pragma clang fp contract(off)
+
+namespace {
+
+constexpr int MEAN_CHUNK = 64;  // tokens per partial sum
+
+__device__ __forceinline__ float ld_elem(const float *x, size_t i) { return x[i]; }
+__device__ __forceinline__ float ld_elem(const uint16_t *x, size_t i) { return __uint_as_float((uint32_t)x[i] << 16); }
+
+// part[bh][c][d] = k[64c][d] + k[64c+1][d] + ... in token order
+template <typename T>
+__global__ void k_mean_partial_kernel(const T *x, float *part, int N, int D, int nchunk)
+{
+    const int c = blockIdx.x, bh = blockIdx.y, d = threadIdx.x;
+    const int j0 = c * MEAN_CHUNK;
+    const int j1 = min(N, j0 + MEAN_CHUNK);
+    const size_t base = (size_t)bh * N * D + d;
+    float s = 0.f;
+    for (int j = j0; j < j1; ++j) s += ld_elem(x, base + (size_t)j * D);
+    part[((size_t)bh * nchunk + c) * D + d] = s;
+}
+
+// mean[bh][d] = (part[0] + part[1] + ...) / N in chunk order
+__global__ void k_mean_final_kernel(const float *part, float *mean, int N, int D, int nchunk)
+{
+    const int bh = blockIdx.x, d = threadIdx.x;
+    float tot = 0.f;
+    for (int c = 0; c < nchunk; ++c) tot += part[((size_t)bh * nchunk + c) * D + d];
+    mean[(size_t)bh * D + d] = tot / (float)N;
+}
+
+__device__ __forceinline__ void ld8(const float *x, size_t e, float v[8])
+{
+    const float4 a = *(const float4 *)(x + e), b = *(const float4 *)(x + e + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void ld8(const uint16_t *x, size_t e, float v[8])
+{
+    const uint4 a = *(const uint4 *)(x + e);
+    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+    v[4] = __uint_as_float(a.z << 16); v[5] = __uint_as_float(a.z & 0xffff0000u);
+    v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
+}
+
+// One workgroup per (block of `blk` tokens, head).
+template <typename T, bool SMOOTH>
+__global__ void __launch_bounds__(256) quant_blocks_kernel(const T *x, int8_t *x8, float *scales, const float *mean,
+                                                           int N, int D, int blk, int nblk)
+{
+    __shared__ float red[4];
+    const int bi = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
+    const int r0 = bi * blk;
+    const int r1 = min(N, r0 + blk);
+    const size_t base = ((size_t)bh * N + r0) * D;
+    const int nelem = (r1 - r0) * D;  // multiple of 8
+    const float *mu = SMOOTH ? mean + (size_t)bh * D : nullptr;
+
+    float mx = 0.f;
+    for (int e = tid * 8; e < nelem; e += 256 * 8) {
+        float v[8];
+        ld8(x, base + e, v);
+        const int d = e % D;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float xv = v[i];
+            if (SMOOTH) xv = xv - mu[d + i];
+            mx = fmaxf(mx, fabsf(xv));
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+
+    const float scale = (mx > 0.f) ? mx / 127.0f : 1.f;
+    const float inv = 1.f / scale;
+    if (tid == 0) scales[(size_t)bh * nblk + bi] = scale;
+
+    for (int e = tid * 8; e < nelem; e += 256 * 8) {
+        float v[8];
+        ld8(x, base + e, v);
+        const int d = e % D;
+        uint32_t w[2] = {0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float xv = v[i];
+            if (SMOOTH) xv = xv - mu[d + i];
+            int iv = (int)rintf(xv * inv);
+            iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
+            w[i >> 2] |= ((uint32_t)iv & 0xffu) << ((i & 3) * 8);
+        }
+        *(uint2 *)(x8 + base + e) = make_uint2(w[0], w[1]);
+    }
+}
+
+__global__ void __launch_bounds__(256) cast_bf16_kernel(const float *x, uint16_t *y, size_t n)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const __bf16 b = (__bf16)x[i];  // round-to-nearest-even
+        y[i] = __builtin_bit_cast(uint16_t, b);
+    }
+}
+
+}  // namespace
+
+extern "C" size_t arhip_sage_quant_workspace(int64_t B, int64_t H, int64_t N, int64_t D)
+{
+    if (B <= 0 || H <= 0 || N <= 0 || D <= 0) return 0;
+    const int64_t nchunk = (N + MEAN_CHUNK - 1) / MEAN_CHUNK;
+    return (size_t)(B * H * nchunk * D) * sizeof(float);
+}
+
+extern "C" int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, float *scales, float *mean,
+                                void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
+                                int64_t block, int dtype, int smooth, int wait, double *secs)
+{
+    ARHIP_REQUIRE(dev != nullptr, "arhip_sage_quant: null device");
+    ARHIP_REQUIRE(x && x8 && scales, "arhip_sage_quant: null pointer");
+    ARHIP_REQUIRE(B > 0 && H > 0 && N > 0 && block > 0, "arhip_sage_quant: empty shape");
+    if (D != 64 && D != 128) return arhip_fail(ARHIP_EUNSUPPORTED, "arhip_sage_quant: head_dim %lld (64 or 128)", (long long)D);
+    ARHIP_REQUIRE(dtype == ARHIP_F32 || dtype == ARHIP_BF16, "arhip_sage_quant: dtype %d", dtype);
+    ARHIP_REQUIRE(B * H <= 65535, "arhip_sage_quant: B*H = %lld exceeds the grid limit", (long long)(B * H));
+    ARHIP_REQUIRE(arhip_aligned16(x) && (reinterpret_cast<uintptr_t>(x8) & 7u) == 0,
+                  "arhip_sage_quant: x must be 16-byte and x8 8-byte aligned");
+    ARHIP_REQUIRE(!smooth || (mean && workspace), "arhip_sage_quant: smoothing needs mean and workspace buffers");
+    ARHIP_HIP(hipSetDevice(dev->ordinal));
+    const int nblk = (int)((N + block - 1) / block);
+    const int nchunk = (int)((N + MEAN_CHUNK - 1) / MEAN_CHUNK);
+    const dim3 qgrid((unsigned)nblk, (unsigned)(B * H));
+    arhip_call_timer t{dev, wait, secs};
+    t.kernel = ARHIP_K_SAGE_QUANT;
+    if (int rc = t.begin()) return rc;
+    if (smooth) {
+        const dim3 pgrid((unsigned)nchunk, (unsigned)(B * H));
+        if (dtype == ARHIP_F32)
+            hipLaunchKernelGGL(k_mean_partial_kernel<float>, pgrid, dim3((unsigned)D), 0, dev->stream,
+                               (const float *)x, (float *)workspace, (int)N, (int)D, nchunk);
+        else
+            hipLaunchKernelGGL(k_mean_partial_kernel<uint16_t>, pgrid, dim3((unsigned)D), 0, dev->stream,
+                               (const uint16_t *)x, (float *)workspace, (int)N, (int)D, nchunk);
+        hipLaunchKernelGGL(k_mean_final_kernel, dim3((unsigned)(B * H)), dim3((unsigned)D), 0, dev->stream,
+                           (const float *)workspace, mean, (int)N, (int)D, nchunk);
+        if (dtype == ARHIP_F32)
+            hipLaunchKernelGGL((quant_blocks_kernel<float, true>), qgrid, dim3(256), 0, dev->stream,
+                               (const float *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk);
+        else
+            hipLaunchKernelGGL((quant_blocks_kernel<uint16_t, true>), qgrid, dim3(256), 0, dev->stream,
+                               (const uint16_t *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk);
+    } else {
+        if (dtype == ARHIP_F32)
+            hipLaunchKernelGGL((quant_blocks_kernel<float, false>), qgrid, dim3(256), 0, dev->stream,
+                               (const float *)x, x8, scales, nullptr, (int)N, (int)D, (int)block, nblk);
+        else
+            hipLaunchKernelGGL((quant_blocks_kernel<uint16_t, false>), qgrid, dim3(256), 0, dev->stream,
+                               (const uint16_t *)x, x8, scales, nullptr, (int)N, (int)D, (int)block, nblk);
+    }
+    arhip_note_selected(ARHIP_K_SAGE_QUANT);
+    return t.end();
+}
+
+extern "C" int arhip_cast_bf16(arhip_device *dev, const float *x, uint16_t *y, int64_t n, int wait, double *secs)
+{
+    ARHIP_REQUIRE(dev != nullptr, "arhip_cast_bf16: null device");
+    ARHIP_REQUIRE(n >= 0 && (n == 0 || (x && y)), "arhip_cast_bf16: null pointer");
+    ARHIP_HIP(hipSetDevice(dev->ordinal));
+    arhip_call_timer t{dev, wait, secs};
+    if (int rc = t.begin()) return rc;
+    if (n > 0) {
+        size_t blocks = ((size_t)n + 255) / 256;
+        if (blocks > 16384) blocks = 16384;
+        hipLaunchKernelGGL(cast_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, dev->stream, x, y, (size_t)n);
+    }
+    return t.end();
+}

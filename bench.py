@@ -1,0 +1,272 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-secondary] [--no-cpu]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM.  The headline workload is the Sage INT8 forward at
+B=4, H=32, S=8192, D=128 (the shape the metric and the target are quoted on):
+quantise Q per 128 tokens, smooth + quantise K per 64 tokens, then the int8
+attention kernel.  One JSON line is printed; the other single-GPU
+configurations are reported in its "secondary" array.
+
+Work model: ops = 4*B*H*S^2*D (half for causal); bytes = Q, K, V read once and
+O written once at their storage types.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from autorust_amd import _lib, synth  # noqa: E402
+from autorust_amd.device import BF16, F32, Device  # noqa: E402
+
+PEAK_BF16 = 2500.0   # TFLOP/s, MI355X dense bf16 MFMA
+PEAK_INT8 = 5000.0   # TOP/s, MI355X dense int8 MFMA
+PEAK_HBM = 8000.0    # GB/s, MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def attn_ops(B, H, S, D, causal):
+    return 4.0 * B * H * S * S * D / (2.0 if causal else 1.0)
+
+
+class SageWorkload:
+    """SageAttention INT8 forward: Q ~ N(0,1), K = N(0,1) + per-(head,channel) bias ~ N(0, sigma),
+    V ~ N(0,1); all three stored as bf16; O bf16."""
+
+    def __init__(self, dev, B, H, S, D, causal, sigma, outliers, cfg, bq=128, bk=64):
+        self.dev, self.B, self.H, self.S, self.D, self.causal = dev, B, H, S, D, causal
+        self.bq, self.bk = bq, bk
+        self.name = "sage_int8_b%d_h%d_s%d_d%d%s" % (B, H, S, D, "_causal" if causal else "")
+        n = B * H * S * D
+        base = 1000 * cfg
+        q = synth.normal(base + 1, (B, H, S, D))
+        k = synth.normal(base + 2, (B, H, S, D))
+        k += np.float32(sigma) * synth.normal(base + 4, (1, H, 1, D))
+        if outliers:
+            for t, seed in ((q, base + 6), (k, base + 7)):
+                flat = t.reshape(-1)
+                for o in range(0, n, 1 << 24):
+                    m = min(1 << 24, n - o)
+                    hit = synth.uniform(seed, m, o) < outliers
+                    flat[o:o + m][hit] *= np.float32(20.0)
+        self.host = {"q": q, "k": k}
+        self.dq = dev.from_numpy(synth.to_bf16_bits(q))
+        self.dk = dev.from_numpy(synth.to_bf16_bits(k))
+        v = synth.normal(base + 3, (B, H, S, D))
+        self.host["v"] = v
+        self.dv = dev.from_numpy(synth.to_bf16_bits(v))
+        self.do = dev.alloc(n * 2)
+        self.q8, self.k8 = dev.alloc(n), dev.alloc(n)
+        self.sq = dev.alloc(B * H * ((S + bq - 1) // bq) * 4)
+        self.sk = dev.alloc(B * H * ((S + bk - 1) // bk) * 4)
+        self.mean = dev.alloc(B * H * D * 4)
+        self.ws = dev.alloc(dev.sage_quant_workspace(B, H, S, D))
+        self.ops = attn_ops(B, H, S, D, causal)
+        self.kernel = _lib.K_SAGE
+        # dominant kernel: int8 Q, K (1 B), bf16 V and O (2 B), block scales
+        self.kernel_bytes = n * (1 + 1 + 2 + 2) + 4 * B * H * (S // bq + S // bk)
+        self.dtype = "int8"
+
+    def step(self):
+        d, B, H, S, D = self.dev, self.B, self.H, self.S, self.D
+        d.sage_quant(self.dq, self.q8, self.sq, B, H, S, D, self.bq, BF16, wait=False)
+        d.sage_quant(self.dk, self.k8, self.sk, B, H, S, D, self.bk, BF16, mean=self.mean, workspace=self.ws,
+                     smooth=True, wait=False)
+        d.sage_fwd(self.q8, self.k8, self.sq, self.sk, self.dv, self.do, B, H, H, S, D, self.bq, self.bk,
+                   out_dtype=BF16, causal=self.causal, wait=False)
+
+    def roofline(self, secs):
+        half = self.ops / 2.0
+        t_min = half / (PEAK_INT8 * 1e12) + half / (PEAK_BF16 * 1e12)
+        ach = self.ops / secs / 1e12
+        return {"bound": "mfma", "achieved": ach, "peak": PEAK_INT8, "unit": "TFLOP/s", "frac": ach / PEAK_INT8,
+                "traffic": None, "kernel": "attn_fwd_kernel<int8>", "launch_ms": secs * 1e3,
+                "ops_per_launch": self.ops, "peak_note": "dense int8 MFMA; half of the ops are bf16 (P.V)",
+                "frac_of_mixed_int8_bf16_bound": t_min / secs}
+
+    def free(self):
+        for b in (self.dq, self.dk, self.dv, self.do, self.q8, self.k8, self.sq, self.sk, self.mean, self.ws):
+            b.free()
+
+
+class FlashWorkload:
+    """FlashAttention forward, bf16 or fp32 tensors, Q/K/V ~ N(0,1)."""
+
+    def __init__(self, dev, B, H, S, D, causal, dtype, cfg, kv_lens=False):
+        self.dev, self.B, self.H, self.S, self.D, self.causal, self.dt = dev, B, H, S, D, causal, dtype
+        tag = "bf16" if dtype == BF16 else "f32"
+        self.name = "flash_%s_b%d_h%d_s%d_d%d%s%s" % (tag, B, H, S, D, "_causal" if causal else "",
+                                                       "_kvlen" if kv_lens else "")
+        n = B * H * S * D
+        base = 1000 * cfg
+        arrs = [synth.normal(base + i, (B, H, S, D)) for i in (1, 2, 3)]
+        self.host = dict(zip("qkv", arrs))
+        if dtype == BF16:
+            self.dq, self.dk, self.dv = (dev.from_numpy(synth.to_bf16_bits(a)) for a in arrs)
+        else:
+            self.dq, self.dk, self.dv = (dev.from_numpy(a) for a in arrs)
+        es = 2 if dtype == BF16 else 4
+        self.do = dev.alloc(n * es)
+        self.kv = None
+        if kv_lens:
+            self.kv_host = synth.randint(base + 5, B, S // 2, S)
+            self.kv = dev.from_numpy(self.kv_host)
+        self.ops = attn_ops(B, H, S, D, causal)
+        self.kernel = _lib.K_FLASH_BF16 if dtype == BF16 else _lib.K_FLASH_F32
+        self.kernel_bytes = 4 * n * es
+        self.dtype = tag
+
+    def step(self):
+        self.dev.flash_fwd(self.dq, self.dk, self.dv, self.do, self.B, self.H, self.H, self.S, self.D, self.dt,
+                           kv_len=self.kv, causal=self.causal, wait=False)
+
+    def roofline(self, secs):
+        # short sequences are bandwidth/launch bound, long ones MFMA bound
+        ai = self.ops / self.kernel_bytes
+        if self.dt == BF16 and ai > PEAK_BF16 * 1e12 / (PEAK_HBM * 1e9):
+            ach = self.ops / secs / 1e12
+            return {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_BF16,
+                    "traffic": None, "kernel": "attn_fwd_kernel<bf16>", "launch_ms": secs * 1e3,
+                    "ops_per_launch": self.ops}
+        ach = self.kernel_bytes / secs / 1e9
+        return {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
+                "traffic": None, "kernel": "attn_fwd_kernel<bf16>" if self.dt == BF16 else "flash_f32_kernel",
+                "launch_ms": secs * 1e3, "bytes_per_launch": self.kernel_bytes,
+                "tflops": self.ops / secs / 1e12}
+
+    def free(self):
+        for b in (self.dq, self.dk, self.dv, self.do, self.kv):
+            if b is not None:
+                b.free()
+
+
+def measure(dev, w, steps, warmup):
+    for _ in range(warmup):
+        w.step()
+    dev.sync()
+    dev.kprof_enable(True)
+    for k in range(_lib.K_SAGE_QUANT + 1):
+        dev.kprof_collect(k)
+    dev.timer_start()
+    for _ in range(steps):
+        w.step()
+    total = dev.timer_stop()
+    ksecs, kn = dev.kprof_collect(w.kernel)
+    qsecs, qn = dev.kprof_collect(_lib.K_SAGE_QUANT)
+    dev.kprof_enable(False)
+    ms = total / steps * 1e3
+    res = {"workload": w.name, "ms_per_step": ms, "ops_per_step": w.ops,
+           "tops": w.ops / (total / steps) / 1e12,
+           "roofline": w.roofline(ksecs / max(kn, 1))}
+    if qn:
+        res["prepass_ms_per_step"] = qsecs / steps * 1e3
+    return res
+
+
+def cpu_baseline(w, budget_heads):
+    """The reference CPU backend's attention (oracle/cpu_sdpa_baseline.c) on a head subset of the same inputs."""
+    import oracle
+    oracle.build()
+    heads = max(1, min(budget_heads, w.B * w.H))
+    q = w.host["q"].reshape(-1, w.S, w.D)[:heads][None]
+    k = w.host["k"].reshape(-1, w.S, w.D)[:heads][None]
+    v = w.host["v"].reshape(-1, w.S, w.D)[:heads][None]
+    oracle.cpu_sdpa(q[:, :1], k[:, :1], v[:, :1], causal=w.causal)   # warm-up
+    ts = []
+    threads = 1
+    for _ in range(3):
+        t0 = time.perf_counter()
+        _, threads = oracle.cpu_sdpa(q, k, v, causal=w.causal)
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts)[1]
+    ops = attn_ops(1, heads, w.S, w.D, w.causal)
+    return {"value": ops / t / 1e12, "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+            "sample": "%d of %d (batch,head) slices of the same inputs, fp32 packed-GEMM SDPA "
+                      "(restated RUST/RAYON-equivalent CPU path), median of 3, %.2f s each" % (heads, w.B * w.H, t)}
+
+
+def build_workload(dev, name):
+    if name == "sage":
+        return SageWorkload(dev, 4, 32, 8192, 128, False, 3.0, 0.0, cfg=4)
+    if name == "sage_causal_long":
+        return SageWorkload(dev, 1, 64, 32768, 128, True, 5.0, 0.01, cfg=5)
+    if name == "vit":
+        return FlashWorkload(dev, 8, 12, 197, 64, False, BF16, cfg=2)
+    if name == "decoder":
+        return FlashWorkload(dev, 4, 32, 2048, 128, True, BF16, cfg=3, kv_lens=True)
+    if name == "vit_f32":
+        return FlashWorkload(dev, 1, 12, 197, 64, False, F32, cfg=1)
+    raise SystemExit("unknown workload %r" % name)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="sage",
+                    choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32"])
+    ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    dev = Device(0)
+    log("device", dev.arch, dev.compute_units, "CUs")
+    t0 = time.time()
+    w = build_workload(dev, args.workload)
+    log("inputs for %s ready in %.1f s" % (w.name, time.time() - t0))
+    res = measure(dev, w, args.steps, args.warmup)
+    log(json.dumps(res))
+    cpu = None
+    if not args.no_cpu:
+        heads = {"sage": 2, "sage_causal_long": 1, "decoder": 16, "vit": 96, "vit_f32": 12}[args.workload]
+        cpu = cpu_baseline(w, heads)
+        log(json.dumps(cpu))
+    w.free()
+
+    secondary = []
+    if not args.no_secondary:
+        for name in ("vit", "decoder", "vit_f32", "sage"):
+            if name == args.workload:
+                continue
+            sw = build_workload(dev, name)
+            r = measure(dev, sw, max(args.steps, 20) if name.startswith("vit") else args.steps, args.warmup)
+            sw.free()
+            log(json.dumps(r))
+            secondary.append(r)
+    dev.close()
+
+    line = {
+        "metric": "attention fwd TFLOPS/TOPS + % MFMA peak, ViT-B/16 and S=8192 D=128 shapes",
+        "value": res["tops"], "unit": "TOP/s" if w.dtype == "int8" else "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w.dtype, "data": "synthetic",
+        "config": {"workload": w.name, "B": w.B, "H": w.H, "S": w.S, "D": w.D, "causal": bool(w.causal),
+                   "step": "quantise Q (128-token blocks) + smooth and quantise K (64-token blocks) + int8 attention"
+                           if w.dtype == "int8" else "attention forward"},
+        "roofline": res["roofline"],
+        "cpu_baseline": cpu,
+    }
+    if "prepass_ms_per_step" in res:
+        line["prepass_ms_per_step"] = res["prepass_ms_per_step"]
+    if secondary:
+        line["secondary"] = secondary
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,175 @@
+/*
+ * libarhip — C ABI of the MI355X (gfx950) device and fused-attention kernels.
+ *
+ * This is the boundary a host in any language binds (Rust `libloading`,
+ * ctypes, cgo ...).  It replaces, for the fused attention forward, what the
+ * reference reaches through its Rust device traits; each entry point cites the
+ * reference interface (path:line under the reference tree) it stands in for.
+ *
+ * Conventions
+ *   - every function returns 0 on success and a negative ARHIP_E* code on
+ *     failure; arhip_last_error() returns a thread-local message.  The
+ *     reference's convention is `panic!("TGERR: ...")`; a Rust shim reproduces
+ *     it by panicking on a non-zero return.
+ *   - ARHIP_EUNSUPPORTED is not a failure of the device: it is the typed
+ *     kernels' way of saying "this shape/dtype is not covered", on which the
+ *     reference's dispatcher returns None and the caller runs the general path
+ *     (src/models/flash_attention.rs:470-472).
+ *   - tensors are dense row-major [B, H, N, D] (src/runtime/cuda_flash.rs:199-201),
+ *     caller-owned device memory, 16-byte aligned; K/V may have Hkv heads with
+ *     Hq % Hkv == 0 (grouped-query attention, kv head = head / (Hq/Hkv)).
+ *   - one stream per device handle; calls are asynchronous on it unless `wait`
+ *     is non-zero, in which case the call returns after the kernel finished and
+ *     *secs (if not NULL) receives the elapsed device time in seconds measured
+ *     with events on that stream (src/runtime/device.rs:295-311 `Prog::call`).
+ *   - a handle is used by one host thread at a time.
+ */
+#ifndef ARHIP_H
+#define ARHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct arhip_device arhip_device;
+
+enum {
+    ARHIP_OK = 0,
+    ARHIP_EINVAL = -1,       /* bad argument (shape, alignment, null pointer) */
+    ARHIP_EUNSUPPORTED = -2, /* shape/dtype not covered by the fused kernels */
+    ARHIP_EHIP = -3,         /* a HIP runtime call failed */
+    ARHIP_ENODEVICE = -4     /* no usable gfx950 device */
+};
+
+/* element types of q/k/v/o */
+enum { ARHIP_F32 = 0, ARHIP_BF16 = 1 };
+
+/* attention kinds: src/models/flash_attention.rs:709-717 `AttentionKind` */
+enum { ARHIP_ATTN_SDPA = 0, ARHIP_ATTN_FLASH = 1, ARHIP_ATTN_SAGE = 2 };
+
+/* kernels counted by arhip_selections() */
+enum { ARHIP_K_FLASH_F32 = 0, ARHIP_K_FLASH_BF16 = 1, ARHIP_K_SAGE = 2, ARHIP_K_SAGE_QUANT = 3, ARHIP_K_COUNT = 4 };
+
+const char *arhip_last_error(void);
+
+/* ---- device: src/runtime/ops_cuda.rs:140-174 (open), :1132-1159 (factory) ---- */
+int arhip_device_count(int *count);
+int arhip_open(int ordinal, arhip_device **dev);
+int arhip_close(arhip_device *dev);
+/* "gfx950"; src/runtime/ops_cuda.rs `arch_sm()` */
+const char *arhip_arch(arhip_device *dev);
+int arhip_compute_units(arhip_device *dev);
+
+/* ---- memory: `BackendAllocator`, src/runtime/device.rs:39-62;
+ *      CUDA implementation src/runtime/ops_cuda.rs:595-685 ---- */
+int arhip_alloc(arhip_device *dev, size_t bytes, void **dptr);        /* _alloc: uninitialised */
+int arhip_free(arhip_device *dev, void *dptr);                        /* _free */
+int arhip_copyin(arhip_device *dev, void *dst, const void *host, size_t bytes);  /* _copyin */
+int arhip_copyout(arhip_device *dev, void *host, const void *src, size_t bytes); /* _copyout: syncs first */
+int arhip_copy_d2d(arhip_device *dev, void *dst, const void *src, size_t bytes); /* _copy_into: async, no sync */
+int arhip_fill_zero(arhip_device *dev, void *dst, size_t bytes);      /* fill kernel, async */
+int arhip_mem_info(arhip_device *dev, size_t *free_bytes, size_t *total_bytes);  /* memory_info */
+int arhip_sync(arhip_device *dev);                                    /* Prog::flush */
+/* the handle's stream as a hipStream_t, for callers that order their own work on it */
+void *arhip_stream(arhip_device *dev);
+
+/* ---- timing on the handle's stream (HIP events) ---- */
+int arhip_timer_start(arhip_device *dev);
+int arhip_timer_stop(arhip_device *dev, double *secs); /* records, waits, returns elapsed seconds */
+
+/* ---- per-kernel device time: the reference's AUTORUST_KPROF
+ *      (src/runtime/ops_cuda.rs:1004-1016) without a sync per launch.  While
+ *      enabled, every typed launch below is bracketed by two events on the
+ *      handle's stream; collect() waits for the stream, returns the summed
+ *      elapsed time and the number of launches of `kernel` (ARHIP_K_*) since
+ *      the last collect, and forgets them. ---- */
+int arhip_kprof_enable(arhip_device *dev, int on);
+int arhip_kprof_collect(arhip_device *dev, int kernel, double *total_secs, uint64_t *launches);
+
+/* ---- generic host-kernel launch: `Compiled::run_host_kernel`,
+ *      src/runtime/device.rs:383-402; argument encoding of
+ *      src/runtime/ops_cuda.rs:930-1019 (`CudaProgram::call`) ----
+ * image: a gfx950 code object (hipcc --genco).  Modules are cached per device
+ * by content hash.  args: nbufs device pointers followed by nvals scalars;
+ * val_bits[i] in {32, 64} narrows vals[i] like the reference's signature
+ * dtype does.  grid is in blocks. */
+int arhip_module_load(arhip_device *dev, const void *image, size_t len, void **module);
+int arhip_launch(arhip_device *dev, void *module, const char *name,
+                 const unsigned grid[3], const unsigned block[3],
+                 void *const *bufs, int nbufs,
+                 const int64_t *vals, const int *val_bits, int nvals,
+                 int wait, double *secs);
+
+/* ---- fused attention forward ----
+ * arhip_attn_supported: the `supports` / `supported` gates
+ *   (src/runtime/cuda_flash.rs:145-147, cuda_flash_bf16.rs:431-441,
+ *    cuda_flash_sage.rs:69-74).  Returns 1 or 0.
+ *   The reference's kernels take D == 64 only; these take D in {64, 128}. */
+int arhip_attn_supported(int kind, int64_t n, int64_t d, int dtype);
+
+/* arhip_flash_fwd: `cuda_flash::run_ex` (src/runtime/cuda_flash.rs:203-217,
+ *   fp32 exact mode) and `cuda_flash_bf16::run_ex`
+ *   (src/runtime/cuda_flash_bf16.rs:495-512), selected by dtype.
+ *   o[B,Hq,N,D] = softmax(q.k^T * scale + mask) . v, fp32 accumulate.
+ *   mask: optional additive f32 [N,N] shared by every (b,h), or NULL
+ *         (the reference passes `o` as a dummy, cuda_flash.rs:233-240).
+ *   kv_len: optional device int32[B]; keys j >= kv_len[b] are excluded
+ *         (per-batch key-padding mask).  No counterpart in the reference's
+ *         kernels, which only bound keys by N; NULL means N for every batch.
+ *   causal: keys j > i are excluded (cuda_flash.rs:112).
+ *   scale: the reference hard-codes 0.125 = 1/sqrt(64) (cuda_flash.rs:89);
+ *         pass 1/sqrt(D). */
+int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, const void *v, void *o,
+                    const float *mask, const int32_t *kv_len,
+                    int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                    int causal, int dtype, float scale, int wait, double *secs);
+
+/* arhip_sage_quant: the quantiser of the Sage kernel hoisted into a pre-pass
+ *   (the reference quantises inside the attention kernel, K once per query
+ *   block: src/runtime/cuda_flash_sage.rs:201-223, 248-278).
+ *   x [B,H,N,D] (f32 or bf16, `dtype`) -> x8 int8 [B,H,N,D] and
+ *   scales f32 [B,H,ceil(N/block)], in blocks of `block` tokens:
+ *     scale = absmax > 0 ? absmax/127 : 1;  x8 = clamp(rint(x * (1/scale)), +-127)
+ *   (cuda_flash_sage.rs:124-137, 209-222; block == 1 is the reference's rule).
+ *   smooth != 0 first subtracts the per-(b,h,channel) mean over the N tokens
+ *   (K smoothing; not in the reference) and writes that mean to
+ *   mean f32 [B,H,D] (required then, else may be NULL).
+ *   workspace: device scratch of arhip_sage_quant_workspace(B,H,N,D) bytes
+ *   when smooth != 0 (may be NULL otherwise). */
+size_t arhip_sage_quant_workspace(int64_t B, int64_t H, int64_t N, int64_t D);
+int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, float *scales, float *mean,
+                     void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
+                     int64_t block, int dtype, int smooth, int wait, double *secs);
+
+/* arhip_cast_bf16: f32 -> bf16 round-to-nearest-even of n elements (the V
+ *   operand of the Sage kernel: cuda_flash_sage.rs:99-103, 257-262). */
+int arhip_cast_bf16(arhip_device *dev, const float *x, uint16_t *y, int64_t n, int wait, double *secs);
+
+/* arhip_sage_fwd: `cuda_flash_sage::run_ex` (src/runtime/cuda_flash_sage.rs:452-485)
+ *   on pre-quantised operands: int8 q8/k8 with block scales sq [B,Hq,ceil(N/bq)],
+ *   sk [B,Hkv,ceil(N/bk)], v bf16 [B,Hkv,N,D]; logits int32 = q8.k8^T,
+ *   s = (float)logit * ((sq*sk)*scale) (cuda_flash_sage.rs:315-322), fp32
+ *   softmax, P and V in bf16, fp32 accumulate; o is f32 (out_dtype ARHIP_F32,
+ *   the reference's convention) or bf16.
+ *   dbg_logits: optional device int32 [32 x 64] receiving the raw logits of the
+ *   tile (query rows dbg_sel[1]*32.., keys dbg_sel[2]*64..) of head dbg_sel[0]
+ *   (b*Hq+h), row-major [query][key]; pass NULL in production. */
+int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t *k8,
+                   const float *sq, const float *sk, const uint16_t *v, void *o,
+                   const float *mask, const int32_t *kv_len,
+                   int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                   int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
+                   int32_t *dbg_logits, const int32_t dbg_sel[3],
+                   int wait, double *secs);
+
+/* dispatch counters: `selections()` (src/runtime/cuda_flash_bf16.rs:443-461,
+ *   cuda_flash_sage.rs:417-436) */
+uint64_t arhip_selections(int kernel);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARHIP_H */

@@ -1,0 +1,125 @@
+"""FlashAttention forward on the GPU (through the C ABI) against the CPU oracle.
+
+Mirrors the reference's kernel tests: tests/flash_cuda.rs (fp32 exact, < 2e-5),
+tests/flash_cuda_bf16.rs (bf16 vs the bf16-emulating reference, < 5e-3, for
+n in {1,7,8,31,32,33,63,64,65,100,224,789}) and tests/flash_cuda_masks.rs
+(causal / additive mask / GQA, 2e-4 fp32 and 5e-3 bf16), at D = 64 as there and
+at D = 128, plus the per-batch key lengths of the decoder configuration.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from autorust_amd import _lib, synth
+from autorust_amd.device import BF16, F32, selections
+from gpu_util import fill_qkv, ref_mask, run_flash
+
+pytestmark = pytest.mark.gpu
+
+N_LIST = [1, 7, 8, 31, 32, 33, 63, 64, 65, 100, 224, 789]  # tests/flash_cuda_bf16.rs:120
+MASK_CASES = [  # tests/flash_cuda_masks.rs:237-244: label, b, hq, hkv, n, causal, has_mask
+    ("causal", 1, 2, 2, 100, True, False),
+    ("mask", 1, 2, 2, 64, False, True),
+    ("causal+mask", 1, 2, 2, 100, True, True),
+    ("gqa", 2, 4, 2, 64, False, False),
+    ("gqa+causal", 2, 4, 2, 100, True, False),
+    ("gqa+mask", 2, 4, 1, 64, False, True),
+]
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("N", N_LIST)
+def test_bf16_matches_reference(dev, N, D):
+    q, k, v = fill_qkv(1, 6, 6, N, D)
+    before = selections(_lib.K_FLASH_BF16)
+    got = run_flash(dev, q, k, v, BF16)
+    assert selections(_lib.K_FLASH_BF16) == before + 1
+    want = oracle.attn_bf16(q, k, v)
+    assert np.abs(got - want).max() < 5e-3          # tests/flash_cuda_bf16.rs:131
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("N", [1, 33, 64, 197, 789])
+def test_f32_exact_matches_reference(dev, N, D):
+    q, k, v = fill_qkv(1, 6, 6, N, D)               # tests/flash_cuda.rs: (1,6,789,64)
+    got = run_flash(dev, q, k, v, F32)
+    want = oracle.flash_f32(q, k, v)
+    assert np.abs(got - want).max() < 2e-5          # tests/flash_cuda.rs:74
+    truth = oracle.sdpa_f64(q, k, v)
+    assert (np.abs(got - truth) / np.maximum(np.abs(truth), 1)).max() <= 1e-5
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("case", MASK_CASES, ids=lambda c: c[0])
+def test_causal_mask_gqa(dev, case, D):
+    _, B, Hq, Hkv, N, causal, has_mask = case
+    q, k, v = fill_qkv(B, Hq, Hkv, N, D)
+    mask = ref_mask(N).reshape(N, N) if has_mask else None
+    got = run_flash(dev, q, k, v, BF16, mask=mask, causal=causal)
+    want = oracle.attn_bf16(q, k, v, mask=mask, causal=causal)
+    assert np.abs(got - want).max() < 5e-3          # tests/flash_cuda_masks.rs:289 (bf16)
+    got = run_flash(dev, q, k, v, F32, mask=mask, causal=causal)
+    want = oracle.flash_f32(q, k, v, mask=mask, causal=causal)
+    assert np.abs(got - want).max() < 2e-4          # tests/flash_cuda_masks.rs:289 (f32)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("dtype", [BF16, F32])
+def test_random_inputs_causal_and_key_lengths(dev, dtype, D):
+    B, Hq, Hkv, N = 3, 4, 2, 300
+    q, k, v = synth.normal(101, (B, Hq, N, D)), synth.normal(102, (B, Hkv, N, D)), synth.normal(103, (B, Hkv, N, D))
+    kv_len = np.array([150, 300, 1], np.int32)
+    got = run_flash(dev, q, k, v, dtype, kv_len=kv_len, causal=True)
+    truth = oracle.sdpa_f64(q, k, v, kv_len=kv_len, causal=True)
+    if dtype == F32:
+        assert (np.abs(got - truth) / np.maximum(np.abs(truth), 1)).max() <= 1e-5
+    else:
+        want = oracle.attn_bf16(q, k, v, kv_len=kv_len, causal=True)
+        assert np.abs(got - want).max() < 1.6e-2     # two bf16 steps at |o| ~ 2..4
+        assert np.abs(got - truth).max() <= 2e-2 * max(1.0, np.abs(truth).max())
+    # non-causal with key lengths
+    got = run_flash(dev, q, k, v, dtype, kv_len=kv_len)
+    truth = oracle.sdpa_f64(q, k, v, kv_len=kv_len)
+    tol = 1e-5 if dtype == F32 else 2e-2
+    assert (np.abs(got - truth) / np.maximum(np.abs(truth), 1)).max() <= tol
+
+
+def test_edge_cases(dev):
+    D = 64
+    q, k, v = synth.normal(111, (1, 2, 40, D)), synth.normal(112, (1, 2, 40, D)), synth.normal(113, (1, 2, 40, D))
+    # kv_len == 0: no key contributes, l == 0, output is zero (acc * (l > 0 ? 1/l : 0))
+    for dtype in (BF16, F32):
+        got = run_flash(dev, q, k, v, dtype, kv_len=np.array([0], np.int32))
+        assert not got.any()
+    # a row masked with -inf everywhere yields zeros (not NaN), the others are untouched
+    mask = np.zeros((40, 40), np.float32)
+    mask[5, :] = -np.inf
+    for dtype, tol in ((BF16, 2e-2), (F32, 1e-5)):
+        got = run_flash(dev, q, k, v, dtype, mask=mask)
+        assert not got[:, :, 5].any()
+        truth = oracle.sdpa_f64(q, k, v)
+        assert np.abs(np.delete(got, 5, 2) - np.delete(truth, 5, 2)).max() <= tol * 4
+    # scale is a parameter
+    got = run_flash(dev, q, k, v, F32, scale=0.3)
+    truth = oracle.sdpa_f64(q, k, v, scale=0.3)
+    assert np.abs(got - truth).max() < 1e-5
+
+
+def test_unsupported_shapes_are_declined_not_faked(dev):
+    # head_dim 32: the dispatcher's cue to use the general path (flash_attention.rs:470-472)
+    q = dev.alloc(4096)
+    with pytest.raises(_lib.Unsupported):
+        dev.flash_fwd(q, q, q, q, 1, 1, 1, 8, 32, BF16)
+    with pytest.raises(_lib.ArhipError):
+        dev.flash_fwd(q, q, q, q, 1, 3, 2, 8, 64, BF16)      # Hq % Hkv != 0
+    with pytest.raises(_lib.ArhipError):
+        dev.flash_fwd(q.ptr + 2, q, q, q, 1, 1, 1, 8, 64, BF16)  # misaligned
+    q.free()
+
+
+def test_bf16_is_deterministic(dev):
+    # tests/flash_cuda_bf16.rs:181-268 asserts bit-identical outputs across launches
+    q, k, v = synth.normal(121, (2, 6, 789, 64)), synth.normal(122, (2, 6, 789, 64)), synth.normal(123, (2, 6, 789, 64))
+    a = run_flash(dev, q, k, v, BF16)
+    b = run_flash(dev, q, k, v, BF16)
+    assert np.array_equal(a, b)

@@ -1,0 +1,115 @@
+"""SageAttention-style int8 path on the GPU against the CPU oracle.
+
+Bit-exact: int8 tensors, block scales, K mean, bf16 V, int32 QK^T logits.
+Within tolerance: outputs vs the oracle's emulation of the kernel (< 2e-3,
+tests/sage_int8.rs:148) and vs the float64 result (<= 2e-2).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from autorust_amd import _lib, synth
+from autorust_amd.device import BF16, F32, selections
+from gpu_util import fill_qkv, run_sage
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(B, Hq, Hkv, N, D, bias=3.0, seed=200):
+    q = synth.normal(seed + 1, (B, Hq, N, D))
+    k = synth.normal(seed + 2, (B, Hkv, N, D)) + np.float32(bias) * synth.normal(seed + 4, (1, Hkv, 1, D))
+    v = synth.normal(seed + 3, (B, Hkv, N, D))
+    return q, k.astype(np.float32), v
+
+
+def _check_bits(r, q, k, v, bq, bk, smooth, in_dtype=F32):
+    if in_dtype == BF16:
+        q, k = oracle.bf16_round(q), oracle.bf16_round(k)
+    mu = oracle.k_mean(k) if smooth else None
+    q8, sq = oracle.quant_blocks(q, bq)
+    k8, sk = oracle.quant_blocks(k, bk, sub=mu)
+    assert np.array_equal(r["sq"], sq) and np.array_equal(r["sk"], sk)
+    assert np.array_equal(r["q8"], q8) and np.array_equal(r["k8"], k8)
+    if smooth:
+        assert np.array_equal(r["mean"], mu)
+    assert np.array_equal(r["vb"], oracle.bf16_round(v))
+    return q8, sq, k8, sk
+
+
+@pytest.mark.parametrize("N", [1, 8, 33, 100, 789])   # tests/sage_int8.rs:133
+def test_int8_sage_matches_reference_per_row(dev, N):
+    """The reference's own case: (1, 6, n, 64), fill data, per-row / per-key scales, no smoothing."""
+    q, k, v = fill_qkv(1, 6, 6, N, 64)
+    before = selections(_lib.K_SAGE)
+    r = run_sage(dev, q, k, v, 1, 1, smooth=False)
+    assert selections(_lib.K_SAGE) == before + 1
+    q8, sq, k8, sk = _check_bits(r, q, k, v, 1, 1, False)
+    want = oracle.sage(q8, k8, sq, sk, v, 1, 1)
+    assert np.abs(r["out"] - want).max() < 2e-3       # tests/sage_int8.rs:148
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("N,causal", [(256, False), (300, True), (1000, False), (1000, True), (64, False), (129, True)])
+def test_block_quantised_smoothed(dev, N, causal, D):
+    B, Hq, Hkv, bq, bk = 2, 4, 2, 128, 64
+    q, k, v = _inputs(B, Hq, Hkv, N, D)
+    # a tile on or below the diagonal so that the causal kernel visits it
+    qt, kt = (N - 1) // 32, ((N - 1) // 64) // 2
+    sel = (B * Hq - 1, qt, kt)
+    r = run_sage(dev, q, k, v, bq, bk, smooth=True, causal=causal, dbg_sel=sel)
+    q8, sq, k8, sk = _check_bits(r, q, k, v, bq, bk, True)
+    b, h = divmod(sel[0], Hq)
+    i0, i1, j0, j1 = qt * 32, min(N, qt * 32 + 32), kt * 64, min(N, kt * 64 + 64)
+    want_logits = oracle.logits_i32(q8[b, h], k8[b, h // (Hq // Hkv)], i0, i1, j0, j1)
+    assert np.array_equal(r["logits"][:i1 - i0, :j1 - j0], want_logits)
+    want = oracle.sage(q8, k8, sq, sk, v, bq, bk, causal=causal)
+    assert np.abs(r["out"] - want).max() < 2e-3
+    if not causal:
+        truth = oracle.sdpa_f64(q, k, v)
+        assert np.abs(r["out"] - truth).max() <= 2e-2
+
+
+def test_bf16_inputs_and_bf16_output(dev):
+    B, Hq, Hkv, N, D, bq, bk = 1, 4, 4, 512, 128, 128, 64
+    q, k, v = _inputs(B, Hq, Hkv, N, D)
+    r = run_sage(dev, q, k, v, bq, bk, smooth=True, in_dtype=BF16, out_dtype=BF16)
+    q8, sq, k8, sk = _check_bits(r, q, k, v, bq, bk, True, in_dtype=BF16)
+    want = oracle.sage(q8, k8, sq, sk, v, bq, bk, round_out=True)
+    assert np.abs(r["out"] - want).max() < 8e-3       # one bf16 step at |o| < 1
+    truth = oracle.sdpa_f64(q, k, v)
+    assert np.abs(r["out"] - truth).max() <= 2e-2
+
+
+def test_smoothing_reduces_error(dev):
+    """K = N(0,1) + per-channel bias: without smoothing the bias eats the int8 range."""
+    B, Hq, Hkv, N, D = 1, 2, 2, 512, 128
+    q, k, v = _inputs(B, Hq, Hkv, N, D, bias=3.0)
+    truth = oracle.sdpa_f64(q, k, v)
+    e_smooth = np.abs(run_sage(dev, q, k, v, 128, 64, smooth=True)["out"] - truth).max()
+    e_plain = np.abs(run_sage(dev, q, k, v, 128, 64, smooth=False)["out"] - truth).max()
+    assert e_smooth <= 2e-2
+    assert e_smooth < e_plain
+
+
+def test_mask_and_key_lengths(dev):
+    B, Hq, Hkv, N, D = 2, 2, 1, 200, 64
+    q, k, v = _inputs(B, Hq, Hkv, N, D, bias=1.0)
+    mask = (synth.normal(301, (N, N)) * 0.5).astype(np.float32)
+    kv_len = np.array([200, 77], np.int32)
+    r = run_sage(dev, q, k, v, 128, 64, smooth=True, mask=mask, kv_len=kv_len, causal=True)
+    q8, sq, k8, sk = _check_bits(r, q, k, v, 128, 64, True)
+    want = oracle.sage(q8, k8, sq, sk, v, 128, 64, mask=mask, kv_len=kv_len, causal=True)
+    assert np.abs(r["out"] - want).max() < 2e-3
+
+
+def test_zero_block_and_outliers(dev):
+    B, H, N, D = 1, 1, 256, 64
+    q, k, v = _inputs(B, H, H, N, D, bias=0.0)
+    q[0, 0, :128] = 0.0                       # an all-zero block: scale guard = 1
+    k[0, 0, 70, 5] = 500.0                    # an outlier stretches one block's scale
+    r = run_sage(dev, q, k, v, 128, 64, smooth=False)
+    q8, sq, k8, sk = _check_bits(r, q, k, v, 128, 64, False)
+    assert sq[0, 0, 0] == 1.0 and not q8[0, 0, :128].any()
+    assert k8[0, 0, 70, 5] == 127
+    want = oracle.sage(q8, k8, sq, sk, v, 128, 64)
+    assert np.abs(r["out"] - want).max() < 2e-3

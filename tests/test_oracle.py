@@ -1,0 +1,272 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Sources of truth used here, none of which is the oracle's own formula retyped:
+  - the reference's six SDPA vectors (tests/golden/sdpa_golden.json, from the
+    reference's tests/attention_golden.rs; tolerance of tests/nn_attention.rs:20)
+  - torch's CPU scaled_dot_product_attention and torch.bfloat16 casts (library)
+  - float64 evaluation, exact integer arithmetic, and special cases with a
+    known closed-form answer
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from autorust_amd import synth
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "sdpa_golden.json")
+
+
+def _golden_cases():
+    with open(GOLDEN) as fh:
+        return json.load(fh)["cases"]
+
+
+def _as4d(c):
+    """3-D inputs are [batch, n, d]: give them a head axis of one."""
+    def arr(key):
+        a = np.array(c[key], np.float32).reshape(c[key + "_shape"])
+        return a[:, None] if a.ndim == 3 else a
+    q, k, v = arr("q"), arr("k"), arr("v")
+    mask = None
+    if c["mask_shape"]:
+        m = np.array(c["mask"], np.float32).reshape(c["mask_shape"])
+        if c["mask_bool"]:
+            m = np.where(m != 0, np.float32(0), np.float32(-np.inf))
+        mask = m[:, None] if (m.ndim == 3 and len(c["q_shape"]) == 3) else m
+    want = np.array(c["out"], np.float32).reshape(c["out_shape"])
+    want = want[:, None] if want.ndim == 3 else want
+    return q, k, v, mask, want
+
+
+def _close_ref(got, want, rtol=1e-5):
+    # tests/nn_attention.rs:11-24
+    return np.all(np.abs(got - want) <= rtol * np.maximum(np.abs(want), 1.0))
+
+
+@pytest.mark.parametrize("case", _golden_cases(), ids=lambda c: c["name"])
+@pytest.mark.parametrize("fn", ["sdpa_f32", "sdpa_f64", "flash_f32"])
+def test_reference_golden_vectors(case, fn):
+    q, k, v, mask, want = _as4d(case)
+    got = getattr(oracle, fn)(q, k, v, mask=mask, causal=case["is_causal"])
+    assert got.shape == want.shape
+    assert _close_ref(got, want), (case["name"], fn, np.abs(got - want).max())
+
+
+@pytest.mark.parametrize("causal,use_mask,hkv", [(False, False, 4), (True, False, 4), (False, True, 4),
+                                                 (False, False, 2), (True, False, 1)])
+def test_against_torch_cpu_sdpa(causal, use_mask, hkv):
+    torch = pytest.importorskip("torch")
+    B, Hq, N, D = 2, 4, 37, 64
+    q, k, v = synth.normal(11, (B, Hq, N, D)), synth.normal(12, (B, hkv, N, D)), synth.normal(13, (B, hkv, N, D))
+    mask = (synth.normal(14, (N, N)) * 2).astype(np.float32) if use_mask else None
+    rep = Hq // hkv
+    tq, tk, tv = (torch.from_numpy(x).double() for x in (q, np.repeat(k, rep, 1), np.repeat(v, rep, 1)))
+    tm = None if mask is None else torch.from_numpy(mask).double()
+    want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, attn_mask=tm, is_causal=causal).numpy()
+    for fn, tol in (("sdpa_f64", 2e-7), ("sdpa_f32", 1e-5), ("flash_f32", 1e-5)):
+        got = getattr(oracle, fn)(q, k, v, mask=mask, causal=causal)
+        err = np.abs(got - want) / np.maximum(np.abs(want), 1.0)
+        assert err.max() <= tol, (fn, err.max())
+
+
+def test_kv_len_is_a_key_padding_mask():
+    # keys >= kv_len[b] excluded == attention over the truncated K/V (closed form)
+    B, H, N, D = 2, 2, 50, 64
+    q, k, v = synth.normal(1, (B, H, N, D)), synth.normal(2, (B, H, N, D)), synth.normal(3, (B, H, N, D))
+    kv = np.array([17, 50], np.int32)
+    for fn in ("sdpa_f32", "sdpa_f64", "flash_f32", "attn_bf16"):
+        got = getattr(oracle, fn)(q, k, v, kv_len=kv)
+        for b in range(B):
+            L = kv[b]
+            # truncated problem: same queries, first L keys; take matching rows
+            kt, vt = np.zeros_like(k[b:b + 1]), np.zeros_like(v[b:b + 1])
+            sub = getattr(oracle, fn)(np.ascontiguousarray(q[b:b + 1, :, :L]), np.ascontiguousarray(k[b:b + 1, :, :L]),
+                                      np.ascontiguousarray(v[b:b + 1, :, :L]))
+            assert np.abs(got[b, :, :L] - sub[0]).max() <= (1e-2 if fn == "attn_bf16" else 2e-6), fn
+
+
+def test_rows_subset_matches_full():
+    B, H, N, D = 1, 2, 70, 64
+    q, k, v = synth.normal(4, (B, H, N, D)), synth.normal(5, (B, H, N, D)), synth.normal(6, (B, H, N, D))
+    rows = np.array([0, 3, 69, 31], np.int32)
+    for fn in ("sdpa_f32", "sdpa_f64", "flash_f32", "attn_bf16"):
+        full = getattr(oracle, fn)(q, k, v, causal=True)
+        part = getattr(oracle, fn)(q, k, v, causal=True, rows=rows)
+        assert np.array_equal(part, full[:, :, rows]), fn
+
+
+def test_flash_sentinel_semantics():
+    """A row whose visited keys are all masked with the finite sentinel averages the
+    visited V rows (src/runtime/cuda_flash.rs:105-125); an additive -inf mask on every
+    key gives l == 0 and therefore zeros (cuda_flash.rs:138)."""
+    N, D = 40, 64
+    q, k, v = synth.normal(7, (1, 1, N, D)), synth.normal(8, (1, 1, N, D)), synth.normal(9, (1, 1, N, D))
+    mask = np.zeros((N, N), np.float32)
+    mask[5, :] = -np.inf
+    got = oracle.flash_f32(q, k, v, mask=mask)
+    assert np.array_equal(got[0, 0, 5], np.zeros(D, np.float32))
+    ok = oracle.sdpa_f64(q, k, v)
+    assert np.abs(np.delete(got, 5, 2) - np.delete(ok, 5, 2)).max() < 1e-5
+    # a constant finite mask on every key of a row == plain softmax of that row (shift invariance)
+    mask2 = np.zeros((N, N), np.float32)
+    mask2[7, :] = -32.0
+    got2 = oracle.flash_f32(q, k, v, mask=mask2)
+    assert np.abs(got2 - ok).max() < 1e-4
+
+
+def test_bf16_rounding_matches_torch():
+    torch = pytest.importorskip("torch")
+    x = np.concatenate([synth.normal(21, (4096,)) * 100, synth.normal(22, (4096,)) * 1e-3,
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38, np.inf, -np.inf], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(oracle.bf16_round(x), want)
+    assert np.array_equal(oracle.bf16_from_bits(oracle.bf16_bits(x)), want)
+    assert np.array_equal(synth.to_bf16_bits(x), oracle.bf16_bits(x))
+    assert np.array_equal(synth.from_bf16_bits(synth.to_bf16_bits(x)), want)
+    # ties go to even: 1 + 2^-8 is halfway between 1 and 1 + 2^-7
+    assert oracle.bf16_round(np.array([1.00390625], np.float32))[0] == 1.0
+    assert oracle.bf16_round(np.array([1.01171875], np.float32))[0] == np.float32(1.015625)
+
+
+@pytest.mark.parametrize("causal,use_mask,hkv", [(False, False, 2), (True, False, 2), (True, True, 1)])
+def test_bf16_reference_against_torch_casts(causal, use_mask, hkv):
+    """Rounding points of the bf16-emulating reference (tests/flash_cuda_masks.rs:41-104),
+    re-derived with torch tensor ops and torch's own bf16 casts."""
+    torch = pytest.importorskip("torch")
+    B, Hq, N, D = 1, 2, 45, 64
+    q, k, v = synth.normal(31, (B, Hq, N, D)), synth.normal(32, (B, hkv, N, D)), synth.normal(33, (B, hkv, N, D))
+    mask = (synth.normal(34, (N, N))).astype(np.float32) if use_mask else None
+    bf = lambda t: t.to(torch.bfloat16).to(torch.float32)
+    rep = Hq // hkv
+    tq = bf(torch.from_numpy(q))
+    tk = bf(torch.from_numpy(np.repeat(k, rep, 1)))
+    tv = bf(torch.from_numpy(np.repeat(v, rep, 1)))
+    s = (tq.double() @ tk.double().transpose(-1, -2)).float() * np.float32(1.0 / np.sqrt(np.float32(D)))
+    if mask is not None:
+        s = s + torch.from_numpy(mask)
+    if causal:
+        s = s.masked_fill(torch.ones(N, N, dtype=torch.bool).triu(1), float("-inf"))
+    p = torch.exp(s - s.max(-1, keepdim=True).values)
+    want = bf((bf(p).double() @ tv.double()).float() / p.sum(-1, keepdim=True)).numpy()
+    got = oracle.attn_bf16(q, k, v, mask=mask, causal=causal)
+    # one bf16 ulp of slack for fp32 summation-order differences that land on a rounding boundary
+    assert np.abs(got - want).max() <= 2.0 ** -7 * np.abs(want).max()
+    assert np.mean(got != want) < 0.02
+
+
+def test_quantiser_known_values():
+    """Closed-form cases of the rule of src/runtime/cuda_flash_sage.rs:124-137,209-222."""
+    D = 64
+    x = np.zeros((1, 1, 3, D), np.float32)
+    # row 0: absmax 127 -> scale exactly 1 -> q = rint(x), ties to even, clamp at +-127
+    x[0, 0, 0, :8] = [127.0, -127.0, 0.5, 1.5, 2.5, -0.5, -1.5, 63.49]
+    # row 1: all zero -> scale 1 (guard), q 0
+    # row 2: absmax 2.54 -> scale 0.02 -> 1.27 -> 63.5 -> 64 (tie to even) or 63 depending on fp32 rounding
+    x[0, 0, 2, :3] = [2.54, -2.54, 1.27]
+    q, s = oracle.quant_blocks(x, 1)
+    assert s[0, 0, 0] == 1.0 and s[0, 0, 1] == 1.0
+    assert q[0, 0, 0, :8].tolist() == [127, -127, 0, 2, 2, 0, -2, 63]
+    assert not q[0, 0, 1].any()
+    assert q[0, 0, 2, 0] == 127 and q[0, 0, 2, 1] == -127
+    sc = np.float32(2.54) / np.float32(127.0)
+    assert s[0, 0, 2] == sc
+    assert q[0, 0, 2, 2] == int(np.rint(np.float32(1.27) * (np.float32(1.0) / sc)))
+
+
+def test_quantiser_block_reduces_to_row_rule_and_max():
+    B, H, N, D = 1, 2, 200, 64
+    x = synth.normal(41, (B, H, N, D)) * 3
+    q1, s1 = oracle.quant_blocks(x, 1)
+    # per-row rule evaluated independently with numpy float32 scalars
+    mx = np.abs(x).max(-1)
+    sc = np.where(mx > 0, mx / np.float32(127.0), np.float32(1.0)).astype(np.float32)
+    inv = (np.float32(1.0) / sc).astype(np.float32)
+    want = np.clip(np.rint((x * inv[..., None]).astype(np.float32)), -127, 127).astype(np.int8)
+    assert np.array_equal(s1, sc) and np.array_equal(q1, want)
+    # block scale == max of the row scales' absmax / 127 (max is order independent), ragged tail block
+    for blk in (64, 128):
+        qb, sb = oracle.quant_blocks(x, blk)
+        nb = (N + blk - 1) // blk
+        assert sb.shape == (B, H, nb)
+        for b in range(nb):
+            m = mx[:, :, b * blk:(b + 1) * blk].max(-1)
+            assert np.array_equal(sb[:, :, b], (m / np.float32(127.0)).astype(np.float32))
+        assert np.abs(qb.astype(np.int32)).max() == 127
+    # the two rounding variants inside the reference (kernel: x*(1/s); its test: x/s) differ by at most one step
+    qd, _ = oracle.quant_blocks(x, 1, use_div=True)
+    assert np.abs(qd.astype(np.int32) - q1.astype(np.int32)).max() <= 1
+
+
+def test_int32_logits_known_answer():
+    # tests/sage_layout_probe.rs:73-84: A[16x32] = (i*7)%19 - 9, B[32x8] = (i*5)%13 - 6, C brute force
+    a = [((i * 7) % 19) - 9 for i in range(512)]
+    b = [((i * 5) % 13) - 6 for i in range(256)]
+    want = [[sum(a[i * 32 + t] * b[t * 8 + j] for t in range(32)) for j in range(8)] for i in range(16)]
+    A = np.array(a, np.int8).reshape(16, 32)
+    Bt = np.ascontiguousarray(np.array(b, np.int8).reshape(32, 8).T)  # keys as rows
+    got = oracle.logits_i32(A, Bt, 0, 16, 0, 8)
+    assert got.tolist() == want
+    # extreme values do not overflow: 128 * 127 * 127
+    q8 = np.full((4, 128), 127, np.int8)
+    k8 = np.full((4, 128), -127, np.int8)
+    assert (oracle.logits_i32(q8, k8, 0, 4, 0, 4) == -128 * 127 * 127).all()
+
+
+def test_k_mean_order_and_value():
+    """K smoothing is not in the reference (parity unpinned there): the mean is pinned by
+    its value (float64 mean within fp32 rounding) and by its defined summation order."""
+    B, H, N, D = 1, 2, 333, 64
+    k = synth.normal(51, (B, H, N, D)) + 3 * synth.normal(52, (1, H, 1, D))
+    got = oracle.k_mean(k)
+    assert np.abs(got - k.astype(np.float64).mean(2)).max() < 5e-6
+    # the defined order, spelled out with numpy float32 adds
+    want = np.zeros((B, H, D), np.float32)
+    for c0 in range(0, N, 64):
+        part = np.zeros((B, H, D), np.float32)
+        for j in range(c0, min(N, c0 + 64)):
+            part = part + k[:, :, j]
+        want = want + part
+    want = want / np.float32(N)
+    assert np.array_equal(got, want)
+
+
+def test_sage_reference_properties():
+    B, H, N, D = 1, 2, 256, 64
+    q = synth.normal(61, (B, H, N, D))
+    k = synth.normal(62, (B, H, N, D)) + 3 * synth.normal(64, (1, H, 1, D))
+    v = synth.normal(63, (B, H, N, D))
+    truth = oracle.sdpa_f64(q, k, v)
+    q8, sq = oracle.quant_blocks(q, 128)
+    # without smoothing the channel bias eats the int8 range
+    k8n, skn = oracle.quant_blocks(k, 64)
+    err_plain = np.abs(oracle.sage(q8, k8n, sq, skn, v, 128, 64) - truth).max()
+    # with smoothing: softmax(q.(k - mu)) == softmax(q.k) exactly, and the quantisation error drops
+    mu = oracle.k_mean(k)
+    k8s, sks = oracle.quant_blocks(k, 64, sub=mu)
+    err_smooth = np.abs(oracle.sage(q8, k8s, sq, sks, v, 128, 64) - truth).max()
+    assert err_smooth < 2e-2
+    assert err_smooth < err_plain
+    # block size 1 == the reference's per-row/per-key kernel; its own test bound is 2e-3
+    # against its emulation (tests/sage_int8.rs:148); against the truth int8 costs ~1e-2
+    q81, sq1 = oracle.quant_blocks(q, 1)
+    k81, sk1 = oracle.quant_blocks(k, 1, sub=mu)
+    err_row = np.abs(oracle.sage(q81, k81, sq1, sk1, v, 1, 1) - truth).max()
+    assert err_row < 2e-2
+    # dequantised logits reproduce q.k up to quantisation error
+    lg = oracle.logits_i32(q81[0, 0], k81[0, 0], 0, N, 0, N).astype(np.float64)
+    approx = lg * sq1[0, 0][:, None] * sk1[0, 0][None, :]
+    exact = q[0, 0].astype(np.float64) @ (k[0, 0] - mu[0, 0]).astype(np.float64).T
+    assert np.abs(approx - exact).max() < 0.5
+
+
+def test_cpu_baseline_matches_oracle():
+    B, H, N, D = 1, 3, 197, 64
+    q, k, v = synth.normal(71, (B, H, N, D)), synth.normal(72, (B, H, N, D)), synth.normal(73, (B, H, N, D))
+    for causal in (False, True):
+        out, threads = oracle.cpu_sdpa(q, k, v, causal=causal)
+        want = oracle.sdpa_f64(q, k, v, causal=causal)
+        assert threads >= 1
+        assert (np.abs(out - want) / np.maximum(np.abs(want), 1)).max() <= 1e-5
