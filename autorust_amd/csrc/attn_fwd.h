@@ -2,16 +2,20 @@
 // FlashAttention path and the int8 (SageAttention-style) path.
 //
 // Work decomposition
-//   grid  : one workgroup per (batch*head, tile of BQ = 32*NW queries)
-//   wave  : 32 queries; the wave computes S^T = K . Q^T, so that in the MFMA
-//           result layout every lane owns ONE query (column lane%32) and 16 of
-//           the 32 keys of a block.  Row max / row sum are then per-lane
-//           reductions plus one exchange with lane^32, and the probabilities
-//           are already in the operand layout the second product needs:
-//           O^T = V^T . P^T, again with one query per lane.
+//   grid  : one workgroup per (batch*head, tile of BQ = 32*QG*NW queries)
+//   wave  : 32*QG queries.  The wave computes S^T = K . Q^T, so that in the
+//           MFMA result layout every lane owns ONE query per group (column
+//           lane%32) and 16 of the 32 keys of a block.  Row max / row sum are
+//           per-lane reductions plus one exchange with lane^32, and the
+//           probabilities are already in the operand layout the second product
+//           needs: O^T = V^T . P^T, again with one query per lane.  With QG = 2
+//           every K / V^T fragment read from LDS feeds two MFMAs.
 //   tiles : BK = 64 keys per step, K and V^T staged through LDS by the whole
-//           workgroup (128-bit global loads issued one tile ahead into
-//           registers, written to the other LDS buffer after the math).
+//           workgroup: 128-bit global loads issued one tile ahead into
+//           registers, written to the other LDS buffer after the math.
+//   blocks: inside a tile the online softmax advances in blocks of 32 keys and
+//           Q.K^T of the next block is issued before the softmax of the current
+//           one, so that the matrix pipe works while the vector ALU exponentiates.
 //
 // MFMA shapes (wave64):
 //   v_mfma_f32_32x32x16_bf16  A[32 x 16] . B[16 x 32]   lane: row/col = lane%32,
@@ -23,12 +27,14 @@
 // Key order inside a 16-key step of P.V: the B operand wants, in lane half h,
 // keys "8h + t" (t = 0..7) of the step, while the S^T result gives half h the
 // keys 8*(t/4) + 4h + t%4.  A sum over keys does not care about their order,
-// so V^T is simply stored in LDS with the two middle groups of four keys of
-// every 16 swapped, and P is used exactly as the first MFMA produced it.
+// so V^T is stored in LDS with the two middle groups of four keys of every 16
+// swapped, and P is used exactly as the first MFMA produced it.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 namespace arhip {
 
@@ -68,14 +74,39 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     return __builtin_bit_cast(uint32_t, p);
 }
 
-// max over both lane halves (lane and lane^32 hold the same query)
+// lane and lane^32 hold the same query: combine their partial results
+__device__ __forceinline__ float xhalf_other(float x)
+{
+#if ARHIP_NO_PERMLANE_SWAP
+    return __shfl_xor(x, 32);
+#else
+    // v_permlane32_swap exchanges the upper half of the first operand with the
+    // lower half of the second: (x, x) -> ({lo,lo}, {hi,hi})
+    const uint32_t u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const int h = (threadIdx.x >> 5) & 1;
+    return __uint_as_float(h ? r[0] : r[1]);
+#endif
+}
 __device__ __forceinline__ float xhalf_max(float x)
 {
+#if ARHIP_NO_PERMLANE_SWAP
     return fmaxf(x, __shfl_xor(x, 32));
+#else
+    const uint32_t u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+#endif
 }
 __device__ __forceinline__ float xhalf_sum(float x)
 {
+#if ARHIP_NO_PERMLANE_SWAP
     return x + __shfl_xor(x, 32);
+#else
+    const uint32_t u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+#endif
 }
 
 // byte offset of V^T element (d, pos) in a [D][64] bf16 tile whose 16-byte
@@ -88,16 +119,21 @@ __device__ __forceinline__ int vt_off(int d, int pos)
     return d * 128 + ((chunk ^ sw) << 4) + ((pos & 7) << 1);
 }
 
-template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool OUT_F32, bool DBG>
+// s_waitcnt vmcnt(0): all outstanding global loads of this wave have landed.
+__device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+template <int D, int NW, int QG, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG>
 __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
 {
     constexpr int T = NW * 64;
-    constexpr int BQ = NW * 32;
-    constexpr int QK_BYTES = (MODE == MODE_I8) ? 1 : 2;       // bytes per q/k element
+    constexpr int WQ = 32 * QG;                                // queries per wave
+    constexpr int BQ = NW * WQ;
+    constexpr int QK_BYTES = (MODE == MODE_I8) ? 1 : 2;        // bytes per q/k element
     constexpr int KROW = D * QK_BYTES + 16;                    // padded K row in LDS
     constexpr int K_TILE = BK * KROW;
     constexpr int V_TILE = D * 128;
-    constexpr int STAGE = K_TILE + V_TILE;
+    constexpr int S_TILE = PER_KEY ? BK * 4 : 0;               // per-key scales of the tile
+    constexpr int STAGE = K_TILE + V_TILE + S_TILE;
     constexpr int K_CPR = D * QK_BYTES / 16;                   // 16-byte chunks per K row
     constexpr int K_CHUNKS = BK * K_CPR;
     constexpr int K_PER_THREAD = (K_CHUNKS + T - 1) / T;
@@ -107,6 +143,7 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
     constexpr int DB = D / 32;                                 // 32-channel output blocks
     static_assert(K_CHUNKS % T == 0 || K_CHUNKS < T, "K staging must divide evenly");
     static_assert(V_UNITS % T == 0 || V_UNITS < T, "V staging must divide evenly");
+    static_assert(!PER_KEY || MODE == MODE_I8, "per-key scales belong to the int8 path");
 
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE];
 
@@ -131,8 +168,7 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
     const int N = p.N;
 
     const int qblk = qt * BQ;
-    const int wq0 = qblk + wave * 32;  // first query of this wave
-    const int q_row = wq0 + i32;
+    const int wq0 = qblk + wave * WQ;  // first query of this wave
 
     int kvl = N;
     if (p.kv_len) {
@@ -146,32 +182,40 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
     const unsigned char *kbase = (const unsigned char *)p.k + (size_t)kv_bh * N * D * QK_BYTES;
     const uint16_t *vbase = p.v + (size_t)kv_bh * N * D;
 
-    // ---- Q operand, resident in registers for the whole kernel ----
-    uint4 qreg[KSTEPS];
-    {
-        const unsigned char *qb = (const unsigned char *)p.q + ((size_t)bh * N + (size_t)(q_row < N ? q_row : 0)) * D * QK_BYTES;
+    // ---- Q operand, resident in registers for the whole kernel.  Rows past N
+    // read row N-1: their results are never stored. ----
+    uint4 qreg[QG][KSTEPS];
+    int q_row[QG];
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) {
-            uint4 val = *(const uint4 *)(qb + s * 32 + h * 16);
-            if (q_row >= N) val = make_uint4(0, 0, 0, 0);
-            qreg[s] = val;
-        }
+    for (int g = 0; g < QG; ++g) {
+        q_row[g] = wq0 + g * 32 + i32;
+        const unsigned char *qb =
+            (const unsigned char *)p.q + ((size_t)bh * N + (size_t)min(q_row[g], N - 1)) * D * QK_BYTES;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) qreg[g][s] = *(const uint4 *)(qb + s * 32 + h * 16);
     }
 
     // ---- staging registers (tile i+1 in flight while tile i is computed) ----
     uint4 kst[K_PER_THREAD];
     uint4 vst[V_PER_THREAD][4];
+    float sst = 0.f;
+    const int nkb = (MODE == MODE_I8) ? (N + p.bk - 1) / p.bk : 0;
 
     auto load_tile = [&](int k0) {
+        const bool full = k0 + BK <= kend;  // uniform: the common case has no bounds logic
 #pragma unroll
         for (int j = 0; j < K_PER_THREAD; ++j) {
             const int c = tid + j * T;
             if (K_CHUNKS >= T || c < K_CHUNKS) {
                 const int row = c / K_CPR, col = c % K_CPR;
                 const int gr = k0 + row;
-                uint4 val = make_uint4(0, 0, 0, 0);
-                if (gr < kend) val = *(const uint4 *)(kbase + (size_t)gr * D * QK_BYTES + col * 16);
-                kst[j] = val;
+                if (full) {
+                    kst[j] = *(const uint4 *)(kbase + (size_t)gr * (D * QK_BYTES) + col * 16);
+                } else {
+                    uint4 val = *(const uint4 *)(kbase + (size_t)min(gr, kend - 1) * (D * QK_BYTES) + col * 16);
+                    if (gr >= kend) val = make_uint4(0, 0, 0, 0);
+                    kst[j] = val;
+                }
             }
         }
 #pragma unroll
@@ -182,12 +226,17 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) {
                     const int gr = k0 + m * 4 + kk;
-                    uint4 val = make_uint4(0, 0, 0, 0);
-                    if (gr < kend) val = *(const uint4 *)(vbase + (size_t)gr * D + dc * 8);
-                    vst[j][kk] = val;
+                    if (full) {
+                        vst[j][kk] = *(const uint4 *)(vbase + (size_t)gr * D + dc * 8);
+                    } else {
+                        uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * D + dc * 8);
+                        if (gr >= kend) val = make_uint4(0, 0, 0, 0);
+                        vst[j][kk] = val;
+                    }
                 }
             }
         }
+        if (PER_KEY && tid < BK) sst = p.sk[(size_t)kv_bh * nkb + min(k0 + tid, N - 1) / p.bk];
     };
 
     auto store_tile = [&](int stage) {
@@ -225,194 +274,206 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
                 }
             }
         }
+        if (PER_KEY && tid < BK) *(float *)(vl + V_TILE + tid * 4) = sst;
     };
 
-    // ---- accumulators ----
-    f32x16 oacc[DB];
+    // ---- accumulators and softmax state, one query per lane and group ----
+    f32x16 oacc[QG][DB];
+    float m_run[QG], l_run[QG], sq_lane[QG];
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+    for (int g = 0; g < QG; ++g) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
-    float m_run = NEG_SENTINEL;  // running max, in the exp2 domain (x * log2e)
-    float l_run = 0.f;           // this lane half's part of the running sum
-
-    float sq_lane = 1.f;
-    if (MODE == MODE_I8) {
-        const int nqb = (N + p.bq - 1) / p.bq;
-        sq_lane = p.sq[(size_t)bh * nqb + (q_row < N ? q_row : N - 1) / p.bq];
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[g][db][r] = 0.f;
+        m_run[g] = NEG_SENTINEL;  // running max in the exp2 domain (x * log2e)
+        l_run[g] = 0.f;           // this lane half's part of the running sum
+        sq_lane[g] = 1.f;
+        if (MODE == MODE_I8) {
+            const int nqb = (N + p.bq - 1) / p.bq;
+            sq_lane[g] = p.sq[(size_t)bh * nqb + min(q_row[g], N - 1) / p.bq];
+        }
     }
-    const int nkb = (MODE == MODE_I8) ? (N + p.bk - 1) / p.bk : 0;
     const float c_scale = p.scale * LOG2E;
 
     if (ntiles > 0) {
         load_tile(0);
         store_tile(0);
     }
+    wait_vmem();  // Q and the first tile have landed: nothing is pending at loop entry
     __syncthreads();
 
+    // S^T block: 32 keys x 32 queries for every query group, raw accumulators
+    typedef typename std::conditional<MODE == MODE_I8, i32x16, f32x16>::type acc_t;
+    auto qk_block = [&](const unsigned char *kl, int blk, acc_t (&s)[QG]) {
+        const unsigned char *krow = kl + (blk * 32 + i32) * KROW + h * 16;
+#pragma unroll
+        for (int g = 0; g < QG; ++g)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[g][r] = 0;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            const uint4 a = *(const uint4 *)(krow + st * 32);
+#pragma unroll
+            for (int g = 0; g < QG; ++g) {
+                if constexpr (MODE == MODE_I8)
+                    s[g] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a),
+                                                                 __builtin_bit_cast(i32x4, qreg[g][st]), s[g], 0, 0, 0);
+                else
+                    s[g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                                   __builtin_bit_cast(bf16x8, qreg[g][st]), s[g], 0, 0, 0);
+            }
+        }
+    };
+
+    int sk_idx = 0, sk_fill = 0;
     for (int it = 0; it < ntiles; ++it) {
         const int k0 = it * BK;
         const int stage = it & 1;
         if (it + 1 < ntiles) load_tile(k0 + BK);
 
         // a wave whose queries all precede this tile has nothing to do in it
-        const bool active = !CAUSAL || (k0 <= wq0 + 31);
+        const bool active = !CAUSAL || (k0 <= wq0 + WQ - 1);
         if (active) {
             const unsigned char *kl = lds + stage * STAGE;
             const unsigned char *vl = kl + K_TILE;
 
-            // ---- S^T = K . Q^T : two blocks of 32 keys x 32 queries ----
-            float x[2][16];
+            // tile-uniform K scale (block sizes that are multiples of the tile)
+            float f_tile = c_scale;
+            if (MODE == MODE_I8 && !PER_KEY) f_tile = p.sk[(size_t)kv_bh * nkb + sk_idx];
+
+            acc_t sacc[2][QG];
+            qk_block(kl, 0, sacc[0]);
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const unsigned char *krow = kl + (kb * 32 + i32) * KROW + h * 16;
-                if (MODE == MODE_I8) {
-                    i32x16 acc;
+            for (int blk = 0; blk < 2; ++blk) {
+                if (blk == 0) qk_block(kl, 1, sacc[1]);
+                const int kb0 = k0 + blk * 32;  // first key of the block
+
+                uint4 pb[QG][2];
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[r] = 0;
-#pragma unroll
-                    for (int s = 0; s < KSTEPS; ++s) {
-                        const uint4 a = *(const uint4 *)(krow + s * 32);
-                        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                            __builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, qreg[s]), acc, 0, 0, 0);
-                    }
+                for (int g = 0; g < QG; ++g) {
+                    acc_t &s = sacc[blk][g];
                     if (DBG) {
-                        if (bh == p.dbg_bh && (wq0 >> 5) == p.dbg_qt && it == p.dbg_kt) {
+                        if (bh == p.dbg_bh && ((wq0 >> 5) + g) == p.dbg_qt && it == p.dbg_kt) {
 #pragma unroll
-                            for (int r = 0; r < 16; ++r) {
-                                const int key = kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                                p.dbg[i32 * 64 + key] = acc[r];
-                            }
+                            for (int r = 0; r < 16; ++r)
+                                p.dbg[i32 * 64 + blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] = (int32_t)s[r];
                         }
                     }
-                    // s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322
-                    if ((p.bk & 31) == 0) {
-                        const float skv = p.sk[(size_t)kv_bh * nkb + min(k0 + kb * 32, N - 1) / p.bk];
-                        const float f = ((sq_lane * skv) * p.scale) * LOG2E;
+                    float x[16];
+                    float m_new;
+                    const bool edge = (kb0 + 32 > kend) || (CAUSAL && (kb0 + 31 > wq0 + g * 32));
+                    if (!HAS_MASK && !PER_KEY && !edge) {
+                        // fast path: max over the raw accumulators, scale folded into the exponent
+                        // s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322
+                        const float c = (MODE == MODE_I8) ? ((sq_lane[g] * f_tile) * p.scale) * LOG2E : c_scale;
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) x[kb][r] = (float)acc[r] * f;
+                        for (int r = 0; r < 16; ++r) x[r] = (float)s[r];
+                        float mx = fmaxf(x[0], x[1]);
+#pragma unroll
+                        for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(x[r], x[r + 1]));
+                        mx = xhalf_max(mx);
+                        m_new = fmaxf(m_run[g], mx * c);
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -m_new));
                     } else {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
-                            const int key = k0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                            const float skv = p.sk[(size_t)kv_bh * nkb + min(key, N - 1) / p.bk];
-                            x[kb][r] = (float)acc[r] * (((sq_lane * skv) * p.scale) * LOG2E);
+                            const int key = kb0 + 8 * (r >> 2) + 4 * h + (r & 3);
+                            float c = c_scale;
+                            if (MODE == MODE_I8) {
+                                const float skv = PER_KEY ? *(const float *)(vl + V_TILE + (key - k0) * 4) : f_tile;
+                                c = ((sq_lane[g] * skv) * p.scale) * LOG2E;
+                            }
+                            float xv = (float)s[r] * c;
+                            if (HAS_MASK) {
+                                if (key < N && q_row[g] < N) xv += p.mask[(size_t)q_row[g] * N + key] * LOG2E;
+                            }
+                            if (key >= kend || (CAUSAL && key > q_row[g])) xv = NEG_SENTINEL;
+                            x[r] = xv;
                         }
+                        float mx = fmaxf(x[0], x[1]);
+#pragma unroll
+                        for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(x[r], x[r + 1]));
+                        mx = xhalf_max(mx);
+                        m_new = fmaxf(m_run[g], mx);
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
                     }
-                } else {
-                    f32x16 acc;
+                    const float alpha = __builtin_amdgcn_exp2f(m_run[g] - m_new);
+                    m_run[g] = m_new;
+                    float rs = (x[0] + x[1]) + (x[2] + x[3]);
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+                    for (int r = 4; r < 16; r += 4) rs += (x[r] + x[r + 1]) + (x[r + 2] + x[r + 3]);
+                    l_run[g] = l_run[g] * alpha + rs;
+                    // rescale the accumulators only when some lane's maximum moved
+                    if (__any(alpha != 1.0f)) {
 #pragma unroll
-                    for (int s = 0; s < KSTEPS; ++s) {
-                        const uint4 a = *(const uint4 *)(krow + s * 32);
-                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, qreg[s]), acc, 0, 0, 0);
+                        for (int db = 0; db < DB; ++db)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) oacc[g][db][r] *= alpha;
                     }
+                    // P (bf16) as the B operand: 2 steps of 16 keys
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) x[kb][r] = acc[r] * c_scale;
+                    for (int ks = 0; ks < 2; ++ks) {
+                        pb[g][ks].x = pack_bf16x2(x[ks * 8 + 0], x[ks * 8 + 1]);
+                        pb[g][ks].y = pack_bf16x2(x[ks * 8 + 2], x[ks * 8 + 3]);
+                        pb[g][ks].z = pack_bf16x2(x[ks * 8 + 4], x[ks * 8 + 5]);
+                        pb[g][ks].w = pack_bf16x2(x[ks * 8 + 6], x[ks * 8 + 7]);
+                    }
                 }
-            }
 
-            // ---- additive mask, causal and key-length masking ----
-            if (HAS_MASK) {
+                // ---- O^T += V^T . P^T for the 32 keys of the block ----
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int db = 0; db < DB; ++db) {
+                    const int d = db * 32 + i32;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int key = k0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                        if (key < N && q_row < N) x[kb][r] += p.mask[(size_t)q_row * N + key] * LOG2E;
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const uint4 a = *(const uint4 *)(vl + vt_off(d, blk * 32 + ks * 16 + h * 8));
+#pragma unroll
+                        for (int g = 0; g < QG; ++g)
+                            oacc[g][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, pb[g][ks]), oacc[g][db], 0, 0, 0);
                     }
-            }
-            const bool edge = (k0 + BK > kend) || (CAUSAL && (k0 + BK - 1 > wq0));
-            if (edge) {
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int key = k0 + kb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                        if (key >= kend || (CAUSAL && key > q_row)) x[kb][r] = NEG_SENTINEL;
-                    }
-            }
-
-            // ---- online softmax, one query per lane ----
-            float mx = x[0][0];
-#pragma unroll
-            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, x[0][r]);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, x[1][r]);
-            mx = xhalf_max(mx);
-            const float m_new = fmaxf(m_run, mx);
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            m_run = m_new;
-            float rs = 0.f;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float pv = __builtin_amdgcn_exp2f(x[kb][r] - m_new);
-                    x[kb][r] = pv;
-                    rs += pv;
-                }
-            l_run = l_run * alpha + rs;
-
-            // rescale the accumulators only when some lane's maximum moved
-            if (__any(alpha != 1.0f)) {
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-            }
-
-            // ---- P (bf16) as the B operand: 4 steps of 16 keys ----
-            uint4 pb[4];
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const int kb = ks >> 1, r0 = (ks & 1) * 8;
-                pb[ks].x = pack_bf16x2(x[kb][r0 + 0], x[kb][r0 + 1]);
-                pb[ks].y = pack_bf16x2(x[kb][r0 + 2], x[kb][r0 + 3]);
-                pb[ks].z = pack_bf16x2(x[kb][r0 + 4], x[kb][r0 + 5]);
-                pb[ks].w = pack_bf16x2(x[kb][r0 + 6], x[kb][r0 + 7]);
-            }
-
-            // ---- O^T += V^T . P^T ----
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const int d = db * 32 + i32;
-#pragma unroll
-                for (int ks = 0; ks < 4; ++ks) {
-                    const uint4 a = *(const uint4 *)(vl + vt_off(d, ks * 16 + h * 8));
-                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, pb[ks]), oacc[db], 0, 0, 0);
                 }
             }
         }
 
         if (it + 1 < ntiles) store_tile(stage ^ 1);
         __syncthreads();
+        if (MODE == MODE_I8 && !PER_KEY) {  // advance the K-block index without dividing
+            sk_fill += BK;
+            if (sk_fill >= p.bk) {
+                sk_fill = 0;
+                ++sk_idx;
+            }
+        }
     }
 
     // ---- normalise and store: acc * (l > 0 ? 1/l : 0), cuda_flash_bf16.rs:414-426 ----
-    const float l_tot = xhalf_sum(l_run);
-    const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
-    if (q_row < N) {
-        const size_t obase = ((size_t)bh * N + q_row) * D;
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+    for (int g = 0; g < QG; ++g) {
+        const float l_tot = xhalf_sum(l_run[g]);
+        const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+        if (q_row[g] < N) {
+            const size_t obase = ((size_t)bh * N + q_row[g]) * D;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int d = db * 32 + 8 * g + 4 * h;
-                const float o0 = oacc[db][4 * g + 0] * inv, o1 = oacc[db][4 * g + 1] * inv;
-                const float o2 = oacc[db][4 * g + 2] * inv, o3 = oacc[db][4 * g + 3] * inv;
-                if (OUT_F32) {
-                    *(float4 *)((float *)p.o + obase + d) = make_float4(o0, o1, o2, o3);
-                } else {
-                    uint2 w;
-                    w.x = pack_bf16x2(o0, o1);
-                    w.y = pack_bf16x2(o2, o3);
-                    *(uint2 *)((uint16_t *)p.o + obase + d) = w;
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int gg = 0; gg < 4; ++gg) {
+                    const int d = db * 32 + 8 * gg + 4 * h;
+                    const float o0 = oacc[g][db][4 * gg + 0] * inv, o1 = oacc[g][db][4 * gg + 1] * inv;
+                    const float o2 = oacc[g][db][4 * gg + 2] * inv, o3 = oacc[g][db][4 * gg + 3] * inv;
+                    if (OUT_F32) {
+                        *(float4 *)((float *)p.o + obase + d) = make_float4(o0, o1, o2, o3);
+                    } else {
+                        uint2 w;
+                        w.x = pack_bf16x2(o0, o1);
+                        w.y = pack_bf16x2(o2, o3);
+                        *(uint2 *)((uint16_t *)p.o + obase + d) = w;
+                    }
                 }
-            }
+        }
     }
 }
 

@@ -8,6 +8,8 @@
 #include "attn_fwd.h"
 #include "flash_f32.h"
 
+#include <cstdlib>
+
 using namespace arhip;
 
 extern "C" int arhip_attn_supported(int kind, int64_t n, int64_t d, int dtype)
@@ -38,32 +40,48 @@ static int check_common(const char *fn, arhip_device *dev, const void *q, const 
     return ARHIP_OK;
 }
 
-template <int D, int NW, int MODE, bool OUT_F32, bool DBG>
+// CAUSAL / HAS_MASK dispatch for one tiling variant.
+template <int D, int NW, int QG, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool MASKS>
 static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bool has_mask)
 {
     const dim3 grid((unsigned)p.total), block(NW * 64);
-    if (DBG) {  // debug export: never combined with an additive mask
-        if (causal) hipLaunchKernelGGL((attn_fwd_kernel<D, NW, true, false, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, false, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
-    } else if (causal) {
-        if (has_mask)
-            hipLaunchKernelGGL((attn_fwd_kernel<D, NW, true, true, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
-        else
-            hipLaunchKernelGGL((attn_fwd_kernel<D, NW, true, false, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
-    } else {
-        if (has_mask)
-            hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, true, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
-        else
-            hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, false, MODE, OUT_F32, DBG>), grid, block, 0, stream, p);
+    if constexpr (MASKS) {
+        if (has_mask) {
+            if (causal)
+                hipLaunchKernelGGL((attn_fwd_kernel<D, NW, QG, true, true, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
+            else
+                hipLaunchKernelGGL((attn_fwd_kernel<D, NW, QG, false, true, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
+            return;
+        }
     }
+    if (causal)
+        hipLaunchKernelGGL((attn_fwd_kernel<D, NW, QG, true, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((attn_fwd_kernel<D, NW, QG, false, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
 }
 
-// Waves per workgroup: 4 (128 queries) when that still fills the chip, else 1
-// (32 queries) so that short sequences spread over more compute units.
-static int pick_nw(arhip_device *dev, int64_t heads, int64_t N)
+// Tiling variants: waves per workgroup x query groups (of 32) per wave.
+//   V_1x1  32 queries per workgroup: short sequences, spreads over the chip
+//   V_4x1  128 queries, every K/V fragment read from LDS feeds one MFMA
+//   V_8x1  256 queries, two waves per SIMD
+//   V_4x2  256 queries, every fragment feeds two MFMAs (half the LDS traffic)
+enum { V_1x1 = 0, V_4x1 = 1, V_8x1 = 2, V_4x2 = 3 };
+
+static int variant_queries(int v) { return v == V_1x1 ? 32 : (v == V_4x1 ? 128 : 256); }
+
+static int pick_variant(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bool special)
 {
-    const int64_t wg4 = heads * ((N + 127) / 128);
-    return (wg4 >= 2 * (int64_t)dev->cus) ? 4 : 1;
+    // masks, per-key scales and the debug export are only built for V_4x1 (and V_1x1 at D = 64)
+    int v;
+    const int64_t wg128 = heads * ((N + 127) / 128);
+    if (D == 64 && wg128 < 2 * (int64_t)dev->cus) v = V_1x1;
+    else if (special) v = V_4x1;
+    else v = (heads * ((N + 255) / 256) >= 2 * (int64_t)dev->cus) ? V_8x1 : V_4x1;
+    if (const char *e = getenv("ARHIP_ATTN_VARIANT")) {  // tuning aid; results do not depend on it
+        const int w = atoi(e);
+        if (w >= V_1x1 && w <= V_4x2 && !special && (w != V_1x1 || D == 64)) v = w;
+    }
+    return v;
 }
 
 extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, const void *v, void *o,
@@ -103,15 +121,25 @@ extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, 
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
     p.bq = p.bk = 1;
     p.scale = scale;
-    const int nw = (D == 64) ? pick_nw(dev, B * Hq, N) : 4;
-    p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
+    const bool c = causal != 0, hm = mask != nullptr;
+    const int var = pick_variant(dev, B * Hq, N, D, hm);
+    const int bqv = variant_queries(var);
+    p.nq = (int)((N + bqv - 1) / bqv);
     p.total = (int)(p.nq * B * Hq);
     if (int rc = t.begin()) return rc;
     if (D == 64) {
-        if (nw == 4) launch_attn<64, 4, MODE_BF16, false, false>(dev->stream, p, causal != 0, mask != nullptr);
-        else launch_attn<64, 1, MODE_BF16, false, false>(dev->stream, p, causal != 0, mask != nullptr);
+        switch (var) {
+        case V_1x1: launch_attn<64, 1, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm); break;
+        case V_4x1: launch_attn<64, 4, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm); break;
+        case V_8x1: launch_attn<64, 8, 1, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm); break;
+        default: launch_attn<64, 4, 2, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm); break;
+        }
     } else {
-        launch_attn<128, 4, MODE_BF16, false, false>(dev->stream, p, causal != 0, mask != nullptr);
+        switch (var) {
+        case V_4x1: launch_attn<128, 4, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm); break;
+        case V_8x1: launch_attn<128, 8, 1, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm); break;
+        default: launch_attn<128, 4, 2, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm); break;
+        }
     }
     arhip_note_selected(ARHIP_K_FLASH_BF16);
     return t.end();
@@ -140,10 +168,16 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
     p.bq = (int)bq; p.bk = (int)bk;
     p.scale = scale;
-    const int nw = 4;
-    p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
-    p.total = (int)(p.nq * B * Hq);
     const bool dbg = dbg_logits != nullptr;
+    const bool c = causal != 0, hm = mask != nullptr, f32o = out_dtype == ARHIP_F32;
+    // K scales that are uniform over a 64-key tile take the fast kernel; anything else
+    // (including the reference's per-key scales, bk == 1) stages the tile's scales in LDS
+    const bool per_key = (bk % 64) != 0;
+    int var = pick_variant(dev, B * Hq, N, D, hm || per_key || dbg);
+    if (var == V_1x1) var = V_4x1;
+    const int bqv = variant_queries(var);
+    p.nq = (int)((N + bqv - 1) / bqv);
+    p.total = (int)(p.nq * B * Hq);
     if (dbg) {
         p.dbg = dbg_logits;
         p.dbg_bh = dbg_sel[0]; p.dbg_qt = dbg_sel[1]; p.dbg_kt = dbg_sel[2];
@@ -151,23 +185,28 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
                           p.dbg_kt >= 0 && (int64_t)p.dbg_kt * 64 < N,
                       "arhip_sage_fwd: debug tile selector out of range");
     }
-    const bool c = causal != 0, hm = mask != nullptr, f32o = out_dtype == ARHIP_F32;
     arhip_call_timer t{dev, wait, secs};
     t.kernel = ARHIP_K_SAGE;
     if (int rc = t.begin()) return rc;
-#define SAGE_LAUNCH(DD)                                                                              \
-    do {                                                                                             \
-        if (dbg) {                                                                                   \
-            if (f32o) launch_attn<DD, 4, MODE_I8, true, true>(dev->stream, p, c, hm);                \
-            else launch_attn<DD, 4, MODE_I8, false, true>(dev->stream, p, c, hm);                    \
-        } else {                                                                                     \
-            if (f32o) launch_attn<DD, 4, MODE_I8, true, false>(dev->stream, p, c, hm);               \
-            else launch_attn<DD, 4, MODE_I8, false, false>(dev->stream, p, c, hm);                   \
-        }                                                                                            \
+#define SAGE_V(DD, NWW, QGG, PK, DB_, MK)                                                              \
+    do {                                                                                               \
+        if (f32o) launch_attn<DD, NWW, QGG, MODE_I8, PK, true, DB_, MK>(dev->stream, p, c, hm);        \
+        else launch_attn<DD, NWW, QGG, MODE_I8, PK, false, DB_, MK>(dev->stream, p, c, hm);            \
     } while (0)
-    if (D == 64) SAGE_LAUNCH(64);
-    else SAGE_LAUNCH(128);
-#undef SAGE_LAUNCH
+#define SAGE_D(DD)                                                                                     \
+    do {                                                                                               \
+        if (dbg) {                                                                                     \
+            if (per_key) SAGE_V(DD, 4, 1, true, true, false);                                          \
+            else SAGE_V(DD, 4, 1, false, true, false);                                                 \
+        } else if (per_key) SAGE_V(DD, 4, 1, true, false, true);                                       \
+        else if (var == V_4x1) SAGE_V(DD, 4, 1, false, false, true);                                   \
+        else if (var == V_8x1) SAGE_V(DD, 8, 1, false, false, false);                                  \
+        else SAGE_V(DD, 4, 2, false, false, false);                                                    \
+    } while (0)
+    if (D == 64) SAGE_D(64);
+    else SAGE_D(128);
+#undef SAGE_D
+#undef SAGE_V
     arhip_note_selected(ARHIP_K_SAGE);
     return t.end();
 }
