@@ -22,7 +22,9 @@ HEADERS = ["arhip_internal.h", "attn_fwd.h", "flash_f32.h", os.path.join("..", "
 # -packed-fp32-ops off: packed fp32 VALU instructions are not used by this build.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wall", "-Wno-unused-function"]
+         "-Wall", "-Wno-unused-function",
+         # loop strength reduction multiplies the address registers of the tile loop and spills them
+         "-mllvm", "-disable-lsr"]
 
 
 def _newer(target, deps):

@@ -2,20 +2,24 @@
 // FlashAttention path and the int8 (SageAttention-style) path.
 //
 // Work decomposition
-//   grid  : one workgroup per (batch*head, tile of BQ = 32*QG*NW queries)
-//   wave  : 32*QG queries.  The wave computes S^T = K . Q^T, so that in the
-//           MFMA result layout every lane owns ONE query per group (column
-//           lane%32) and 16 of the 32 keys of a block.  Row max / row sum are
-//           per-lane reductions plus one exchange with lane^32, and the
-//           probabilities are already in the operand layout the second product
-//           needs: O^T = V^T . P^T, again with one query per lane.  With QG = 2
-//           every K / V^T fragment read from LDS feeds two MFMAs.
+//   grid  : one workgroup per (batch*head, tile of BQ = 32*NW queries)
+//   wave  : 32 queries.  The wave computes S^T = K . Q^T, so that in the MFMA
+//           result layout every lane owns ONE query (column lane%32) and 16 of
+//           the 32 keys of a block.  Row max / row sum are per-lane reductions
+//           plus one exchange with lane^32, and the probabilities are already in
+//           the operand layout the second product needs: O^T = V^T . P^T, again
+//           with one query per lane (the softmax rescale is a per-lane scalar).
 //   tiles : BK = 64 keys per step, K and V^T staged through LDS by the whole
 //           workgroup: 128-bit global loads issued one tile ahead into
-//           registers, written to the other LDS buffer after the math.
-//   blocks: inside a tile the online softmax advances in blocks of 32 keys and
-//           Q.K^T of the next block is issued before the softmax of the current
-//           one, so that the matrix pipe works while the vector ALU exponentiates.
+//           registers, written to the next LDS stage after the math; one
+//           barrier per tile.
+//   skew  : with 8 waves (two per SIMD) the upper four run one phase behind the
+//           lower four: while waves 0-3 multiply Q.K^T of tile i on the matrix
+//           cores, waves 4-7 exponentiate tile i-1 on the vector ALU, and vice
+//           versa.  Both halves of a SIMD's issue slots stay busy instead of
+//           all waves queueing for the same pipe after every barrier.  The
+//           lagging waves still read V of tile i-1 while tile i+1 is written, so
+//           this mode cycles through three LDS stages instead of two.
 //
 // MFMA shapes (wave64):
 //   v_mfma_f32_32x32x16_bf16  A[32 x 16] . B[16 x 32]   lane: row/col = lane%32,
@@ -24,11 +28,13 @@
 //   result C[32 x 32]: lane holds column lane%32 and rows
 //                             8*(r/4) + 4*(lane/32) + r%4,  r = 0..15
 //
-// Key order inside a 16-key step of P.V: the B operand wants, in lane half h,
-// keys "8h + t" (t = 0..7) of the step, while the S^T result gives half h the
-// keys 8*(t/4) + 4h + t%4.  A sum over keys does not care about their order,
-// so V^T is stored in LDS with the two middle groups of four keys of every 16
-// swapped, and P is used exactly as the first MFMA produced it.
+// V^T operand without a transpose pass: V sits in LDS row-major like K, and
+// ds_read_b64_tr_b16 hands every lane four keys of ONE channel (within 16 lanes,
+// result element e of lane i is element i%4 of the 8 bytes lane 4e + i/4 pointed
+// at).  The S^T result gives lane half h the keys 8*(t/4) + 4h + t%4 of a 16-key
+// step as B-operand elements t = 0..7, so the two transposing reads of a step
+// simply fetch keys 4h..4h+3 and 8+4h..8+4h+3: P is used exactly as the first
+// MFMA produced it and nothing is shuffled.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -42,6 +48,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(16))) int i32x16;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
 
 constexpr int MODE_BF16 = 0;  // q, k bf16
 constexpr int MODE_I8 = 1;    // q, k int8 with block scales
@@ -62,8 +69,9 @@ struct AttnParams {
     int dbg_bh, dbg_qt, dbg_kt;
     int Hq, Hkv, N;
     int bq, bk;
-    int nq;     // query tiles per head
-    int total;  // workgroups
+    int bk_tile_shift;  // log2(bk / 64) when the K scales are tile-uniform
+    int nq;        // query tiles per head
+    int total;     // workgroups
     float scale;
 };
 
@@ -74,78 +82,67 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     return __builtin_bit_cast(uint32_t, p);
 }
 
-// lane and lane^32 hold the same query: combine their partial results
-__device__ __forceinline__ float xhalf_other(float x)
-{
-#if ARHIP_NO_PERMLANE_SWAP
-    return __shfl_xor(x, 32);
-#else
-    // v_permlane32_swap exchanges the upper half of the first operand with the
-    // lower half of the second: (x, x) -> ({lo,lo}, {hi,hi})
-    const uint32_t u = __float_as_uint(x);
-    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    const int h = (threadIdx.x >> 5) & 1;
-    return __uint_as_float(h ? r[0] : r[1]);
-#endif
-}
+// lane and lane^32 hold the same query: combine their partial results.
+// v_permlane32_swap exchanges the upper half of its first operand with the lower
+// half of its second: (x, x) -> ({lo,lo}, {hi,hi}).
 __device__ __forceinline__ float xhalf_max(float x)
 {
-#if ARHIP_NO_PERMLANE_SWAP
-    return fmaxf(x, __shfl_xor(x, 32));
-#else
     const uint32_t u = __float_as_uint(x);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-#endif
 }
 __device__ __forceinline__ float xhalf_sum(float x)
 {
-#if ARHIP_NO_PERMLANE_SWAP
-    return x + __shfl_xor(x, 32);
-#else
     const uint32_t u = __float_as_uint(x);
     const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-#endif
 }
 
-// byte offset of V^T element (d, pos) in a [D][64] bf16 tile whose 16-byte
-// chunks are XOR-swizzled per row so that both the transposing 8-byte writes
-// and the 16-byte operand reads spread over the LDS banks.
-__device__ __forceinline__ int vt_off(int d, int pos)
+// Four keys of one channel: the transposing LDS read described above.
+__device__ __forceinline__ uint2 lds_read_tr16(const unsigned char *p)
 {
-    const int chunk = pos >> 3;
-    const int sw = (d ^ (d >> 3)) & 7;
-    return d * 128 + ((chunk ^ sw) << 4) + ((pos & 7) << 1);
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
+    return __builtin_bit_cast(uint2, v);
 }
+
+#ifndef ARHIP_FENCES
+#define ARHIP_FENCES 1
+#endif
+#if ARHIP_FENCES
+#define ARHIP_FENCE() __builtin_amdgcn_sched_barrier(0)
+#else
+#define ARHIP_FENCE() ((void)0)
+#endif
 
 // s_waitcnt vmcnt(0): all outstanding global loads of this wave have landed.
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-template <int D, int NW, int QG, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG>
-__global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
+template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG>
+__global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(const AttnParams p)
 {
+    constexpr int NSTAGE = 2;
     constexpr int T = NW * 64;
-    constexpr int WQ = 32 * QG;                                // queries per wave
-    constexpr int BQ = NW * WQ;
+    constexpr int BQ = NW * 32;
     constexpr int QK_BYTES = (MODE == MODE_I8) ? 1 : 2;        // bytes per q/k element
     constexpr int KROW = D * QK_BYTES + 16;                    // padded K row in LDS
     constexpr int K_TILE = BK * KROW;
-    constexpr int V_TILE = D * 128;
+    constexpr int VROW = D * 2 + 64;                           // V row in LDS: 4 rows fill the 64 banks
+    constexpr int V_TILE = BK * VROW;
     constexpr int S_TILE = PER_KEY ? BK * 4 : 0;               // per-key scales of the tile
     constexpr int STAGE = K_TILE + V_TILE + S_TILE;
     constexpr int K_CPR = D * QK_BYTES / 16;                   // 16-byte chunks per K row
     constexpr int K_CHUNKS = BK * K_CPR;
     constexpr int K_PER_THREAD = (K_CHUNKS + T - 1) / T;
-    constexpr int V_UNITS = (BK / 4) * (D / 8);                // 4 keys x 8 channels each
-    constexpr int V_PER_THREAD = (V_UNITS + T - 1) / T;
+    constexpr int V_CPR = D * 2 / 16;                          // 16-byte chunks per V row
+    constexpr int V_CHUNKS = BK * V_CPR;
+    constexpr int V_PER_THREAD = (V_CHUNKS + T - 1) / T;
     constexpr int KSTEPS = (MODE == MODE_I8) ? D / 32 : D / 16;  // MFMA k steps over D
     constexpr int DB = D / 32;                                 // 32-channel output blocks
     static_assert(K_CHUNKS % T == 0 || K_CHUNKS < T, "K staging must divide evenly");
-    static_assert(V_UNITS % T == 0 || V_UNITS < T, "V staging must divide evenly");
+    static_assert(V_CHUNKS % T == 0 || V_CHUNKS < T, "V staging must divide evenly");
     static_assert(!PER_KEY || MODE == MODE_I8, "per-key scales belong to the int8 path");
 
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char lds[NSTAGE * STAGE];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -168,7 +165,8 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
     const int N = p.N;
 
     const int qblk = qt * BQ;
-    const int wq0 = qblk + wave * WQ;  // first query of this wave
+    const int wq0 = qblk + wave * 32;  // first query of this wave
+    const int q_row = wq0 + i32;
 
     int kvl = N;
     if (p.kv_len) {
@@ -178,30 +176,28 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
     int kend = kvl;
     if (CAUSAL) kend = min(kend, min(N, qblk + BQ));
     const int ntiles = (kend + BK - 1) / BK;
+    // tiles this wave takes part in: under the causal mask, none past its last query
+    const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / BK + 1) : ntiles;
 
     const unsigned char *kbase = (const unsigned char *)p.k + (size_t)kv_bh * N * D * QK_BYTES;
     const uint16_t *vbase = p.v + (size_t)kv_bh * N * D;
 
     // ---- Q operand, resident in registers for the whole kernel.  Rows past N
     // read row N-1: their results are never stored. ----
-    uint4 qreg[QG][KSTEPS];
-    int q_row[QG];
+    uint4 qreg[KSTEPS];
+    {
+        const unsigned char *qb = (const unsigned char *)p.q + ((size_t)bh * N + (size_t)min(q_row, N - 1)) * D * QK_BYTES;
 #pragma unroll
-    for (int g = 0; g < QG; ++g) {
-        q_row[g] = wq0 + g * 32 + i32;
-        const unsigned char *qb =
-            (const unsigned char *)p.q + ((size_t)bh * N + (size_t)min(q_row[g], N - 1)) * D * QK_BYTES;
-#pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) qreg[g][s] = *(const uint4 *)(qb + s * 32 + h * 16);
+        for (int s = 0; s < KSTEPS; ++s) qreg[s] = *(const uint4 *)(qb + s * 32 + h * 16);
     }
 
     // ---- staging registers (tile i+1 in flight while tile i is computed) ----
     uint4 kst[K_PER_THREAD];
-    uint4 vst[V_PER_THREAD][4];
+    uint4 vst[V_PER_THREAD];
     float sst = 0.f;
     const int nkb = (MODE == MODE_I8) ? (N + p.bk - 1) / p.bk : 0;
 
-    auto load_tile = [&](int k0) {
+    auto load_tile = [&](int k0) __attribute__((always_inline)) {
         const bool full = k0 + BK <= kend;  // uniform: the common case has no bounds logic
 #pragma unroll
         for (int j = 0; j < K_PER_THREAD; ++j) {
@@ -220,26 +216,23 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
         }
 #pragma unroll
         for (int j = 0; j < V_PER_THREAD; ++j) {
-            const int u = tid + j * T;
-            if (V_UNITS >= T || u < V_UNITS) {
-                const int m = u / (D / 8), dc = u % (D / 8);
-#pragma unroll
-                for (int kk = 0; kk < 4; ++kk) {
-                    const int gr = k0 + m * 4 + kk;
-                    if (full) {
-                        vst[j][kk] = *(const uint4 *)(vbase + (size_t)gr * D + dc * 8);
-                    } else {
-                        uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * D + dc * 8);
-                        if (gr >= kend) val = make_uint4(0, 0, 0, 0);
-                        vst[j][kk] = val;
-                    }
+            const int c = tid + j * T;
+            if (V_CHUNKS >= T || c < V_CHUNKS) {
+                const int row = c / V_CPR, col = c % V_CPR;
+                const int gr = k0 + row;
+                if (full) {
+                    vst[j] = *(const uint4 *)(vbase + (size_t)gr * D + col * 8);
+                } else {
+                    uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * D + col * 8);
+                    if (gr >= kend) val = make_uint4(0, 0, 0, 0);
+                    vst[j] = val;
                 }
             }
         }
         if (PER_KEY && tid < BK) sst = p.sk[(size_t)kv_bh * nkb + min(k0 + tid, N - 1) / p.bk];
     };
 
-    auto store_tile = [&](int stage) {
+    auto store_tile = [&](int stage) __attribute__((always_inline)) {
         unsigned char *kl = lds + stage * STAGE;
         unsigned char *vl = kl + K_TILE;
 #pragma unroll
@@ -252,49 +245,176 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
         }
 #pragma unroll
         for (int j = 0; j < V_PER_THREAD; ++j) {
-            const int u = tid + j * T;
-            if (V_UNITS >= T || u < V_UNITS) {
-                const int m = u / (D / 8), dc = u % (D / 8);
-                // keys 4m..4m+3 -> position group: swap the middle two groups of every 16 keys
-                const int g4 = m & 3;
-                const int pos = ((m & ~3) + ((g4 & 1) << 1) + (g4 >> 1)) << 2;
-                const uint32_t r0[4] = {vst[j][0].x, vst[j][0].y, vst[j][0].z, vst[j][0].w};
-                const uint32_t r1[4] = {vst[j][1].x, vst[j][1].y, vst[j][1].z, vst[j][1].w};
-                const uint32_t r2[4] = {vst[j][2].x, vst[j][2].y, vst[j][2].z, vst[j][2].w};
-                const uint32_t r3[4] = {vst[j][3].x, vst[j][3].y, vst[j][3].z, vst[j][3].w};
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    uint2 lo, hi;
-                    lo.x = (r0[c] & 0xffffu) | (r1[c] << 16);
-                    lo.y = (r2[c] & 0xffffu) | (r3[c] << 16);
-                    hi.x = (r0[c] >> 16) | (r1[c] & 0xffff0000u);
-                    hi.y = (r2[c] >> 16) | (r3[c] & 0xffff0000u);
-                    *(uint2 *)(vl + vt_off(dc * 8 + 2 * c, pos)) = lo;
-                    *(uint2 *)(vl + vt_off(dc * 8 + 2 * c + 1, pos)) = hi;
-                }
+            const int c = tid + j * T;
+            if (V_CHUNKS >= T || c < V_CHUNKS) {
+                const int row = c / V_CPR, col = c % V_CPR;
+                *(uint4 *)(vl + row * VROW + col * 16) = vst[j];
             }
         }
         if (PER_KEY && tid < BK) *(float *)(vl + V_TILE + tid * 4) = sst;
     };
 
-    // ---- accumulators and softmax state, one query per lane and group ----
-    f32x16 oacc[QG][DB];
-    float m_run[QG], l_run[QG], sq_lane[QG];
+    // ---- accumulators and softmax state, one query per lane ----
+    typedef typename std::conditional<MODE == MODE_I8, i32x16, f32x16>::type acc_t;
+    f32x16 oacc[DB];
 #pragma unroll
-    for (int g = 0; g < QG; ++g) {
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+    float m_run = NEG_SENTINEL;  // running max in the exp2 domain (x * log2e)
+    float l_run = 0.f;           // this lane half's part of the running sum
+    float sq_lane = 1.f;
+    if (MODE == MODE_I8) {
+        const int nqb = (N + p.bq - 1) / p.bq;
+        sq_lane = p.sq[(size_t)bh * nqb + min(q_row, N - 1) / p.bq];
+    }
+    const float c_scale = p.scale * LOG2E;
+    // ---- per-block pipeline ----------------------------------------------------------
+    // A tile is two blocks of 32 keys.  For every block the wave alternates between the
+    // matrix pipe and the vector ALU, and every LDS fragment is requested one phase before
+    // the MFMAs that consume it, so that no MFMA waits for LDS latency:
+    //   P1  request V^T fragments of the block;  S^T = K . Q^T   (K fragments already here)
+    //   P2  online softmax of the block (vector ALU)
+    //   P3  request K fragments of the next block;  O^T += V^T . P^T
+    // The other wave of the SIMD is in a different phase most of the time, which is what
+    // keeps both pipes busy; the fences stop the compiler from merging the phases.
+    uint4 kf[KSTEPS];   // K fragments of the block about to be multiplied
+    uint2 vf[DB][2][2]; // V^T fragments of the block about to be added: [channel block][16-key step][4+4 keys]
+
+    auto load_kf = [&](const unsigned char *kl, int blk) __attribute__((always_inline)) {
+        const unsigned char *krow = kl + (blk * 32 + i32) * KROW + h * 16;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) kf[st] = *(const uint4 *)(krow + st * 32);
+    };
+    auto load_vf = [&](const unsigned char *vl, int blk) __attribute__((always_inline)) {
+        // this lane's corner of the transposing reads: key row 4h + (lane%16)/4, channels
+        // 16*((lane/16)%2) + 4*(lane%4) .. +3 of a 32-channel block
+        const unsigned char *vrd = vl + (blk * 32 + 4 * h + ((lane & 15) >> 2)) * VROW + (((lane >> 4) & 1) * 16 + (lane & 3) * 4) * 2;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[g][db][r] = 0.f;
-        m_run[g] = NEG_SENTINEL;  // running max in the exp2 domain (x * log2e)
-        l_run[g] = 0.f;           // this lane half's part of the running sum
-        sq_lane[g] = 1.f;
-        if (MODE == MODE_I8) {
-            const int nqb = (N + p.bq - 1) / p.bq;
-            sq_lane[g] = p.sq[(size_t)bh * nqb + min(q_row[g], N - 1) / p.bq];
+            for (int ks = 0; ks < 2; ++ks) {
+                vf[db][ks][0] = lds_read_tr16(vrd + (ks * 16) * VROW + db * 64);
+                vf[db][ks][1] = lds_read_tr16(vrd + (ks * 16 + 8) * VROW + db * 64);
+            }
+    };
+    auto mfma_qk = [&]() __attribute__((always_inline)) -> acc_t {
+        acc_t s;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            if constexpr (MODE == MODE_I8)
+                s = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kf[st]), __builtin_bit_cast(i32x4, qreg[st]), s, 0, 0, 0);
+            else
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s, 0, 0, 0);
         }
-    }
-    const float c_scale = p.scale * LOG2E;
+        return s;
+    };
+    auto mfma_pv = [&](const uint4 (&pb)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const uint4 a = make_uint4(vf[db][ks][0].x, vf[db][ks][0].y, vf[db][ks][1].x, vf[db][ks][1].y);
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                                   __builtin_bit_cast(bf16x8, pb[ks]), oacc[db], 0, 0, 0);
+            }
+    };
+
+    // GENERIC handles everything (additive mask, causal and key-length masking, per-key
+    // scales); the other instantiation is for tiles in which no key is masked for this wave.
+    auto tile_body = [&](auto generic_c, int it) __attribute__((always_inline)) {
+        constexpr bool GENERIC = decltype(generic_c)::value;
+        const int k0 = it * BK;
+        const unsigned char *kl = lds + (it % NSTAGE) * STAGE;
+        const unsigned char *vl = kl + K_TILE;
+        float f_tile = 1.f;
+        if (MODE == MODE_I8 && !PER_KEY) f_tile = p.sk[(size_t)kv_bh * nkb + (it >> p.bk_tile_shift)];
+        load_kf(kl, 0);
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            // ---- P1 ----
+            load_vf(vl, blk);
+            acc_t s = mfma_qk();
+            ARHIP_FENCE();
+            // ---- P2 ----
+            if (DBG) {
+                if (bh == p.dbg_bh && (wq0 >> 5) == p.dbg_qt && it == p.dbg_kt) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p.dbg[i32 * 64 + blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] = (int32_t)s[r];
+                }
+            }
+            float x[16];
+            float m_new;
+            if (!GENERIC) {
+                // max over the raw accumulators, scale folded into the exponent:
+                // s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322
+                const float c = (MODE == MODE_I8) ? ((sq_lane * f_tile) * p.scale) * LOG2E : c_scale;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x[r] = (float)s[r];
+                float mx = fmaxf(x[0], x[1]);
+#pragma unroll
+                for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(x[r], x[r + 1]));
+                mx = xhalf_max(mx);
+                m_new = fmaxf(m_run, mx * c);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -m_new));
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kt = blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3);  // key within the tile
+                    const int key = k0 + kt;
+                    float c = c_scale;
+                    if (MODE == MODE_I8) {
+                        const float skv = PER_KEY ? *(const float *)(vl + V_TILE + kt * 4) : f_tile;
+                        c = ((sq_lane * skv) * p.scale) * LOG2E;
+                    }
+                    float xv = (float)s[r] * c;
+                    if (HAS_MASK) {
+                        if (key < N && q_row < N) xv += p.mask[(size_t)q_row * N + key] * LOG2E;
+                    }
+                    if (key >= kend || (CAUSAL && key > q_row)) xv = NEG_SENTINEL;
+                    x[r] = xv;
+                }
+                float mx = fmaxf(x[0], x[1]);
+#pragma unroll
+                for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(x[r], x[r + 1]));
+                mx = xhalf_max(mx);
+                m_new = fmaxf(m_run, mx);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+            }
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            // row sum over the unrounded probabilities (src/runtime/cuda_flash_bf16.rs:365-377)
+            float rs0 = (x[0] + x[1]) + (x[2] + x[3]), rs1 = (x[8] + x[9]) + (x[10] + x[11]);
+            rs0 += (x[4] + x[5]) + (x[6] + x[7]);
+            rs1 += (x[12] + x[13]) + (x[14] + x[15]);
+            // P (bf16) as the B operand, 2 steps of 16 keys
+            uint4 pb[2];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                pb[ks].x = pack_bf16x2(x[ks * 8 + 0], x[ks * 8 + 1]);
+                pb[ks].y = pack_bf16x2(x[ks * 8 + 2], x[ks * 8 + 3]);
+                pb[ks].z = pack_bf16x2(x[ks * 8 + 4], x[ks * 8 + 5]);
+                pb[ks].w = pack_bf16x2(x[ks * 8 + 6], x[ks * 8 + 7]);
+            }
+            l_run = l_run * alpha + (rs0 + rs1);
+            ARHIP_FENCE();
+            // rescale the accumulators only when some lane's maximum moved
+            if (__any(alpha != 1.0f)) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+            }
+            // ---- P3 ----
+            if (blk == 0) load_kf(kl, 1);
+            mfma_pv(pb);
+            ARHIP_FENCE();
+        }
+    };
 
     if (ntiles > 0) {
         load_tile(0);
@@ -303,177 +423,53 @@ __global__ void __launch_bounds__(NW * 64) attn_fwd_kernel(const AttnParams p)
     wait_vmem();  // Q and the first tile have landed: nothing is pending at loop entry
     __syncthreads();
 
-    // S^T block: 32 keys x 32 queries for every query group, raw accumulators
-    typedef typename std::conditional<MODE == MODE_I8, i32x16, f32x16>::type acc_t;
-    auto qk_block = [&](const unsigned char *kl, int blk, acc_t (&s)[QG]) {
-        const unsigned char *krow = kl + (blk * 32 + i32) * KROW + h * 16;
-#pragma unroll
-        for (int g = 0; g < QG; ++g)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[g][r] = 0;
-#pragma unroll
-        for (int st = 0; st < KSTEPS; ++st) {
-            const uint4 a = *(const uint4 *)(krow + st * 32);
-#pragma unroll
-            for (int g = 0; g < QG; ++g) {
-                if constexpr (MODE == MODE_I8)
-                    s[g] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a),
-                                                                 __builtin_bit_cast(i32x4, qreg[g][st]), s[g], 0, 0, 0);
-                else
-                    s[g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                                   __builtin_bit_cast(bf16x8, qreg[g][st]), s[g], 0, 0, 0);
-            }
+    if constexpr (!CAUSAL && !HAS_MASK && !PER_KEY) {
+        // only the last tile can hold masked keys: keep it out of the loop
+        const int nfull = kend / BK;
+#pragma clang loop unroll(disable)
+        for (int it = 0; it < nfull; ++it) {
+            if (it + 1 < ntiles) load_tile((it + 1) * BK);
+            tile_body(std::false_type{}, it);
+            if (it + 1 < ntiles) store_tile((it + 1) % NSTAGE);
+            __syncthreads();
         }
-    };
-
-    int sk_idx = 0, sk_fill = 0;
-    for (int it = 0; it < ntiles; ++it) {
-        const int k0 = it * BK;
-        const int stage = it & 1;
-        if (it + 1 < ntiles) load_tile(k0 + BK);
-
-        // a wave whose queries all precede this tile has nothing to do in it
-        const bool active = !CAUSAL || (k0 <= wq0 + WQ - 1);
-        if (active) {
-            const unsigned char *kl = lds + stage * STAGE;
-            const unsigned char *vl = kl + K_TILE;
-
-            // tile-uniform K scale (block sizes that are multiples of the tile)
-            float f_tile = c_scale;
-            if (MODE == MODE_I8 && !PER_KEY) f_tile = p.sk[(size_t)kv_bh * nkb + sk_idx];
-
-            acc_t sacc[2][QG];
-            qk_block(kl, 0, sacc[0]);
-#pragma unroll
-            for (int blk = 0; blk < 2; ++blk) {
-                if (blk == 0) qk_block(kl, 1, sacc[1]);
-                const int kb0 = k0 + blk * 32;  // first key of the block
-
-                uint4 pb[QG][2];
-#pragma unroll
-                for (int g = 0; g < QG; ++g) {
-                    acc_t &s = sacc[blk][g];
-                    if (DBG) {
-                        if (bh == p.dbg_bh && ((wq0 >> 5) + g) == p.dbg_qt && it == p.dbg_kt) {
-#pragma unroll
-                            for (int r = 0; r < 16; ++r)
-                                p.dbg[i32 * 64 + blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] = (int32_t)s[r];
-                        }
-                    }
-                    float x[16];
-                    float m_new;
-                    const bool edge = (kb0 + 32 > kend) || (CAUSAL && (kb0 + 31 > wq0 + g * 32));
-                    if (!HAS_MASK && !PER_KEY && !edge) {
-                        // fast path: max over the raw accumulators, scale folded into the exponent
-                        // s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322
-                        const float c = (MODE == MODE_I8) ? ((sq_lane[g] * f_tile) * p.scale) * LOG2E : c_scale;
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) x[r] = (float)s[r];
-                        float mx = fmaxf(x[0], x[1]);
-#pragma unroll
-                        for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(x[r], x[r + 1]));
-                        mx = xhalf_max(mx);
-                        m_new = fmaxf(m_run[g], mx * c);
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -m_new));
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int key = kb0 + 8 * (r >> 2) + 4 * h + (r & 3);
-                            float c = c_scale;
-                            if (MODE == MODE_I8) {
-                                const float skv = PER_KEY ? *(const float *)(vl + V_TILE + (key - k0) * 4) : f_tile;
-                                c = ((sq_lane[g] * skv) * p.scale) * LOG2E;
-                            }
-                            float xv = (float)s[r] * c;
-                            if (HAS_MASK) {
-                                if (key < N && q_row[g] < N) xv += p.mask[(size_t)q_row[g] * N + key] * LOG2E;
-                            }
-                            if (key >= kend || (CAUSAL && key > q_row[g])) xv = NEG_SENTINEL;
-                            x[r] = xv;
-                        }
-                        float mx = fmaxf(x[0], x[1]);
-#pragma unroll
-                        for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(x[r], x[r + 1]));
-                        mx = xhalf_max(mx);
-                        m_new = fmaxf(m_run[g], mx);
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
-                    }
-                    const float alpha = __builtin_amdgcn_exp2f(m_run[g] - m_new);
-                    m_run[g] = m_new;
-                    float rs = (x[0] + x[1]) + (x[2] + x[3]);
-#pragma unroll
-                    for (int r = 4; r < 16; r += 4) rs += (x[r] + x[r + 1]) + (x[r + 2] + x[r + 3]);
-                    l_run[g] = l_run[g] * alpha + rs;
-                    // rescale the accumulators only when some lane's maximum moved
-                    if (__any(alpha != 1.0f)) {
-#pragma unroll
-                        for (int db = 0; db < DB; ++db)
-#pragma unroll
-                            for (int r = 0; r < 16; ++r) oacc[g][db][r] *= alpha;
-                    }
-                    // P (bf16) as the B operand: 2 steps of 16 keys
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        pb[g][ks].x = pack_bf16x2(x[ks * 8 + 0], x[ks * 8 + 1]);
-                        pb[g][ks].y = pack_bf16x2(x[ks * 8 + 2], x[ks * 8 + 3]);
-                        pb[g][ks].z = pack_bf16x2(x[ks * 8 + 4], x[ks * 8 + 5]);
-                        pb[g][ks].w = pack_bf16x2(x[ks * 8 + 6], x[ks * 8 + 7]);
-                    }
-                }
-
-                // ---- O^T += V^T . P^T for the 32 keys of the block ----
-#pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    const int d = db * 32 + i32;
-#pragma unroll
-                    for (int ks = 0; ks < 2; ++ks) {
-                        const uint4 a = *(const uint4 *)(vl + vt_off(d, blk * 32 + ks * 16 + h * 8));
-#pragma unroll
-                        for (int g = 0; g < QG; ++g)
-                            oacc[g][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, pb[g][ks]), oacc[g][db], 0, 0, 0);
-                    }
-                }
+        if (nfull < ntiles) tile_body(std::true_type{}, nfull);
+    } else {
+#pragma clang loop unroll(disable)
+        for (int it = 0; it < ntiles; ++it) {
+            if (it + 1 < ntiles) load_tile((it + 1) * BK);
+            if (it < my_tiles) {
+                const int k0 = it * BK;
+                const bool masked = (k0 + BK > kend) || (CAUSAL && (k0 + BK - 1 > wq0));
+                if (HAS_MASK || PER_KEY || masked) tile_body(std::true_type{}, it);
+                else tile_body(std::false_type{}, it);
             }
-        }
-
-        if (it + 1 < ntiles) store_tile(stage ^ 1);
-        __syncthreads();
-        if (MODE == MODE_I8 && !PER_KEY) {  // advance the K-block index without dividing
-            sk_fill += BK;
-            if (sk_fill >= p.bk) {
-                sk_fill = 0;
-                ++sk_idx;
-            }
+            if (it + 1 < ntiles) store_tile((it + 1) % NSTAGE);
+            __syncthreads();
         }
     }
 
     // ---- normalise and store: acc * (l > 0 ? 1/l : 0), cuda_flash_bf16.rs:414-426 ----
+    const float l_tot = xhalf_sum(l_run);
+    const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+    if (q_row < N) {
+        const size_t obase = ((size_t)bh * N + q_row) * D;
 #pragma unroll
-    for (int g = 0; g < QG; ++g) {
-        const float l_tot = xhalf_sum(l_run[g]);
-        const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
-        if (q_row[g] < N) {
-            const size_t obase = ((size_t)bh * N + q_row[g]) * D;
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int gg = 0; gg < 4; ++gg) {
-                    const int d = db * 32 + 8 * gg + 4 * h;
-                    const float o0 = oacc[g][db][4 * gg + 0] * inv, o1 = oacc[g][db][4 * gg + 1] * inv;
-                    const float o2 = oacc[g][db][4 * gg + 2] * inv, o3 = oacc[g][db][4 * gg + 3] * inv;
-                    if (OUT_F32) {
-                        *(float4 *)((float *)p.o + obase + d) = make_float4(o0, o1, o2, o3);
-                    } else {
-                        uint2 w;
-                        w.x = pack_bf16x2(o0, o1);
-                        w.y = pack_bf16x2(o2, o3);
-                        *(uint2 *)((uint16_t *)p.o + obase + d) = w;
-                    }
+            for (int gg = 0; gg < 4; ++gg) {
+                const int d = db * 32 + 8 * gg + 4 * h;
+                const float o0 = oacc[db][4 * gg + 0] * inv, o1 = oacc[db][4 * gg + 1] * inv;
+                const float o2 = oacc[db][4 * gg + 2] * inv, o3 = oacc[db][4 * gg + 3] * inv;
+                if (OUT_F32) {
+                    *(float4 *)((float *)p.o + obase + d) = make_float4(o0, o1, o2, o3);
+                } else {
+                    uint2 w;
+                    w.x = pack_bf16x2(o0, o1);
+                    w.y = pack_bf16x2(o2, o3);
+                    *(uint2 *)((uint16_t *)p.o + obase + d) = w;
                 }
-        }
+            }
     }
 }
 

@@ -41,47 +41,41 @@ static int check_common(const char *fn, arhip_device *dev, const void *q, const 
 }
 
 // CAUSAL / HAS_MASK dispatch for one tiling variant.
-template <int D, int NW, int QG, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool MASKS>
+template <int D, int NW, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool MASKS>
 static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bool has_mask)
 {
     const dim3 grid((unsigned)p.total), block(NW * 64);
     if constexpr (MASKS) {
         if (has_mask) {
             if (causal)
-                hipLaunchKernelGGL((attn_fwd_kernel<D, NW, QG, true, true, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
+                hipLaunchKernelGGL((attn_fwd_kernel<D, NW, true, true, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
             else
-                hipLaunchKernelGGL((attn_fwd_kernel<D, NW, QG, false, true, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
+                hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, true, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
             return;
         }
     }
     if (causal)
-        hipLaunchKernelGGL((attn_fwd_kernel<D, NW, QG, true, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((attn_fwd_kernel<D, NW, true, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL((attn_fwd_kernel<D, NW, QG, false, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
 }
 
-// Tiling variants: waves per workgroup x query groups (of 32) per wave.
-//   V_1x1  32 queries per workgroup: short sequences, spreads over the chip
-//   V_4x1  128 queries, every K/V fragment read from LDS feeds one MFMA
-//   V_8x1  256 queries, two waves per SIMD
-//   V_4x2  256 queries, every fragment feeds two MFMAs (half the LDS traffic)
-enum { V_1x1 = 0, V_4x1 = 1, V_8x1 = 2, V_4x2 = 3 };
-
-static int variant_queries(int v) { return v == V_1x1 ? 32 : (v == V_4x1 ? 128 : 256); }
-
-static int pick_variant(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bool special)
+// Tiling variants = waves (of 32 queries) per workgroup.
+//   1  32 queries per workgroup: short sequences, spreads the heads over the chip
+//   4  128 queries
+//   8  256 queries, two waves per SIMD running one phase apart (long sequences)
+static int pick_waves(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bool special)
 {
-    // masks, per-key scales and the debug export are only built for V_4x1 (and V_1x1 at D = 64)
-    int v;
-    const int64_t wg128 = heads * ((N + 127) / 128);
-    if (D == 64 && wg128 < 2 * (int64_t)dev->cus) v = V_1x1;
-    else if (special) v = V_4x1;
-    else v = (heads * ((N + 255) / 256) >= 2 * (int64_t)dev->cus) ? V_8x1 : V_4x1;
-    if (const char *e = getenv("ARHIP_ATTN_VARIANT")) {  // tuning aid; results do not depend on it
+    // masks, per-key scales and the debug export are built for 4 waves (and 1 at D = 64) only
+    int nw;
+    if (D == 64 && heads * ((N + 127) / 128) < 2 * (int64_t)dev->cus) nw = 1;
+    else if (special) nw = 4;
+    else nw = (heads * ((N + 255) / 256) >= 2 * (int64_t)dev->cus) ? 8 : 4;
+    if (const char *e = getenv("ARHIP_ATTN_WAVES")) {  // tuning aid; results do not depend on it
         const int w = atoi(e);
-        if (w >= V_1x1 && w <= V_4x2 && !special && (w != V_1x1 || D == 64)) v = w;
+        if ((w == 1 || w == 4 || w == 8) && !special && (w != 1 || D == 64)) nw = w;
     }
-    return v;
+    return nw;
 }
 
 extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, const void *v, void *o,
@@ -122,24 +116,17 @@ extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, 
     p.bq = p.bk = 1;
     p.scale = scale;
     const bool c = causal != 0, hm = mask != nullptr;
-    const int var = pick_variant(dev, B * Hq, N, D, hm);
-    const int bqv = variant_queries(var);
-    p.nq = (int)((N + bqv - 1) / bqv);
+    const int nw = pick_waves(dev, B * Hq, N, D, hm);
+    p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     if (int rc = t.begin()) return rc;
     if (D == 64) {
-        switch (var) {
-        case V_1x1: launch_attn<64, 1, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm); break;
-        case V_4x1: launch_attn<64, 4, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm); break;
-        case V_8x1: launch_attn<64, 8, 1, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm); break;
-        default: launch_attn<64, 4, 2, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm); break;
-        }
+        if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
+        else if (nw == 4) launch_attn<64, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
+        else launch_attn<64, 8, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm);
     } else {
-        switch (var) {
-        case V_4x1: launch_attn<128, 4, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm); break;
-        case V_8x1: launch_attn<128, 8, 1, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm); break;
-        default: launch_attn<128, 4, 2, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm); break;
-        }
+        if (nw == 4) launch_attn<128, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
+        else launch_attn<128, 8, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm);
     }
     arhip_note_selected(ARHIP_K_FLASH_BF16);
     return t.end();
@@ -170,13 +157,15 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
     p.scale = scale;
     const bool dbg = dbg_logits != nullptr;
     const bool c = causal != 0, hm = mask != nullptr, f32o = out_dtype == ARHIP_F32;
-    // K scales that are uniform over a 64-key tile take the fast kernel; anything else
-    // (including the reference's per-key scales, bk == 1) stages the tile's scales in LDS
-    const bool per_key = (bk % 64) != 0;
-    int var = pick_variant(dev, B * Hq, N, D, hm || per_key || dbg);
-    if (var == V_1x1) var = V_4x1;
-    const int bqv = variant_queries(var);
-    p.nq = (int)((N + bqv - 1) / bqv);
+    // K scales that are uniform over a 64-key tile (bk = 64 * 2^n) take the fast kernel; anything
+    // else, including the reference's per-key scales (bk == 1), stages the tile's scales in LDS
+    int shift = 0;
+    while (((int64_t)64 << shift) < bk) ++shift;
+    const bool per_key = ((int64_t)64 << shift) != bk;
+    p.bk_tile_shift = shift;
+    int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg);
+    if (nw == 1) nw = 4;
+    p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     if (dbg) {
         p.dbg = dbg_logits;
@@ -188,20 +177,19 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
     arhip_call_timer t{dev, wait, secs};
     t.kernel = ARHIP_K_SAGE;
     if (int rc = t.begin()) return rc;
-#define SAGE_V(DD, NWW, QGG, PK, DB_, MK)                                                              \
+#define SAGE_V(DD, NWW, PK, DB_, MK)                                                                   \
     do {                                                                                               \
-        if (f32o) launch_attn<DD, NWW, QGG, MODE_I8, PK, true, DB_, MK>(dev->stream, p, c, hm);        \
-        else launch_attn<DD, NWW, QGG, MODE_I8, PK, false, DB_, MK>(dev->stream, p, c, hm);            \
+        if (f32o) launch_attn<DD, NWW, MODE_I8, PK, true, DB_, MK>(dev->stream, p, c, hm);             \
+        else launch_attn<DD, NWW, MODE_I8, PK, false, DB_, MK>(dev->stream, p, c, hm);                 \
     } while (0)
 #define SAGE_D(DD)                                                                                     \
     do {                                                                                               \
         if (dbg) {                                                                                     \
-            if (per_key) SAGE_V(DD, 4, 1, true, true, false);                                          \
-            else SAGE_V(DD, 4, 1, false, true, false);                                                 \
-        } else if (per_key) SAGE_V(DD, 4, 1, true, false, true);                                       \
-        else if (var == V_4x1) SAGE_V(DD, 4, 1, false, false, true);                                   \
-        else if (var == V_8x1) SAGE_V(DD, 8, 1, false, false, false);                                  \
-        else SAGE_V(DD, 4, 2, false, false, false);                                                    \
+            if (per_key) SAGE_V(DD, 4, true, true, false);                                             \
+            else SAGE_V(DD, 4, false, true, false);                                                    \
+        } else if (per_key) SAGE_V(DD, 4, true, false, true);                                          \
+        else if (nw == 4) SAGE_V(DD, 4, false, false, true);                                           \
+        else SAGE_V(DD, 8, false, false, false);                                                       \
     } while (0)
     if (D == 64) SAGE_D(64);
     else SAGE_D(128);

@@ -64,8 +64,12 @@ def test_block_quantised_smoothed(dev, N, causal, D):
     assert np.array_equal(r["logits"][:i1 - i0, :j1 - j0], want_logits)
     want = oracle.sage(q8, k8, sq, sk, v, bq, bk, causal=causal)
     assert np.abs(r["out"] - want).max() < 2e-3
-    if not causal:
-        truth = oracle.sdpa_f64(q, k, v)
+    # against the exact result the int8 quantisation itself costs ~1e-2 (more when a row sees
+    # few keys: the emulation, not the kernel, is what exceeds 2e-2 at N = 64); the kernel must
+    # not add to that, and meets the 2e-2 bound where the algorithm does
+    truth = oracle.sdpa_f64(q, k, v, causal=causal)
+    assert np.abs(r["out"] - truth).max() <= np.abs(want - truth).max() + 2e-3
+    if not causal and N >= 256:
         assert np.abs(r["out"] - truth).max() <= 2e-2
 
 
