@@ -55,6 +55,7 @@ constexpr int MODE_I8 = 1;    // q, k int8 with block scales
 constexpr int BK = 64;        // keys per tile
 constexpr float NEG_SENTINEL = -1e30f;  // src/runtime/cuda_flash_bf16.rs:106 (AR_NEG)
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LAZY_TAU = 8.0f;  // log2 units the running maximum may outgrow the exponent reference
 
 struct AttnParams {
     const void *q;
@@ -80,6 +81,14 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
     bf16x2 p = {(__bf16)lo, (__bf16)hi};  // round-to-nearest-even
     return __builtin_bit_cast(uint32_t, p);
+}
+
+// v_max3_f32 (the generic fmaxf spends an extra instruction per operand on NaN quieting)
+__device__ __forceinline__ float max3(float a, float b, float c)
+{
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
 }
 
 // lane and lane^32 hold the same query: combine their partial results.
@@ -345,52 +354,62 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
                     for (int r = 0; r < 16; ++r) p.dbg[i32 * 64 + blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] = (int32_t)s[r];
                 }
             }
+            // The exponent reference m_run is only moved when some query's maximum outgrows it
+            // by more than LAZY_TAU (then the accumulators are rescaled); otherwise it stays put and
+            // the probabilities of this block are at most 2^LAZY_TAU.  Softmax does not depend on
+            // the reference, so this only saves the rescale almost every time.
             float x[16];
-            float m_new;
+            float c = c_scale;  // fast path: scale folded into the exponent
             if (!GENERIC) {
-                // max over the raw accumulators, scale folded into the exponent:
                 // s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322
-                const float c = (MODE == MODE_I8) ? ((sq_lane * f_tile) * p.scale) * LOG2E : c_scale;
+                if (MODE == MODE_I8) c = ((sq_lane * f_tile) * p.scale) * LOG2E;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) x[r] = (float)s[r];
-                float mx = fmaxf(x[0], x[1]);
-#pragma unroll
-                for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(x[r], x[r + 1]));
-                mx = xhalf_max(mx);
-                m_new = fmaxf(m_run, mx * c);
-#pragma unroll
-                for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -m_new));
             } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int kt = blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3);  // key within the tile
                     const int key = k0 + kt;
-                    float c = c_scale;
+                    float cc = c_scale;
                     if (MODE == MODE_I8) {
                         const float skv = PER_KEY ? *(const float *)(vl + V_TILE + kt * 4) : f_tile;
-                        c = ((sq_lane * skv) * p.scale) * LOG2E;
+                        cc = ((sq_lane * skv) * p.scale) * LOG2E;
                     }
-                    float xv = (float)s[r] * c;
+                    float xv = (float)s[r] * cc;
                     if (HAS_MASK) {
                         if (key < N && q_row < N) xv += p.mask[(size_t)q_row * N + key] * LOG2E;
                     }
                     if (key >= kend || (CAUSAL && key > q_row)) xv = NEG_SENTINEL;
                     x[r] = xv;
                 }
-                float mx = fmaxf(x[0], x[1]);
-#pragma unroll
-                for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(x[r], x[r + 1]));
-                mx = xhalf_max(mx);
-                m_new = fmaxf(m_run, mx);
-#pragma unroll
-                for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
             }
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            m_run = m_new;
+            float mx = max3(x[0], x[1], x[2]);
+#pragma unroll
+            for (int r = 3; r < 15; r += 2) mx = max3(mx, x[r], x[r + 1]);
+            mx = xhalf_max(fmaxf(mx, x[15]));
+            if (!GENERIC) mx *= c;
+            if (__any(mx > m_run + LAZY_TAU)) {
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+            }
+            if (!GENERIC) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -m_run));
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_run);
+            }
             // row sum over the unrounded probabilities (src/runtime/cuda_flash_bf16.rs:365-377)
             float rs0 = (x[0] + x[1]) + (x[2] + x[3]), rs1 = (x[8] + x[9]) + (x[10] + x[11]);
             rs0 += (x[4] + x[5]) + (x[6] + x[7]);
             rs1 += (x[12] + x[13]) + (x[14] + x[15]);
+            l_run += rs0 + rs1;
             // P (bf16) as the B operand, 2 steps of 16 keys
             uint4 pb[2];
 #pragma unroll
@@ -400,15 +419,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
                 pb[ks].z = pack_bf16x2(x[ks * 8 + 4], x[ks * 8 + 5]);
                 pb[ks].w = pack_bf16x2(x[ks * 8 + 6], x[ks * 8 + 7]);
             }
-            l_run = l_run * alpha + (rs0 + rs1);
             ARHIP_FENCE();
-            // rescale the accumulators only when some lane's maximum moved
-            if (__any(alpha != 1.0f)) {
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-            }
             // ---- P3 ----
             if (blk == 0) load_kf(kl, 1);
             mfma_pv(pb);
