@@ -9,17 +9,18 @@
 //           plus one exchange with lane^32, and the probabilities are already in
 //           the operand layout the second product needs: O^T = V^T . P^T, again
 //           with one query per lane (the softmax rescale is a per-lane scalar).
-//   tiles : BK = 64 keys per step, K and V^T staged through LDS by the whole
+//   tiles : BK = 64 keys per step, K and V staged through LDS by the whole
 //           workgroup: 128-bit global loads issued one tile ahead into
-//           registers, written to the next LDS stage after the math; one
+//           registers, written to the other LDS stage after the math; one
 //           barrier per tile.
-//   skew  : with 8 waves (two per SIMD) the upper four run one phase behind the
-//           lower four: while waves 0-3 multiply Q.K^T of tile i on the matrix
-//           cores, waves 4-7 exponentiate tile i-1 on the vector ALU, and vice
-//           versa.  Both halves of a SIMD's issue slots stay busy instead of
-//           all waves queueing for the same pipe after every barrier.  The
-//           lagging waves still read V of tile i-1 while tile i+1 is written, so
-//           this mode cycles through three LDS stages instead of two.
+//   blocks: inside a tile the online softmax advances 32 keys at a time and the
+//           wave alternates between the matrix pipe and the vector ALU; every
+//           LDS fragment is requested one phase before the MFMAs that use it.
+//           With 8 waves per workgroup each SIMD holds two waves, and one of
+//           them can exponentiate while the other multiplies.
+//   lazy  : the exponent reference only moves (and the accumulators are only
+//           rescaled) when a row maximum outgrows it by 2^8; softmax does not
+//           depend on the reference, so the result is the same function.
 //
 // MFMA shapes (wave64):
 //   v_mfma_f32_32x32x16_bf16  A[32 x 16] . B[16 x 32]   lane: row/col = lane%32,
@@ -114,14 +115,8 @@ __device__ __forceinline__ uint2 lds_read_tr16(const unsigned char *p)
     return __builtin_bit_cast(uint2, v);
 }
 
-#ifndef ARHIP_FENCES
-#define ARHIP_FENCES 1
-#endif
-#if ARHIP_FENCES
+// Scheduling fence: the compiler may reorder freely inside a phase, not across this line.
 #define ARHIP_FENCE() __builtin_amdgcn_sched_barrier(0)
-#else
-#define ARHIP_FENCE() ((void)0)
-#endif
 
 // s_waitcnt vmcnt(0): all outstanding global loads of this wave have landed.
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
