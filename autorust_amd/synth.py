@@ -1,8 +1,9 @@
 """Synthetic inputs for tests, smoke and bench: a counter-based generator that
 does not depend on NumPy's RNG state or version, plus bf16 bit conversions.
 
-normal(seed, n): splitmix64(seed, index) -> two 32-bit uniforms -> Box-Muller in
-float64 -> float32.  The same seed and index give the same value everywhere.
+normal(seed, n): splitmix64(seed, index // 2) -> two 32-bit uniforms -> Box-Muller in
+float64 (cosine branch for even indices, sine branch for odd ones) -> float32.  The same
+seed and index give the same value everywhere.
 """
 import numpy as np
 
@@ -26,16 +27,36 @@ def uniform(seed, n, offset=0):
     return ((z >> np.uint64(11)).astype(np.float64) + 0.5) * (1.0 / 9007199254740992.0)
 
 
-def normal(seed, shape, chunk=1 << 24):
-    """float32 N(0,1) of the given shape."""
+def _normal_chunk(args):
+    seed, out, o, m = args
+    # element i comes from counter i // 2: the cosine branch for even i, the sine branch for odd i
+    p0, p1 = o // 2, (o + m + 1) // 2
+    z = splitmix64(seed, p1 - p0, p0)
+    u1 = ((z >> np.uint64(32)).astype(np.float64) + 0.5) * (1.0 / 4294967296.0)
+    u2 = ((z & np.uint64(0xFFFFFFFF)).astype(np.float64) + 0.5) * (1.0 / 4294967296.0)
+    r = np.sqrt(-2.0 * np.log(u1))
+    t = (2.0 * np.pi) * u2
+    both = np.empty(2 * (p1 - p0), dtype=np.float32)
+    both[0::2] = r * np.cos(t)
+    both[1::2] = r * np.sin(t)
+    out[o:o + m] = both[o - 2 * p0:o - 2 * p0 + m]
+
+
+def normal(seed, shape, chunk=1 << 21):
+    """float32 N(0,1) of the given shape (chunks are generated on a few threads; the values do
+    not depend on the chunking)."""
+    import concurrent.futures
+    import os
     n = int(np.prod(shape))
     out = np.empty(n, dtype=np.float32)
-    for o in range(0, n, chunk):
-        m = min(chunk, n - o)
-        z = splitmix64(seed, m, o)
-        u1 = ((z >> np.uint64(32)).astype(np.float64) + 0.5) * (1.0 / 4294967296.0)
-        u2 = ((z & np.uint64(0xFFFFFFFF)).astype(np.float64) + 0.5) * (1.0 / 4294967296.0)
-        out[o:o + m] = (np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)).astype(np.float32)
+    jobs = [(seed, out, o, min(chunk, n - o)) for o in range(0, n, chunk)]
+    workers = max(1, min(16, os.cpu_count() or 1, len(jobs)))
+    if workers == 1:
+        for j in jobs:
+            _normal_chunk(j)
+    else:
+        with concurrent.futures.ThreadPoolExecutor(workers) as ex:
+            list(ex.map(_normal_chunk, jobs))
     return out.reshape(shape)
 
 

@@ -108,3 +108,23 @@ def run_sage(dev, q, k, v, bq, bk, smooth=True, in_dtype=F32, out_dtype=F32, mas
         if dbg is not None:
             res["logits"] = dbg.copyout(np.int32, (32, 64))
         return res
+
+
+def bf16_ulps(got, want, floor=0.5):
+    """Largest |got - want| in units of the bf16 step at max(|want|, floor), the step being
+    2^(floor(log2 m) - 7).  A bf16-stored output that differs from the emulation only through
+    rounding points is a couple of steps away at most; below `floor` the error is governed by
+    the rounding of the probabilities (relative to sum p|v|, not to |o|), hence the floor.
+    Three steps at the floor are 5.9e-3, the reference's 5e-3 (tests/flash_cuda_bf16.rs:131)."""
+    mag = np.maximum(np.abs(want), floor)
+    step = 2.0 ** (np.floor(np.log2(mag)) - 7)
+    return float((np.abs(got - want) / step).max())
+
+
+def max_abs(a, b):
+    return float(np.abs(a - b).max())
+
+
+def max_rel1(a, b):
+    """max |a-b| / max(|b|, 1): the reference's closeness measure (tests/nn_attention.rs:11-24)."""
+    return float((np.abs(a - b) / np.maximum(np.abs(b), 1.0)).max())
