@@ -81,3 +81,11 @@ extern "C" __global__ void probe_axpb(const float *x, float *y, int n)
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) y[i] = x[i] * 3.0f + 1.0f;
 }
+
+// Plain streaming copy of n 16-byte words: the calibration kernel for the HBM traffic
+// counters (its traffic is known: n*16 bytes read, n*16 bytes written).
+extern "C" __global__ void probe_copy(const uint4 *src, uint4 *dst, long n)
+{
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}

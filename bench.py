@@ -218,6 +218,9 @@ def main():
     ap.add_argument("--workload", default="sage",
                     choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32"])
     ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="one step of the workload plus one plain 1 GiB copy kernel and nothing else: "
+                         "the run to put under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -228,6 +231,17 @@ def main():
     t0 = time.time()
     w = build_workload(dev, args.workload)
     log("inputs for %s ready in %.1f s" % (w.name, time.time() - t0))
+    if args.traffic_probe:
+        w.step()
+        dev.sync()
+        n16 = (1 << 30) // 16
+        src, dst = dev.alloc(n16 * 16), dev.alloc(n16 * 16)
+        src.zero()
+        mod = dev.module_load(open(_lib.PROBES_PATH, "rb").read())
+        dev.launch(mod, "probe_copy", (4096, 1, 1), (256, 1, 1), [src, dst], [n16], [64])
+        print(json.dumps({"traffic_probe": w.name, "kernel_bytes_algorithmic": w.kernel_bytes,
+                          "copy_bytes_read": n16 * 16, "copy_bytes_written": n16 * 16}))
+        return
     res = measure(dev, w, args.steps, args.warmup)
     log(json.dumps(res))
     cpu = None
@@ -239,7 +253,7 @@ def main():
 
     secondary = []
     if not args.no_secondary:
-        for name in ("vit", "decoder", "vit_f32", "sage"):
+        for name in ("vit", "decoder", "vit_f32", "sage", "sage_causal_long"):
             if name == args.workload:
                 continue
             sw = build_workload(dev, name)
