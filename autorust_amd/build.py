@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libarhip.so")
 PROBES = os.path.join(HERE, "probes.hsaco")
+HOST_LIB = os.path.join(HERE, "libautorust_host.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 SOURCES = ["device.hip", "flash.hip", "sage_quant.hip"]
@@ -69,6 +70,12 @@ def build(force=False, verbose=False):
             if out.strip():
                 sys.stderr.write(out + "\n")
         _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    # C++ mirror of the reference's attention interface (+ the flat C shim the tests drive it with)
+    host_srcs = [os.path.join(CSRC, "host", f) for f in ("autorust_host.cpp", "host_capi.cpp")]
+    host_deps = host_srcs + [os.path.join(CSRC, "host", "autorust_host.h"), LIB]
+    if force or _newer(HOST_LIB, host_deps):
+        _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", HOST_LIB] + host_srcs +
+             ["-L" + HERE, "-larhip", "-Wl,-rpath,$ORIGIN"])
     probe_src = os.path.join(CSRC, "probes.hip")
     if os.path.exists(probe_src) and (force or _newer(PROBES, [probe_src])):
         _run([HIPCC] + FLAGS + ["--genco", probe_src, "-o", PROBES])

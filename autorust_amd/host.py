@@ -1,0 +1,226 @@
+"""Python view of the C++ host layer (csrc/host/autorust_host.h): Tensor, Session,
+AttentionKind and the attention entry points with the reference's names
+(src/tensor/mod.rs:2045-2161, src/models/flash_attention.rs:292-747).  Thin ctypes calls;
+the logic lives in C++ and computes through libarhip.so.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import _lib
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+HOST_LIB_PATH = os.path.join(_HERE, "libautorust_host.so")
+_host = None
+
+FLOAT32, BFLOAT16, OTHER = 0, 1, 2
+K_NONE, K_FLASH_F32, K_FLASH_BF16, K_SAGE = -1, 0, 1, 2
+
+
+class AttentionKind:
+    Sdpa, Flash, Sage = 0, 1, 2
+
+    @staticmethod
+    def name(k):
+        return host().arh_attention_kind_name(k).decode()
+
+    @staticmethod
+    def from_str(s):
+        return host().arh_attention_kind_from_str(s.encode())
+
+
+class Settings(ctypes.Structure):
+    _fields_ = [("attention", ctypes.c_int), ("tensor_cores", ctypes.c_int), ("async_pipeline", ctypes.c_int),
+                ("math_exact", ctypes.c_int), ("sage_block_q", ctypes.c_int64), ("sage_block_k", ctypes.c_int64),
+                ("sage_smooth_k", ctypes.c_int)]
+
+    @staticmethod
+    def default():
+        s = Settings()
+        host().arh_settings_default(ctypes.byref(s))
+        return s
+
+    @staticmethod
+    def from_env():
+        s = Settings()
+        host().arh_settings_from_env(ctypes.byref(s))
+        return s
+
+
+def host():
+    global _host
+    if _host is None:
+        _lib.load()  # libarhip.so first (the host library links against it)
+        if not os.path.exists(HOST_LIB_PATH):
+            raise FileNotFoundError("%s is missing: build it with `python -m autorust_amd.build`" % HOST_LIB_PATH)
+        h = ctypes.CDLL(HOST_LIB_PATH)
+        vp, ci, i64p = ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_int64)
+        h.arh_last_error.restype = ctypes.c_char_p
+        h.arh_attention_kind_name.restype = ctypes.c_char_p
+        h.arh_attention_kind_name.argtypes = [ci]
+        h.arh_attention_kind_from_str.argtypes = [ctypes.c_char_p]
+        h.arh_device_open.restype = vp
+        h.arh_device_open.argtypes = [ci]
+        h.arh_device_close.argtypes = [vp]
+        h.arh_device_raw_allocs.restype = ctypes.c_uint64
+        h.arh_device_raw_allocs.argtypes = [vp]
+        h.arh_tensor_from_slice.restype = vp
+        h.arh_tensor_from_slice.argtypes = [vp, ctypes.c_void_p, i64p, ci, ci]
+        h.arh_tensor_free.argtypes = [vp]
+        h.arh_tensor_numel.restype = ctypes.c_int64
+        h.arh_tensor_numel.argtypes = [vp]
+        h.arh_tensor_dtype.argtypes = [vp]
+        h.arh_tensor_shape.argtypes = [vp, i64p, ci]
+        h.arh_tensor_to_list.argtypes = [vp, ctypes.c_void_p]
+        h.arh_session_new.restype = vp
+        for f in ("arh_session_free", "arh_session_begin_capture", "arh_session_end_capture", "arh_session_replay"):
+            getattr(h, f).argtypes = [vp]
+        h.arh_session_step_info.argtypes = [vp, ci, ctypes.c_char_p, ci, i64p, i64p]
+        h.arh_attention.restype = vp
+        h.arh_attention.argtypes = [vp, vp, vp, vp, ctypes.c_double, ci, ci, vp, ctypes.POINTER(Settings)]
+        h.arh_plan_fused.argtypes = [i64p, ci, i64p, ci, i64p, ci, ci, ci, ci, i64p, ci, ci, ci, ci,
+                                     ctypes.POINTER(Settings), ctypes.POINTER(ci)]
+        h.arh_wants_fused.argtypes = [ci, ctypes.POINTER(Settings), ctypes.c_double, ci, ctypes.POINTER(ci)]
+        h.arh_selections.restype = ctypes.c_uint64
+        h.arh_selections.argtypes = [ci]
+        _host = h
+    return _host
+
+
+class HostError(RuntimeError):
+    pass
+
+
+def _err():
+    return HostError(host().arh_last_error().decode("utf-8", "replace"))
+
+
+def _i64(seq):
+    return (ctypes.c_int64 * max(len(seq), 1))(*seq)
+
+
+class HipDevice:
+    """`device("HIP")` with the reference's free-list allocator."""
+
+    def __init__(self, ordinal=0):
+        self.h = host().arh_device_open(ordinal)
+        if not self.h:
+            raise _err()
+
+    def close(self):
+        if self.h:
+            host().arh_device_close(self.h)
+            self.h = None
+
+    @property
+    def raw_allocs(self):
+        return int(host().arh_device_raw_allocs(self.h))
+
+
+class Session:
+    def __init__(self):
+        self.h = host().arh_session_new()
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            host().arh_session_free(self.h)
+            self.h = None
+
+    def begin_capture(self):
+        host().arh_session_begin_capture(self.h)
+
+    def end_capture(self):
+        """Number of captured host launches (kept inside the session for replay)."""
+        return host().arh_session_end_capture(self.h)
+
+    def step(self, i):
+        name = ctypes.create_string_buffer(64)
+        g, v = (ctypes.c_int64 * 3)(), (ctypes.c_int64 * 6)()
+        if host().arh_session_step_info(self.h, i, name, 64, g, v) != 0:
+            raise IndexError(i)
+        return name.value.decode(), list(g), list(v)
+
+    def replay(self):
+        if host().arh_session_replay(self.h) != 0:
+            raise _err()
+
+
+class Tensor:
+    def __init__(self, h):
+        self.h = h
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            host().arh_tensor_free(self.h)
+            self.h = None
+
+    @staticmethod
+    def from_slice(dev, data, shape, dtype=FLOAT32):
+        data = np.ascontiguousarray(data, dtype=np.float32)
+        h = host().arh_tensor_from_slice(dev.h, data.ctypes.data, _i64(list(shape)), len(shape), dtype)
+        if not h:
+            raise _err()
+        return Tensor(h)
+
+    @property
+    def shape(self):
+        out = (ctypes.c_int64 * 8)()
+        n = host().arh_tensor_shape(self.h, out, 8)
+        return tuple(out[:n])
+
+    @property
+    def dtype(self):
+        return host().arh_tensor_dtype(self.h)
+
+    def to_list(self):
+        out = np.empty(host().arh_tensor_numel(self.h), dtype=np.float32)
+        if host().arh_tensor_to_list(self.h, out.ctypes.data) != 0:
+            raise _err()
+        return out.reshape(self.shape)
+
+    def _call(self, api, k, v, mask, dropout_p, is_causal, sess, settings):
+        st = settings if settings is not None else Settings.default()
+        h = host().arh_attention(self.h, k.h, v.h, mask.h if mask is not None else None, float(dropout_p),
+                                 int(is_causal), api, sess.h if sess is not None else None, ctypes.byref(st))
+        if not h:
+            raise _err()
+        return Tensor(h)
+
+    def attention(self, k, v, mask=None, dropout_p=0.0, is_causal=False):
+        return self._call(0, k, v, mask, dropout_p, is_causal, None, None)
+
+    def attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None):
+        return self._call(1, k, v, mask, dropout_p, is_causal, sess, settings)
+
+    def flash_attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None):
+        return self._call(2, k, v, mask, dropout_p, is_causal, sess, settings)
+
+    def sage_attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None):
+        return self._call(3, k, v, mask, dropout_p, is_causal, sess, settings)
+
+
+def plan_fused(q, k, v, qd=FLOAT32, kd=None, vd=None, mask=None, mask_dtype=FLOAT32, enable_gqa=False, quantized=False,
+               settings=None):
+    """(kernel id, sage_declined): the gates of fused_attention_ex without a device."""
+    kd = qd if kd is None else kd
+    vd = qd if vd is None else vd
+    st = settings if settings is not None else Settings.default()
+    declined = ctypes.c_int()
+    kern = host().arh_plan_fused(_i64(q), len(q), _i64(k), len(k), _i64(v), len(v), qd, kd, vd,
+                                 _i64(mask) if mask is not None else None, len(mask) if mask is not None else 0,
+                                 mask_dtype, int(enable_gqa), int(quantized), ctypes.byref(st), ctypes.byref(declined))
+    return kern, bool(declined.value)
+
+
+def wants_fused(force, settings, dropout_p, has_session):
+    """(fused?, quantized?): the policy of Tensor::attention_kind."""
+    st = settings if settings is not None else Settings.default()
+    qz = ctypes.c_int()
+    w = host().arh_wants_fused(-1 if force is None else force, ctypes.byref(st), float(dropout_p), int(has_session),
+                               ctypes.byref(qz))
+    return bool(w), bool(qz.value)
+
+
+def selections(kernel):
+    return int(host().arh_selections(kernel))

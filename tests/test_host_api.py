@@ -1,0 +1,193 @@
+"""The C++ mirror of the reference's attention interface (csrc/host/): policy and gates on the
+CPU, the Tensor / Session path on the GPU.  The GPU cases follow the reference's dispatch tests
+(tests/flash_cuda_masks.rs:298-362, tests/flash_cuda_bf16.rs `bf16_gate_and_dispatch`,
+tests/sage_int8.rs:152-250)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from autorust_amd import host, synth
+from autorust_amd.host import (BFLOAT16, FLOAT32, K_FLASH_BF16, K_FLASH_F32, K_NONE, K_SAGE, OTHER, AttentionKind,
+                               Session, Settings, Tensor)
+
+# ------------------------------------------------------------------ CPU: policy and gates ---
+
+
+def test_attention_kind_names_and_env(monkeypatch):
+    assert [AttentionKind.name(k) for k in (0, 1, 2)] == ["sdpa", "flash", "sage"]   # flash_attention.rs:731-737
+    assert AttentionKind.from_str("sdpa") == AttentionKind.Sdpa
+    assert AttentionKind.from_str("sage") == AttentionKind.Sage
+    assert AttentionKind.from_str("anything") == AttentionKind.Flash                 # default (settings.rs:209-213)
+    monkeypatch.setenv("AUTORUST_ATTN", "sage")
+    monkeypatch.setenv("AUTORUST_MATH", "exact")
+    s = Settings.from_env()
+    assert s.attention == AttentionKind.Sage and s.math_exact == 1 and s.tensor_cores == 0   # settings.rs:202-208
+    monkeypatch.delenv("AUTORUST_MATH")
+    monkeypatch.setenv("AUTORUST_TENSOR_CORES", "0")
+    assert Settings.from_env().tensor_cores == 0
+    d = Settings.default()
+    assert d.attention == AttentionKind.Flash and d.tensor_cores == 1
+    assert (d.sage_block_q, d.sage_block_k, d.sage_smooth_k) == (128, 64, 1)
+
+
+def test_policy_matches_attention_kind():
+    # tensor/mod.rs:2198-2207: fused iff kind != Sdpa and dropout_p == 0 and a session is given
+    d = Settings.default()
+    assert host.wants_fused(None, d, 0.0, True) == (True, False)
+    assert host.wants_fused(None, d, 0.0, False) == (False, False)       # sessionless entry points always run SDPA
+    assert host.wants_fused(None, d, 0.1, True) == (False, False)        # dropout
+    assert host.wants_fused(AttentionKind.Sage, d, 0.0, True) == (True, True)
+    s = Settings.default()
+    s.attention = AttentionKind.Sdpa
+    assert host.wants_fused(None, s, 0.0, True) == (False, False)        # configured sdpa
+    assert host.wants_fused(AttentionKind.Flash, s, 0.0, True) == (True, False)   # explicit calls are never overridden
+
+
+def test_gates_of_fused_attention_ex():
+    q = [2, 4, 100, 64]
+    assert host.plan_fused(q, q, q)[0] == K_FLASH_F32
+    assert host.plan_fused(q, q, q, qd=BFLOAT16)[0] == K_FLASH_BF16
+    assert host.plan_fused(q, q, q, quantized=True) == (K_SAGE, False)
+    assert host.plan_fused([2, 4, 100, 128], [2, 4, 100, 128], [2, 4, 100, 128], qd=BFLOAT16)[0] == K_FLASH_BF16
+    # flash_attention.rs:358-396
+    assert host.plan_fused([4, 100, 64], [4, 100, 64], [4, 100, 64])[0] == K_NONE            # not 4-D
+    assert host.plan_fused(q, [2, 4, 99, 64], [2, 4, 99, 64])[0] == K_NONE                   # nk != n
+    assert host.plan_fused(q, q, [2, 4, 100, 32])[0] == K_NONE                               # dv != d
+    assert host.plan_fused(q, [2, 2, 100, 64], [2, 2, 100, 64])[0] == K_NONE                 # GQA not announced
+    assert host.plan_fused(q, [2, 2, 100, 64], [2, 2, 100, 64], enable_gqa=True)[0] == K_FLASH_F32
+    assert host.plan_fused(q, [2, 3, 100, 64], [2, 3, 100, 64], enable_gqa=True)[0] == K_NONE  # 4 % 3
+    assert host.plan_fused(q, q, q, qd=OTHER)[0] == K_NONE
+    assert host.plan_fused(q, q, q, qd=FLOAT32, kd=BFLOAT16)[0] == K_NONE                    # mixed dtypes
+    assert host.plan_fused(q, q, q, mask=[100, 100])[0] == K_FLASH_F32
+    assert host.plan_fused(q, q, q, mask=[1, 100, 100])[0] == K_NONE                         # broadcast mask -> SDPA
+    assert host.plan_fused(q, q, q, mask=[100, 100], mask_dtype=OTHER)[0] == K_NONE          # bool mask -> SDPA
+    # head_dim the kernels do not cover (tests/flash_cuda_bf16.rs:144 analogue)
+    assert host.plan_fused([1, 2, 64, 32], [1, 2, 64, 32], [1, 2, 64, 32], qd=BFLOAT16)[0] == K_NONE
+    # tensor cores off: bf16 has no fused kernel, f32 keeps the exact one, sage is declined with a notice
+    s = Settings.default()
+    s.tensor_cores = 0
+    assert host.plan_fused(q, q, q, qd=BFLOAT16, settings=s)[0] == K_NONE
+    assert host.plan_fused(q, q, q, settings=s)[0] == K_FLASH_F32
+    assert host.plan_fused(q, q, q, quantized=True, settings=s) == (K_FLASH_F32, True)
+
+
+# ------------------------------------------------------------------ GPU: Tensor / Session ---
+
+gpu = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hdev():
+    d = host.HipDevice(0)
+    yield d
+    d.close()
+
+
+def _fill(shape, seed):
+    return synth.fill(int(np.prod(shape)), seed).reshape(shape)
+
+
+@gpu
+def test_dispatch_handles_mask_and_causal(hdev):
+    """tests/flash_cuda_masks.rs:298-362: attention_with takes the fused kernel for causal + mask and GQA."""
+    n, d = 100, 64
+    sess = Session()
+    for (b, hq, hkv, causal, has_mask) in [(1, 2, 2, True, True), (2, 4, 2, False, False), (2, 4, 1, True, False)]:
+        q, k, v = _fill((b, hq, n, d), 3), _fill((b, hkv, n, d), 11), _fill((b, hkv, n, d), 19)
+        mask = (((np.arange(n * n) * 7) % 23).astype(np.float32) - 11.0).reshape(n, n) * np.float32(0.05) if has_mask else None
+        tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v))
+        tm = Tensor.from_slice(hdev, mask, mask.shape) if has_mask else None
+        before = host.selections(K_FLASH_F32)
+        out = tq.attention_with(tk, tv, tm, 0.0, causal, sess)
+        assert host.selections(K_FLASH_F32) == before + 1
+        assert out.shape == (b, hq, n, d) and out.dtype == FLOAT32
+        want = oracle.sdpa_f64(q, k, v, mask=mask, causal=causal)
+        err = float(np.abs(out.to_list() - want).max())
+        assert err < 2e-4                                   # tests/flash_cuda_masks.rs:289
+
+
+@gpu
+def test_bf16_gate_and_dispatch(hdev):
+    n, d = 197, 64
+    q, k, v = _fill((1, 6, n, d), 3), _fill((1, 6, n, d), 11), _fill((1, 6, n, d), 19)
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape, BFLOAT16) for a in (q, k, v))
+    sess = Session()
+    before = host.selections(K_FLASH_BF16)
+    out = tq.flash_attention_with(tk, tv, None, 0.0, False, sess)
+    assert host.selections(K_FLASH_BF16) == before + 1
+    assert out.dtype == BFLOAT16                             # bf16 tensors give a bf16 result (flash_attention.rs:514-521)
+    err = float(np.abs(out.to_list() - oracle.attn_bf16(q, k, v)).max())
+    assert err < 5e-3
+    # tensor cores off: the bf16 kernel is not selected and the caller is told to take SDPA
+    s = Settings.default()
+    s.tensor_cores = 0
+    with pytest.raises(host.HostError, match="general SDPA path"):
+        tq.flash_attention_with(tk, tv, None, 0.0, False, sess, s)
+
+
+@gpu
+def test_sage_attention_with_selects_the_quantised_kernel(hdev):
+    """tests/sage_int8.rs:152-250; with the reference's per-row quantiser (block 1, no smoothing)
+    and with this build's defaults (128/64 blocks, K smoothing)."""
+    b, h, n, d = 1, 2, 64, 64
+    q, k, v = _fill((b, h, n, d), 3), _fill((b, h, n, d), 11), _fill((b, h, n, d), 19)
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v))
+    sess = Session()
+    ref = Settings.default()
+    ref.sage_block_q = ref.sage_block_k = 1
+    ref.sage_smooth_k = 0
+    before = host.selections(K_SAGE)
+    out = tq.sage_attention_with(tk, tv, None, 0.0, False, sess, ref)
+    assert host.selections(K_SAGE) == before + 1
+    assert out.dtype == FLOAT32                              # the reference's Sage kernel stores f32
+    q8, sq = oracle.quant_blocks(q, 1)
+    k8, sk = oracle.quant_blocks(k, 1)
+    err = float(np.abs(out.to_list() - oracle.sage(q8, k8, sq, sk, v, 1, 1)).max())
+    assert err < 2e-3                                        # tests/sage_int8.rs:148
+    out2 = tq.sage_attention_with(tk, tv, None, 0.0, False, sess)
+    err2 = float(np.abs(out2.to_list() - oracle.sdpa_f64(q, k, v)).max())
+    assert err2 < 2e-2
+
+
+@gpu
+def test_fallback_is_reported_not_faked(hdev):
+    q = _fill((1, 2, 16, 32), 3)                             # head_dim 32: no fused kernel
+    t = Tensor.from_slice(hdev, q, q.shape)
+    sess = Session()
+    with pytest.raises(host.HostError, match="TGERR"):
+        t.attention_with(t, t, None, 0.0, False, sess)
+    q = _fill((1, 2, 16, 64), 3)
+    t = Tensor.from_slice(hdev, q, q.shape)
+    with pytest.raises(host.HostError, match="general SDPA path"):
+        t.attention(t, t)                                    # no session -> SDPA (tensor/mod.rs:2043-2054)
+    with pytest.raises(host.HostError, match="general SDPA path"):
+        t.attention_with(t, t, None, 0.5, False, sess)       # dropout -> SDPA
+
+
+@gpu
+def test_capture_and_replay(hdev):
+    """Session::capture_host + Jit replay (session.rs:138-146, jit.rs:186-195): the captured launch
+    re-runs on the same buffers and reproduces the result; the allocator serves repeats from its
+    free list."""
+    b, h, n, d = 1, 4, 300, 128
+    q, k, v = (synth.normal(700 + i, (b, h, n, d)) for i in range(3))
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape, BFLOAT16) for a in (q, k, v))
+    sess = Session()
+    sess.begin_capture()
+    out = tq.attention_with(tk, tv, None, 0.0, True, sess)
+    o2 = tq.sage_attention_with(tk, tv, None, 0.0, True, sess)
+    assert sess.end_capture() == 2
+    name, grid, vals = sess.step(0)
+    assert name == "ar_flash_bf16" and grid == [(n + 63) // 64, b * h, 1] and vals == [n, d, 1, 0, h, h]
+    assert sess.step(1)[0] == "ar_flash_sage"
+    first = out.to_list().copy()
+    first2 = o2.to_list().copy()
+    allocs = hdev.raw_allocs
+    sess.replay()
+    sess.replay()
+    assert hdev.raw_allocs == allocs                         # scratch came from the free list
+    assert np.array_equal(out.to_list(), first) and np.array_equal(o2.to_list(), first2)
+    err = float(np.abs(first - oracle.attn_bf16(q, k, v, causal=True)).max())
+    assert err < 1.6e-2
