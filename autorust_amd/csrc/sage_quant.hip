@@ -17,30 +17,6 @@ namespace {
 
 constexpr int MEAN_CHUNK = 64;  // tokens per partial sum
 
-__device__ __forceinline__ float ld_elem(const float *x, size_t i) { return x[i]; }
-__device__ __forceinline__ float ld_elem(const uint16_t *x, size_t i) { return __uint_as_float((uint32_t)x[i] << 16); }
-
-// part[bh][c][d] = k[64c][d] + k[64c+1][d] + ... in token order
-template <typename T>
-__global__ void k_mean_partial_kernel(const T *x, float *part, int N, int D, int nchunk)
-{
-    const int c = blockIdx.x, bh = blockIdx.y, d = threadIdx.x;
-    const int j0 = c * MEAN_CHUNK;
-    const int j1 = min(N, j0 + MEAN_CHUNK);
-    const size_t base = (size_t)bh * N * D + d;
-    float s = 0.f;
-    for (int j = j0; j < j1; ++j) s += ld_elem(x, base + (size_t)j * D);
-    part[((size_t)bh * nchunk + c) * D + d] = s;
-}
-
-// mean[bh][d] = (part[0] + part[1] + ...) / N in chunk order
-__global__ void k_mean_final_kernel(const float *part, float *mean, int N, int D, int nchunk)
-{
-    const int bh = blockIdx.x, d = threadIdx.x;
-    float tot = 0.f;
-    for (int c = 0; c < nchunk; ++c) tot += part[((size_t)bh * nchunk + c) * D + d];
-    mean[(size_t)bh * D + d] = tot / (float)N;
-}
 
 __device__ __forceinline__ void ld8(const float *x, size_t e, float v[8])
 {
@@ -56,11 +32,58 @@ __device__ __forceinline__ void ld8(const uint16_t *x, size_t e, float v[8])
     v[6] = __uint_as_float(a.w << 16); v[7] = __uint_as_float(a.w & 0xffff0000u);
 }
 
-// One workgroup per (block of `blk` tokens, head).
+// part[bh][c][d] = k[64c][d] + k[64c+1][d] + ... in token order.
+// One thread owns 8 adjacent channels of one 64-token chunk: D/8 threads read a whole row
+// (coalesced), 256/(D/8) chunks per workgroup.
+template <typename T>
+__global__ void __launch_bounds__(256) k_mean_partial_kernel(const T *x, float *part, int N, int D, int nchunk)
+{
+    const int gpr = D / 8;                       // 8-channel groups per row
+    const int cpb = 256 / gpr;                   // chunks per workgroup
+    const int c = blockIdx.x * cpb + threadIdx.x / gpr;
+    const int g = threadIdx.x % gpr, bh = blockIdx.y;
+    if (c >= nchunk) return;
+    const int j0 = c * MEAN_CHUNK;
+    const int j1 = min(N, j0 + MEAN_CHUNK);
+    const size_t base = (size_t)bh * N * D + g * 8;
+    float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = j0; j < j1; ++j) {
+        float v[8];
+        ld8(x, base + (size_t)j * D, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s[i] += v[i];
+    }
+    float *o = part + ((size_t)bh * nchunk + c) * D + g * 8;
+    *(float4 *)o = make_float4(s[0], s[1], s[2], s[3]);
+    *(float4 *)(o + 4) = make_float4(s[4], s[5], s[6], s[7]);
+}
+
+// mean[bh][d] = (part[0] + part[1] + ...) / N in chunk order (loads batched, adds in order)
+__global__ void k_mean_final_kernel(const float *part, float *mean, int N, int D, int nchunk)
+{
+    const int bh = blockIdx.x, d = threadIdx.x;
+    const float *p = part + (size_t)bh * nchunk * D + d;
+    float tot = 0.f;
+    int c = 0;
+    for (; c + 8 <= nchunk; c += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = p[(size_t)(c + i) * D];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) tot += v[i];
+    }
+    for (; c < nchunk; ++c) tot += p[(size_t)c * D];
+    mean[(size_t)bh * D + d] = tot / (float)N;
+}
+
+// One workgroup per (block of `blk` tokens, head).  Blocks of up to 256*64 elements are kept
+// in registers between the absmax pass and the quantising pass (one trip to memory); larger
+// ones are read twice.
 template <typename T, bool SMOOTH>
 __global__ void __launch_bounds__(256) quant_blocks_kernel(const T *x, int8_t *x8, float *scales, const float *mean,
                                                            int N, int D, int blk, int nblk)
 {
+    constexpr int KEEP = 8;  // 8-element groups a thread can hold
     __shared__ float red[4];
     const int bi = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
     const int r0 = bi * blk;
@@ -68,17 +91,35 @@ __global__ void __launch_bounds__(256) quant_blocks_kernel(const T *x, int8_t *x
     const size_t base = ((size_t)bh * N + r0) * D;
     const int nelem = (r1 - r0) * D;  // multiple of 8
     const float *mu = SMOOTH ? mean + (size_t)bh * D : nullptr;
+    const bool keep = nelem <= 256 * 8 * KEEP;
 
+    float held[KEEP][8];
     float mx = 0.f;
-    for (int e = tid * 8; e < nelem; e += 256 * 8) {
-        float v[8];
-        ld8(x, base + e, v);
-        const int d = e % D;
+    if (keep) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float xv = v[i];
-            if (SMOOTH) xv = xv - mu[d + i];
-            mx = fmaxf(mx, fabsf(xv));
+        for (int it = 0; it < KEEP; ++it) {
+            const int e = (it * 256 + tid) * 8;
+            if (e < nelem) {
+                ld8(x, base + e, held[it]);
+                const int d = e % D;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (SMOOTH) held[it][i] = held[it][i] - mu[d + i];
+                    mx = fmaxf(mx, fabsf(held[it][i]));
+                }
+            }
+        }
+    } else {
+        for (int e = tid * 8; e < nelem; e += 256 * 8) {
+            float v[8];
+            ld8(x, base + e, v);
+            const int d = e % D;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float xv = v[i];
+                if (SMOOTH) xv = xv - mu[d + i];
+                mx = fmaxf(mx, fabsf(xv));
+            }
         }
     }
 #pragma unroll
@@ -91,20 +132,33 @@ __global__ void __launch_bounds__(256) quant_blocks_kernel(const T *x, int8_t *x
     const float inv = 1.f / scale;
     if (tid == 0) scales[(size_t)bh * nblk + bi] = scale;
 
-    for (int e = tid * 8; e < nelem; e += 256 * 8) {
-        float v[8];
-        ld8(x, base + e, v);
-        const int d = e % D;
+    auto quant8 = [&](const float (&v)[8]) {
         uint32_t w[2] = {0u, 0u};
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float xv = v[i];
-            if (SMOOTH) xv = xv - mu[d + i];
-            int iv = (int)rintf(xv * inv);
+            int iv = (int)rintf(v[i] * inv);
             iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
             w[i >> 2] |= ((uint32_t)iv & 0xffu) << ((i & 3) * 8);
         }
-        *(uint2 *)(x8 + base + e) = make_uint2(w[0], w[1]);
+        return make_uint2(w[0], w[1]);
+    };
+    if (keep) {
+#pragma unroll
+        for (int it = 0; it < KEEP; ++it) {
+            const int e = (it * 256 + tid) * 8;
+            if (e < nelem) *(uint2 *)(x8 + base + e) = quant8(held[it]);
+        }
+    } else {
+        for (int e = tid * 8; e < nelem; e += 256 * 8) {
+            float v[8];
+            ld8(x, base + e, v);
+            const int d = e % D;
+            if (SMOOTH) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = v[i] - mu[d + i];
+            }
+            *(uint2 *)(x8 + base + e) = quant8(v);
+        }
     }
 }
 
@@ -147,12 +201,13 @@ extern "C" int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, fl
     t.kernel = ARHIP_K_SAGE_QUANT;
     if (int rc = t.begin()) return rc;
     if (smooth) {
-        const dim3 pgrid((unsigned)nchunk, (unsigned)(B * H));
+        const int cpb = 256 / (int)(D / 8);  // chunks per workgroup
+        const dim3 pgrid((unsigned)((nchunk + cpb - 1) / cpb), (unsigned)(B * H));
         if (dtype == ARHIP_F32)
-            hipLaunchKernelGGL(k_mean_partial_kernel<float>, pgrid, dim3((unsigned)D), 0, dev->stream,
+            hipLaunchKernelGGL(k_mean_partial_kernel<float>, pgrid, dim3(256), 0, dev->stream,
                                (const float *)x, (float *)workspace, (int)N, (int)D, nchunk);
         else
-            hipLaunchKernelGGL(k_mean_partial_kernel<uint16_t>, pgrid, dim3((unsigned)D), 0, dev->stream,
+            hipLaunchKernelGGL(k_mean_partial_kernel<uint16_t>, pgrid, dim3(256), 0, dev->stream,
                                (const uint16_t *)x, (float *)workspace, (int)N, (int)D, nchunk);
         hipLaunchKernelGGL(k_mean_final_kernel, dim3((unsigned)(B * H)), dim3((unsigned)D), 0, dev->stream,
                            (const float *)workspace, mean, (int)N, (int)D, nchunk);
