@@ -94,17 +94,23 @@ extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, 
         fp.q = (const float *)q; fp.k = (const float *)k; fp.v = (const float *)v; fp.o = (float *)o;
         fp.mask = mask; fp.kv_len = kv_len;
         fp.Hq = (int)Hq; fp.Hkv = (int)Hkv; fp.N = (int)N;
-        fp.nq = (int)((N + FLASH_F32_BQ - 1) / FLASH_F32_BQ);
+        // 4 waves (128 queries) per workgroup when that still fills the chip, else 1 wave
+        const int nw = (B * Hq * ((N + 127) / 128) >= 2 * (int64_t)dev->cus) ? 4 : 1;
+        fp.nq = (int)((N + nw * 32 - 1) / (nw * 32));
         fp.scale = scale;
         if (int rc = t.begin()) return rc;
-        const dim3 grid((unsigned)(fp.nq * B * Hq)), block(FLASH_F32_THREADS);
+        const dim3 grid((unsigned)(fp.nq * B * Hq)), block((unsigned)(nw * 64));
+#define F32_LAUNCH(DD, NWW)                                                                           \
+    do {                                                                                              \
+        if (causal) hipLaunchKernelGGL((flash_f32_kernel<DD, NWW, true>), grid, block, 0, dev->stream, fp);  \
+        else hipLaunchKernelGGL((flash_f32_kernel<DD, NWW, false>), grid, block, 0, dev->stream, fp); \
+    } while (0)
         if (D == 64) {
-            if (causal) hipLaunchKernelGGL((flash_f32_kernel<64, true>), grid, block, 0, dev->stream, fp);
-            else hipLaunchKernelGGL((flash_f32_kernel<64, false>), grid, block, 0, dev->stream, fp);
+            if (nw == 4) F32_LAUNCH(64, 4); else F32_LAUNCH(64, 1);
         } else {
-            if (causal) hipLaunchKernelGGL((flash_f32_kernel<128, true>), grid, block, 0, dev->stream, fp);
-            else hipLaunchKernelGGL((flash_f32_kernel<128, false>), grid, block, 0, dev->stream, fp);
+            if (nw == 4) F32_LAUNCH(128, 4); else F32_LAUNCH(128, 1);
         }
+#undef F32_LAUNCH
         arhip_note_selected(ARHIP_K_FLASH_F32);
         return t.end();
     }

@@ -1,10 +1,19 @@
-// fp32 exact-mode FlashAttention forward (no matrix cores, no reduced precision).
+// fp32 exact-mode FlashAttention forward: no reduced precision anywhere.
 //
-// Same schedule and arithmetic as the reference's scalar kernel
-// (src/runtime/cuda_flash.rs:53-141): one thread per query row, BQ = 64 rows per
-// workgroup (one wave64), BK = 32 keys per step broadcast from LDS, fp32 FMA dot
-// products in channel order, `expf`, finite sentinel -1e30 for masked keys,
-// acc * (l > 0 ? 1/l : 0) at the end.  head_dim and scale are parameters here.
+// Semantics of the reference's scalar kernel (src/runtime/cuda_flash.rs:53-141): fp32 products
+// and sums, `expf`, finite sentinel -1e30 for masked keys, acc * (l > 0 ? 1/l : 0) at the end;
+// head_dim and scale are parameters here (the reference hard-codes 64 and 0.125).
+//
+// The two contractions run on the fp32 matrix instruction v_mfma_f32_32x32x2_f32 (fp32 in,
+// fp32 accumulate) with the same decomposition as the bf16 kernel: a wave owns 32 queries and
+// computes S^T = K . Q^T, so each lane owns one query (column lane%32) and 16 of a block's 32
+// keys; O^T = V^T . P^T keeps one query per lane, and the online-softmax state is per lane.
+//   A[32 x 2] . B[2 x 32]: lane holds A[lane%32][lane/32] and B[lane/32][lane%32]
+//   result C[32 x 32]: lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4
+// The order of the channels inside Q.K^T is free as long as Q and K agree, so MFMA step s of
+// lane half h multiplies channel h*D/2 + s: every lane reads its K row as D/2 consecutive
+// floats.  For P.V the step (g, t) multiplies key 8g + 4h + t, which is exactly the key the
+// S^T result left in register 4g + t of that lane.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -12,9 +21,9 @@
 
 namespace arhip {
 
-constexpr int FLASH_F32_BQ = 64;
-constexpr int FLASH_F32_BK = 32;
-constexpr int FLASH_F32_THREADS = 64;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+constexpr int F32_BK = 32;  // keys per tile
 
 struct FlashF32Params {
     const float *q, *k, *v;
@@ -25,24 +34,32 @@ struct FlashF32Params {
     float scale;
 };
 
-template <int D, bool CAUSAL>
-__global__ void __launch_bounds__(FLASH_F32_THREADS) flash_f32_kernel(const FlashF32Params p)
+template <int D, int NW, bool CAUSAL>
+__global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params p)
 {
-    constexpr int BQ = FLASH_F32_BQ, BKK = FLASH_F32_BK;
-    __shared__ __attribute__((aligned(16))) float ks[BKK][D];
-    __shared__ __attribute__((aligned(16))) float vs[BKK][D];
+    constexpr int T = NW * 64;
+    constexpr int BQ = NW * 32;
+    constexpr int HALF = D / 2;          // channels per lane half
+    constexpr int KROW = D + 4;          // padded K row (floats): conflict-free 128-bit row reads
+    constexpr int DB = D / 32;
+    constexpr int CHUNKS = F32_BK * D / 4;             // float4 chunks per K (or V) tile
+    constexpr int PER_THREAD = (CHUNKS + T - 1) / T;
+    static_assert(CHUNKS % T == 0, "tile staging must divide evenly");
 
-    const int t = threadIdx.x;
+    __shared__ __attribute__((aligned(16))) float ks[F32_BK * KROW];
+    __shared__ __attribute__((aligned(16))) float vs[F32_BK * D];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i32 = lane & 31, h = lane >> 5;
     const int bh = blockIdx.x / p.nq;
-    const int qblk = (blockIdx.x - bh * p.nq) * BQ;
-    const int row = qblk + t;
-    const int b = bh / p.Hq;
-    const int head = bh - b * p.Hq;
+    int qt = blockIdx.x - bh * p.nq;
+    if (CAUSAL) qt = p.nq - 1 - qt;
+    const int b = bh / p.Hq, head = bh - b * p.Hq;
     const int kv_bh = b * p.Hkv + head / (p.Hq / p.Hkv);
     const int N = p.N;
-    const float *qp = p.q + ((size_t)bh * N + (row < N ? row : 0)) * D;
-    const float *kp = p.k + (size_t)kv_bh * N * D;
-    const float *vp = p.v + (size_t)kv_bh * N * D;
+    const int qblk = qt * BQ;
+    const int wq0 = qblk + wave * 32;
+    const int q_row = wq0 + i32;
 
     int kvl = N;
     if (p.kv_len) {
@@ -51,71 +68,115 @@ __global__ void __launch_bounds__(FLASH_F32_THREADS) flash_f32_kernel(const Flas
     }
     int kend = kvl;
     if (CAUSAL) kend = min(kend, min(N, qblk + BQ));
+    const int ntiles = (kend + F32_BK - 1) / F32_BK;
+    const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / F32_BK + 1) : ntiles;
 
-    float qr[D];
+    const float *kp = p.k + (size_t)kv_bh * N * D;
+    const float *vp = p.v + (size_t)kv_bh * N * D;
+
+    // Q: this lane's half of its query row (rows past N read row N-1; never stored)
+    float qr[HALF];
+    {
+        const float *qp = p.q + ((size_t)bh * N + min(q_row, N - 1)) * D + h * HALF;
 #pragma unroll
-    for (int d = 0; d < D; d += 4) {
-        float4 x = *(const float4 *)(qp + d);
-        if (row >= N) x = make_float4(0.f, 0.f, 0.f, 0.f);
-        qr[d] = x.x; qr[d + 1] = x.y; qr[d + 2] = x.z; qr[d + 3] = x.w;
+        for (int s = 0; s < HALF; s += 4) {
+            const float4 x = *(const float4 *)(qp + s);
+            qr[s] = x.x; qr[s + 1] = x.y; qr[s + 2] = x.z; qr[s + 3] = x.w;
+        }
     }
-    float acc[D];
-#pragma unroll
-    for (int d = 0; d < D; ++d) acc[d] = 0.f;
-    float m = -1e30f, l = 0.f;
 
-    for (int k0 = 0; k0 < kend; k0 += BKK) {
-        __syncthreads();
-        for (int i = t; i < BKK * D / 4; i += FLASH_F32_THREADS) {
-            const int r = i / (D / 4), c = (i % (D / 4)) * 4;
-            const int gr = k0 + r;
+    f32x16_t oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+    float m_run = -1e30f, l_run = 0.f;
+
+    for (int it = 0; it < ntiles; ++it) {
+        const int k0 = it * F32_BK;
+        __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int c = tid + j * T;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            const int gr = k0 + row;
             float4 kx = make_float4(0.f, 0.f, 0.f, 0.f), vx = kx;
             if (gr < kend) {
-                kx = *(const float4 *)(kp + (size_t)gr * D + c);
-                vx = *(const float4 *)(vp + (size_t)gr * D + c);
+                kx = *(const float4 *)(kp + (size_t)gr * D + col);
+                vx = *(const float4 *)(vp + (size_t)gr * D + col);
             }
-            *(float4 *)&ks[r][c] = kx;
-            *(float4 *)&vs[r][c] = vx;
+            *(float4 *)&ks[row * KROW + col] = kx;
+            *(float4 *)&vs[row * D + col] = vx;
         }
         __syncthreads();
+        if (it >= my_tiles) continue;  // under the causal mask this wave is done (it still helps staging)
 
-        float s[BKK];
-        float mnew = m;
+        // ---- S^T = K . Q^T ----
+        f32x16_t s;
 #pragma unroll
-        for (int j = 0; j < BKK; ++j) {
-            const int gj = k0 + j;
-            float dot = 0.f;
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+        const float *krow = &ks[i32 * KROW + h * HALF];
 #pragma unroll
-            for (int d = 0; d < D; ++d) dot = fmaf(qr[d], ks[j][d], dot);
-            dot *= p.scale;
-            if (p.mask != nullptr && row < N && gj < N) dot += p.mask[(size_t)row * N + gj];
-            if (gj >= kend || (CAUSAL && gj > row)) dot = -1e30f;
-            s[j] = dot;
-            mnew = fmaxf(mnew, dot);
+        for (int st = 0; st < HALF; st += 4) {
+            const float4 kx = *(const float4 *)(krow + st);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx.x, qr[st + 0], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx.y, qr[st + 1], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx.z, qr[st + 2], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx.w, qr[st + 3], s, 0, 0, 0);
         }
-        const float alpha = expf(m - mnew);
-        float sum = 0.f;
+
+        // ---- scale, masks, online softmax (natural exponent, like the reference) ----
+        float x[16];
+        float mx = -1e30f;
 #pragma unroll
-        for (int j = 0; j < BKK; ++j) {
-            s[j] = expf(s[j] - mnew);
-            sum += s[j];
+        for (int r = 0; r < 16; ++r) {
+            const int key = k0 + 8 * (r >> 2) + 4 * h + (r & 3);
+            float xv = s[r] * p.scale;
+            if (p.mask != nullptr && key < N && q_row < N) xv += p.mask[(size_t)q_row * N + key];
+            if (key >= kend || (CAUSAL && key > q_row)) xv = -1e30f;
+            x[r] = xv;
+            mx = fmaxf(mx, xv);
         }
-        l = l * alpha + sum;
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = expf(m_run - m_new);
+        m_run = m_new;
+        float rs = 0.f;
 #pragma unroll
-        for (int d = 0; d < D; ++d) acc[d] *= alpha;
+        for (int r = 0; r < 16; ++r) {
+            x[r] = expf(x[r] - m_new);
+            rs += x[r];
+        }
+        l_run = l_run * alpha + rs;
+        if (__any(alpha != 1.0f)) {
 #pragma unroll
-        for (int j = 0; j < BKK; ++j)
+            for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int d = 0; d < D; ++d) acc[d] = fmaf(s[j], vs[j][d], acc[d]);
-        m = mnew;
+                for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+        }
+
+        // ---- O^T += V^T . P^T : step (g, t) uses key 8g + 4h + t ----
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float *vrow = &vs[(8 * (r >> 2) + 4 * h + (r & 3)) * D + i32];
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[db * 32], x[r], oacc[db], 0, 0, 0);
+        }
     }
 
-    if (row < N) {
-        const float inv = (l > 0.f) ? 1.f / l : 0.f;
-        float *op = p.o + ((size_t)bh * N + row) * D;
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+    if (q_row < N) {
+        float *op = p.o + ((size_t)bh * N + q_row) * D;
 #pragma unroll
-        for (int d = 0; d < D; d += 4)
-            *(float4 *)(op + d) = make_float4(acc[d] * inv, acc[d + 1] * inv, acc[d + 2] * inv, acc[d + 3] * inv);
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = db * 32 + 8 * g + 4 * h;
+                *(float4 *)(op + d) = make_float4(oacc[db][4 * g] * inv, oacc[db][4 * g + 1] * inv,
+                                                  oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
+            }
     }
 }
 
