@@ -335,14 +335,9 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
         const unsigned char *vl = kl + K_TILE;
         float f_tile = 1.f;
         if (MODE == MODE_I8 && !PER_KEY) f_tile = p.sk[(size_t)kv_bh * nkb + (it >> p.bk_tile_shift)];
-        load_kf(kl, 0);
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-            // ---- P1 ----
-            load_vf(vl, blk);
-            acc_t s = mfma_qk();
-            ARHIP_FENCE();
-            // ---- P2 ----
+        // online softmax of one 32-key block: raw accumulators in, probabilities (bf16, B-operand
+        // layout) out; updates the running reference / sum and, rarely, rescales the accumulators
+        auto softmax_block = [&](int blk, const acc_t &s, uint4 (&pb)[2]) __attribute__((always_inline)) {
             if (DBG) {
                 if (bh == p.dbg_bh && (wq0 >> 5) == p.dbg_qt && it == p.dbg_kt) {
 #pragma unroll
@@ -405,8 +400,6 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
             rs0 += (x[4] + x[5]) + (x[6] + x[7]);
             rs1 += (x[12] + x[13]) + (x[14] + x[15]);
             l_run += rs0 + rs1;
-            // P (bf16) as the B operand, 2 steps of 16 keys
-            uint4 pb[2];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
                 pb[ks].x = pack_bf16x2(x[ks * 8 + 0], x[ks * 8 + 1]);
@@ -414,6 +407,18 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
                 pb[ks].z = pack_bf16x2(x[ks * 8 + 4], x[ks * 8 + 5]);
                 pb[ks].w = pack_bf16x2(x[ks * 8 + 6], x[ks * 8 + 7]);
             }
+        };
+
+        load_kf(kl, 0);
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            uint4 pb[2];
+            // ---- P1 ----
+            load_vf(vl, blk);
+            acc_t s = mfma_qk();
+            ARHIP_FENCE();
+            // ---- P2 ----
+            softmax_block(blk, s, pb);
             ARHIP_FENCE();
             // ---- P3 ----
             if (blk == 0) load_kf(kl, 1);
