@@ -121,10 +121,13 @@ __device__ __forceinline__ uint2 lds_read_tr16(const unsigned char *p)
 // s_waitcnt vmcnt(0): all outstanding global loads of this wave have landed.
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG>
-__global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(const AttnParams p)
+template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false>
+__global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd_kernel(const AttnParams p)
 {
-    constexpr int NSTAGE = 2;
+    // SMALL: the whole sequence (at most 4 tiles) is brought into LDS up front, all global loads
+    // in flight at once and a single barrier: short sequences are latency bound, not math bound.
+    constexpr int NSTAGE = SMALL ? 4 : 2;
+    constexpr int NSLOT = SMALL ? 4 : 1;  // register sets for tiles in flight
     constexpr int T = NW * 64;
     constexpr int BQ = NW * 32;
     constexpr int QK_BYTES = (MODE == MODE_I8) ? 1 : 2;        // bytes per q/k element
@@ -196,12 +199,12 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
     }
 
     // ---- staging registers (tile i+1 in flight while tile i is computed) ----
-    uint4 kst[K_PER_THREAD];
-    uint4 vst[V_PER_THREAD];
+    uint4 kst[NSLOT][K_PER_THREAD];
+    uint4 vst[NSLOT][V_PER_THREAD];
     float sst = 0.f;
     const int nkb = (MODE == MODE_I8) ? (N + p.bk - 1) / p.bk : 0;
 
-    auto load_tile = [&](int k0) __attribute__((always_inline)) {
+    auto load_tile = [&](int k0, int slot = 0) __attribute__((always_inline)) {
         const bool full = k0 + BK <= kend;  // uniform: the common case has no bounds logic
 #pragma unroll
         for (int j = 0; j < K_PER_THREAD; ++j) {
@@ -210,11 +213,11 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
                 const int row = c / K_CPR, col = c % K_CPR;
                 const int gr = k0 + row;
                 if (full) {
-                    kst[j] = *(const uint4 *)(kbase + (size_t)gr * (D * QK_BYTES) + col * 16);
+                    kst[slot][j] = *(const uint4 *)(kbase + (size_t)gr * (D * QK_BYTES) + col * 16);
                 } else {
                     uint4 val = *(const uint4 *)(kbase + (size_t)min(gr, kend - 1) * (D * QK_BYTES) + col * 16);
                     if (gr >= kend) val = make_uint4(0, 0, 0, 0);
-                    kst[j] = val;
+                    kst[slot][j] = val;
                 }
             }
         }
@@ -225,18 +228,18 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
                 const int row = c / V_CPR, col = c % V_CPR;
                 const int gr = k0 + row;
                 if (full) {
-                    vst[j] = *(const uint4 *)(vbase + (size_t)gr * D + col * 8);
+                    vst[slot][j] = *(const uint4 *)(vbase + (size_t)gr * D + col * 8);
                 } else {
                     uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * D + col * 8);
                     if (gr >= kend) val = make_uint4(0, 0, 0, 0);
-                    vst[j] = val;
+                    vst[slot][j] = val;
                 }
             }
         }
         if (PER_KEY && tid < BK) sst = p.sk[(size_t)kv_bh * nkb + min(k0 + tid, N - 1) / p.bk];
     };
 
-    auto store_tile = [&](int stage) __attribute__((always_inline)) {
+    auto store_tile = [&](int stage, int slot = 0) __attribute__((always_inline)) {
         unsigned char *kl = lds + stage * STAGE;
         unsigned char *vl = kl + K_TILE;
 #pragma unroll
@@ -244,7 +247,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
             const int c = tid + j * T;
             if (K_CHUNKS >= T || c < K_CHUNKS) {
                 const int row = c / K_CPR, col = c % K_CPR;
-                *(uint4 *)(kl + row * KROW + col * 16) = kst[j];
+                *(uint4 *)(kl + row * KROW + col * 16) = kst[slot][j];
             }
         }
 #pragma unroll
@@ -252,7 +255,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
             const int c = tid + j * T;
             if (V_CHUNKS >= T || c < V_CHUNKS) {
                 const int row = c / V_CPR, col = c % V_CPR;
-                *(uint4 *)(vl + row * VROW + col * 16) = vst[j];
+                *(uint4 *)(vl + row * VROW + col * 16) = vst[slot][j];
             }
         }
         if (PER_KEY && tid < BK) *(float *)(vl + V_TILE + tid * 4) = sst;
@@ -427,6 +430,22 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
         }
     };
 
+    if constexpr (SMALL) {
+        static_assert(!PER_KEY, "the preloading variant has no per-key scales");
+#pragma unroll
+        for (int t = 0; t < NSLOT; ++t)
+            if (t < ntiles) load_tile(t * BK, t);
+#pragma unroll
+        for (int t = 0; t < NSLOT; ++t)
+            if (t < ntiles) store_tile(t, t);
+        __syncthreads();
+        for (int it = 0; it < my_tiles; ++it) {
+            const int k0 = it * BK;
+            const bool masked = (k0 + BK > kend) || (CAUSAL && (k0 + BK - 1 > wq0));
+            if (HAS_MASK || masked) tile_body(std::true_type{}, it);
+            else tile_body(std::false_type{}, it);
+        }
+    } else {
     if (ntiles > 0) {
         load_tile(0);
         store_tile(0);
@@ -458,6 +477,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(co
             if (it + 1 < ntiles) store_tile((it + 1) % NSTAGE);
             __syncthreads();
         }
+    }
     }
 
     // ---- normalise and store: acc * (l > 0 ? 1/l : 0), cuda_flash_bf16.rs:414-426 ----

@@ -126,7 +126,19 @@ extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, 
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     if (int rc = t.begin()) return rc;
-    if (D == 64) {
+    if (N <= 256 && !hm && B * Hq * ((N + 127) / 128) <= 4 * (int64_t)dev->cus && !getenv("ARHIP_ATTN_WAVES")) {
+        // short sequence: bring all of K/V into LDS at once (128 queries per workgroup)
+        p.nq = (int)((N + 127) / 128);
+        p.total = (int)(p.nq * B * Hq);
+        const dim3 grid((unsigned)p.total), block(256);
+        if (D == 64) {
+            if (c) hipLaunchKernelGGL((attn_fwd_kernel<64, 4, true, false, MODE_BF16, false, false, false, true>), grid, block, 0, dev->stream, p);
+            else hipLaunchKernelGGL((attn_fwd_kernel<64, 4, false, false, MODE_BF16, false, false, false, true>), grid, block, 0, dev->stream, p);
+        } else {
+            if (c) hipLaunchKernelGGL((attn_fwd_kernel<128, 4, true, false, MODE_BF16, false, false, false, true>), grid, block, 0, dev->stream, p);
+            else hipLaunchKernelGGL((attn_fwd_kernel<128, 4, false, false, MODE_BF16, false, false, false, true>), grid, block, 0, dev->stream, p);
+        }
+    } else if (D == 64) {
         if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
         else if (nw == 4) launch_attn<64, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
         else launch_attn<64, 8, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm);
