@@ -74,6 +74,7 @@ struct AttnParams {
     int bk_tile_shift;  // log2(bk / 64) when the K scales are tile-uniform
     int nq;        // query tiles per head
     int total;     // workgroups
+    int lpt;       // causal: order the whole grid longest-tile-first (small grids)
     float scale;
 };
 
@@ -161,10 +162,20 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
     // (8 of them, each with its own L2); give every XCD a contiguous range of
     // heads so that the query tiles sharing one head's K/V hit the same L2.
     int wg = blockIdx.x;
-    if ((p.total & 7) == 0) wg = (wg & 7) * (p.total >> 3) + (wg >> 3);
-    const int bh = wg / p.nq;
-    int qt = wg - bh * p.nq;
-    if (CAUSAL) qt = p.nq - 1 - qt;  // longest tiles first
+    int bh, qt;
+    if (CAUSAL && p.lpt) {
+        // Few workgroups per CU and very unequal ones (causal): longest-first over the whole
+        // grid, so that no long tile is left for the end.  K/V of all heads then share the L2s
+        // and the chip-wide cache instead of one XCD's L2.
+        const int nbh = p.total / p.nq;
+        qt = p.nq - 1 - wg / nbh;
+        bh = wg % nbh;
+    } else {
+        if ((p.total & 7) == 0) wg = (wg & 7) * (p.total >> 3) + (wg >> 3);
+        bh = wg / p.nq;
+        qt = wg - bh * p.nq;
+        if (CAUSAL) qt = p.nq - 1 - qt;  // longest tiles first within a head
+    }
     const int b = bh / p.Hq;
     const int head = bh - b * p.Hq;
     const int kvh = head / (p.Hq / p.Hkv);

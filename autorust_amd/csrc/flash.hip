@@ -125,6 +125,7 @@ extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, 
     const int nw = pick_waves(dev, B * Hq, N, D, hm);
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
+    p.lpt = p.total <= 16 * dev->cus;  // few workgroups per CU: balance them globally
     if (int rc = t.begin()) return rc;
     if (N <= 256 && !hm && B * Hq * ((N + 127) / 128) <= 4 * (int64_t)dev->cus && !getenv("ARHIP_ATTN_WAVES")) {
         // short sequence: bring all of K/V into LDS at once (128 queries per workgroup)
@@ -185,6 +186,7 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
     if (nw == 1) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
+    p.lpt = p.total <= 16 * dev->cus;
     if (dbg) {
         p.dbg = dbg_logits;
         p.dbg_bh = dbg_sel[0]; p.dbg_qt = dbg_sel[1]; p.dbg_kt = dbg_sel[2];
