@@ -31,6 +31,10 @@ PEAK_BF16 = 2500.0   # TFLOP/s, MI355X dense bf16 MFMA
 PEAK_INT8 = 5000.0   # TOP/s, MI355X dense int8 MFMA
 PEAK_HBM = 8000.0    # GB/s, MI355X HBM3E
 
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# and calibrated against a 1 GiB copy kernel (profiles/attn_fwd_sage_s8192_hbm_traffic.md).
+MEASURED_TRAFFIC = {"sage_int8_b4_h32_s8192_d128": 805.5e6}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -91,7 +95,7 @@ class SageWorkload:
         t_min = half / (PEAK_INT8 * 1e12) + half / (PEAK_BF16 * 1e12)
         ach = self.ops / secs / 1e12
         return {"bound": "mfma", "achieved": ach, "peak": PEAK_INT8, "unit": "TFLOP/s", "frac": ach / PEAK_INT8,
-                "traffic": None, "kernel": "attn_fwd_kernel<int8>", "launch_ms": secs * 1e3,
+                "traffic": MEASURED_TRAFFIC.get(self.name), "kernel": "attn_fwd_kernel<int8>", "launch_ms": secs * 1e3,
                 "ops_per_launch": self.ops, "peak_note": "dense int8 MFMA; half of the ops are bf16 (P.V)",
                 "frac_of_mixed_int8_bf16_bound": t_min / secs}
 
@@ -203,6 +207,8 @@ def build_workload(dev, name):
         return SageWorkload(dev, 1, 64, 32768, 128, True, 5.0, 0.01, cfg=5)
     if name == "vit":
         return FlashWorkload(dev, 8, 12, 197, 64, False, BF16, cfg=2)
+    if name == "flash_long":
+        return FlashWorkload(dev, 4, 32, 8192, 128, False, BF16, cfg=6)
     if name == "decoder":
         return FlashWorkload(dev, 4, 32, 2048, 128, True, BF16, cfg=3, kv_lens=True)
     if name == "vit_f32":
@@ -216,7 +222,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="sage",
-                    choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32"])
+                    choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32", "flash_long"])
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="one step of the workload plus one plain 1 GiB copy kernel and nothing else: "
@@ -246,14 +252,14 @@ def main():
     log(json.dumps(res))
     cpu = None
     if not args.no_cpu:
-        heads = {"sage": 2, "sage_causal_long": 1, "decoder": 16, "vit": 96, "vit_f32": 12}[args.workload]
+        heads = {"sage": 2, "sage_causal_long": 1, "decoder": 16, "vit": 96, "vit_f32": 12, "flash_long": 2}[args.workload]
         cpu = cpu_baseline(w, heads)
         log(json.dumps(cpu))
     w.free()
 
     secondary = []
     if not args.no_secondary:
-        for name in ("vit", "decoder", "vit_f32", "sage", "sage_causal_long"):
+        for name in ("vit", "decoder", "flash_long", "vit_f32", "sage", "sage_causal_long"):
             if name == args.workload:
                 continue
             sw = build_workload(dev, name)
