@@ -56,7 +56,8 @@ constexpr int MODE_I8 = 1;    // q, k int8 with block scales
 constexpr int BK = 64;        // keys per tile
 constexpr float NEG_SENTINEL = -1e30f;  // src/runtime/cuda_flash_bf16.rs:106 (AR_NEG)
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr float LAZY_TAU = 8.0f;  // log2 units the running maximum may outgrow the exponent reference
+constexpr float LAZY_TAU = 8.0f;     // log2 units the running maximum may outgrow the exponent reference
+constexpr float LAZY_LIMIT = 256.0f;  // = 2^LAZY_TAU: the largest probability the lazy reference lets through
 
 struct AttnParams {
     const void *q;
@@ -342,7 +343,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
 
     // GENERIC handles everything (additive mask, causal and key-length masking, per-key
     // scales); the other instantiation is for tiles in which no key is masked for this wave.
-    auto tile_body = [&](auto generic_c, int it) __attribute__((always_inline)) {
+    auto tile_body = [&](auto generic_c, int it, auto &&mid_tile) __attribute__((always_inline)) {
         constexpr bool GENERIC = decltype(generic_c)::value;
         const int k0 = it * BK;
         const unsigned char *kl = lds + (it % NSTAGE) * STAGE;
@@ -358,17 +359,48 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
                     for (int r = 0; r < 16; ++r) p.dbg[i32 * 64 + blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] = (int32_t)s[r];
                 }
             }
-            // The exponent reference m_run is only moved when some query's maximum outgrows it
-            // by more than LAZY_TAU (then the accumulators are rescaled); otherwise it stays put and
-            // the probabilities of this block are at most 2^LAZY_TAU.  Softmax does not depend on
-            // the reference, so this only saves the rescale almost every time.
+            // The exponent reference m_run is lazy: it only moves when a row maximum outgrows it by
+            // 2^LAZY_TAU (then the accumulators are rescaled).  Softmax does not depend on the
+            // reference, so the result is the same function with almost no rescaling.
             float x[16];
-            float c = c_scale;  // fast path: scale folded into the exponent
-            if (!GENERIC) {
-                // s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322
-                if (MODE == MODE_I8) c = ((sq_lane * f_tile) * p.scale) * LOG2E;
+            float rs;
+            auto move_reference = [&](float mx) __attribute__((always_inline)) {
+                const float m_new = fmaxf(m_run, mx);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                l_run *= alpha;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) x[r] = (float)s[r];
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+            };
+            auto row_sum = [&]() __attribute__((always_inline)) {
+                // over the unrounded probabilities (src/runtime/cuda_flash_bf16.rs:365-377)
+                float rs0 = (x[0] + x[1]) + (x[2] + x[3]), rs1 = (x[8] + x[9]) + (x[10] + x[11]);
+                rs0 += (x[4] + x[5]) + (x[6] + x[7]);
+                rs1 += (x[12] + x[13]) + (x[14] + x[15]);
+                return rs0 + rs1;
+            };
+            if (!GENERIC) {
+                // Unmasked block: exponentiate against the current reference straight away, the scale
+                // folded into the exponent: s = (float)acc * ((sq * sk) * scale),
+                // src/runtime/cuda_flash_sage.rs:315-322.  The row sum bounds the largest probability
+                // (max <= sum <= 16 max), so only a sum that is too large (or not finite: the very first
+                // block, or a jump of the maximum) sends the wave to the exact path below.
+                const float c = (MODE == MODE_I8) ? ((sq_lane * f_tile) * p.scale) * LOG2E : c_scale;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[r], c, -m_run));
+                rs = row_sum();
+                if (__any(!(rs <= 16.0f * LAZY_LIMIT))) {
+                    float mx = max3((float)s[0], (float)s[1], (float)s[2]);
+#pragma unroll
+                    for (int r = 3; r < 15; r += 2) mx = max3(mx, (float)s[r], (float)s[r + 1]);
+                    mx = xhalf_max(fmaxf(mx, (float)s[15])) * c;
+                    move_reference(mx);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[r], c, -m_run));
+                    rs = row_sum();
+                }
             } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
@@ -386,34 +418,16 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
                     if (key >= kend || (CAUSAL && key > q_row)) xv = NEG_SENTINEL;
                     x[r] = xv;
                 }
-            }
-            float mx = max3(x[0], x[1], x[2]);
+                float mx = max3(x[0], x[1], x[2]);
 #pragma unroll
-            for (int r = 3; r < 15; r += 2) mx = max3(mx, x[r], x[r + 1]);
-            mx = xhalf_max(fmaxf(mx, x[15]));
-            if (!GENERIC) mx *= c;
-            if (__any(mx > m_run + LAZY_TAU)) {
-                const float m_new = fmaxf(m_run, mx);
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                m_run = m_new;
-                l_run *= alpha;
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-            }
-            if (!GENERIC) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c, -m_run));
-            } else {
+                for (int r = 3; r < 15; r += 2) mx = max3(mx, x[r], x[r + 1]);
+                mx = xhalf_max(fmaxf(mx, x[15]));
+                if (__any(mx > m_run + LAZY_TAU)) move_reference(mx);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_run);
+                rs = row_sum();
             }
-            // row sum over the unrounded probabilities (src/runtime/cuda_flash_bf16.rs:365-377)
-            float rs0 = (x[0] + x[1]) + (x[2] + x[3]), rs1 = (x[8] + x[9]) + (x[10] + x[11]);
-            rs0 += (x[4] + x[5]) + (x[6] + x[7]);
-            rs1 += (x[12] + x[13]) + (x[14] + x[15]);
-            l_run += rs0 + rs1;
+            l_run += rs;
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
                 pb[ks].x = pack_bf16x2(x[ks * 8 + 0], x[ks * 8 + 1]);
@@ -438,6 +452,10 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
             if (blk == 0) load_kf(kl, 1);
             mfma_pv(pb);
             ARHIP_FENCE();
+            if (blk == 0) {
+                mid_tile();  // staging of the tiles ahead, issued while the matrix pipe has work queued
+                ARHIP_FENCE();
+            }
         }
     };
 
@@ -450,42 +468,54 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
         for (int t = 0; t < NSLOT; ++t)
             if (t < ntiles) store_tile(t, t);
         __syncthreads();
+        auto nothing = [] {};
         for (int it = 0; it < my_tiles; ++it) {
             const int k0 = it * BK;
             const bool masked = (k0 + BK > kend) || (CAUSAL && (k0 + BK - 1 > wq0));
-            if (HAS_MASK || masked) tile_body(std::true_type{}, it);
-            else tile_body(std::false_type{}, it);
+            if (HAS_MASK || masked) tile_body(std::true_type{}, it, nothing);
+            else tile_body(std::false_type{}, it, nothing);
         }
     } else {
+    // Staging runs two tiles ahead of the math with one set of registers: in the middle of the
+    // iteration that computes tile i, tile i+1 (loaded during iteration i-1) goes from registers
+    // to the LDS stage that tile i-1 vacated at the last barrier, and the loads of tile i+2 are
+    // issued; they have a whole iteration to land before anybody waits for them.
     if (ntiles > 0) {
         load_tile(0);
         store_tile(0);
     }
-    wait_vmem();  // Q and the first tile have landed: nothing is pending at loop entry
+    if (ntiles > 1) load_tile(BK);
     __syncthreads();
+    auto nothing = [] {};
 
     if constexpr (!CAUSAL && !HAS_MASK && !PER_KEY) {
         // only the last tile can hold masked keys: keep it out of the loop
         const int nfull = kend / BK;
 #pragma clang loop unroll(disable)
         for (int it = 0; it < nfull; ++it) {
-            if (it + 1 < ntiles) load_tile((it + 1) * BK);
-            tile_body(std::false_type{}, it);
-            if (it + 1 < ntiles) store_tile((it + 1) % NSTAGE);
+            auto stage_ahead = [&]() __attribute__((always_inline)) {
+                if (it + 1 < ntiles) store_tile((it + 1) % NSTAGE);
+                if (it + 2 < ntiles) load_tile((it + 2) * BK);
+            };
+            tile_body(std::false_type{}, it, stage_ahead);
             __syncthreads();
         }
-        if (nfull < ntiles) tile_body(std::true_type{}, nfull);
+        if (nfull < ntiles) tile_body(std::true_type{}, nfull, nothing);
     } else {
 #pragma clang loop unroll(disable)
         for (int it = 0; it < ntiles; ++it) {
-            if (it + 1 < ntiles) load_tile((it + 1) * BK);
+            auto stage_ahead = [&]() __attribute__((always_inline)) {
+                if (it + 1 < ntiles) store_tile((it + 1) % NSTAGE);
+                if (it + 2 < ntiles) load_tile((it + 2) * BK);
+            };
             if (it < my_tiles) {
                 const int k0 = it * BK;
                 const bool masked = (k0 + BK > kend) || (CAUSAL && (k0 + BK - 1 > wq0));
-                if (HAS_MASK || PER_KEY || masked) tile_body(std::true_type{}, it);
-                else tile_body(std::false_type{}, it);
+                if (HAS_MASK || PER_KEY || masked) tile_body(std::true_type{}, it, stage_ahead);
+                else tile_body(std::false_type{}, it, stage_ahead);
+            } else {
+                stage_ahead();
             }
-            if (it + 1 < ntiles) store_tile((it + 1) % NSTAGE);
             __syncthreads();
         }
     }
