@@ -32,7 +32,8 @@ static int check_common(const char *fn, arhip_device *dev, const void *q, const 
                   (long long)B, (long long)Hq, (long long)Hkv, (long long)N);
     ARHIP_REQUIRE(Hq % Hkv == 0, "%s: Hq=%lld is not a multiple of Hkv=%lld", fn, (long long)Hq, (long long)Hkv);
     if (D != 64 && D != 128) return arhip_fail(ARHIP_EUNSUPPORTED, "%s: head_dim %lld (64 or 128)", fn, (long long)D);
-    if (N > ((int64_t)1 << 24) || B * Hq > ((int64_t)1 << 24))
+    // workgroup ids, tile counts and row indices are 32-bit in the kernels
+    if (N > ((int64_t)1 << 24) || B * Hq > ((int64_t)1 << 24) || B * Hq * ((N + 31) / 32) > ((int64_t)1 << 30))
         return arhip_fail(ARHIP_EUNSUPPORTED, "%s: shape too large for 32-bit tile indices", fn);
     ARHIP_REQUIRE(arhip_aligned16(q) && arhip_aligned16(k) && arhip_aligned16(v) && arhip_aligned16(o),
                   "%s: q/k/v/o must be 16-byte aligned", fn);
