@@ -162,6 +162,45 @@ __global__ void __launch_bounds__(256) quant_blocks_kernel(const T *x, int8_t *x
     }
 }
 
+// The reference's own granularity, one scale per token row (block == 1): D/8 lanes share a row,
+// so a workgroup of 256 threads quantises 256/(D/8) rows and the absmax is a shuffle reduction
+// inside the lane group.  Same arithmetic, same order of operations per element.
+template <typename T, bool SMOOTH>
+__global__ void __launch_bounds__(256) quant_rows_kernel(const T *x, int8_t *x8, float *scales, const float *mean,
+                                                         int N, int D, long rows_total)
+{
+    const int gpr = D / 8;                                   // lanes per row (8 or 16)
+    const long row = (long)blockIdx.x * (256 / gpr) + threadIdx.x / gpr;   // global row over [B*H*N]
+    const int g = threadIdx.x % gpr;
+    const bool live = row < rows_total;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        ld8(x, (size_t)row * D + g * 8, v);
+        if (SMOOTH) {
+            const float *mu = mean + (size_t)(row / N) * D + g * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = v[i] - mu[i];
+        }
+    }
+    float mx = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) mx = fmaxf(mx, fabsf(v[i]));
+    for (int off = gpr >> 1; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    const float scale = (mx > 0.f) ? mx / 127.0f : 1.f;
+    const float inv = 1.f / scale;
+    if (live) {
+        if (g == 0) scales[row] = scale;
+        uint32_t w[2] = {0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int iv = (int)rintf(v[i] * inv);
+            iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
+            w[i >> 2] |= ((uint32_t)iv & 0xffu) << ((i & 3) * 8);
+        }
+        *(uint2 *)(x8 + (size_t)row * D + g * 8) = make_uint2(w[0], w[1]);
+    }
+}
+
 __global__ void __launch_bounds__(256) cast_bf16_kernel(const float *x, uint16_t *y, size_t n)
 {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -211,6 +250,27 @@ extern "C" int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, fl
                                (const uint16_t *)x, (float *)workspace, (int)N, (int)D, nchunk);
         hipLaunchKernelGGL(k_mean_final_kernel, dim3((unsigned)(B * H)), dim3((unsigned)D), 0, dev->stream,
                            (const float *)workspace, mean, (int)N, (int)D, nchunk);
+    }
+    if (block == 1) {  // scales [B,H,N]: one per row
+        const long rows = (long)(B * H * N);
+        const int rpb = 256 / (int)(D / 8);
+        const dim3 rgrid((unsigned)((rows + rpb - 1) / rpb));
+        if (smooth) {
+            if (dtype == ARHIP_F32)
+                hipLaunchKernelGGL((quant_rows_kernel<float, true>), rgrid, dim3(256), 0, dev->stream,
+                                   (const float *)x, x8, scales, mean, (int)N, (int)D, rows);
+            else
+                hipLaunchKernelGGL((quant_rows_kernel<uint16_t, true>), rgrid, dim3(256), 0, dev->stream,
+                                   (const uint16_t *)x, x8, scales, mean, (int)N, (int)D, rows);
+        } else {
+            if (dtype == ARHIP_F32)
+                hipLaunchKernelGGL((quant_rows_kernel<float, false>), rgrid, dim3(256), 0, dev->stream,
+                                   (const float *)x, x8, scales, nullptr, (int)N, (int)D, rows);
+            else
+                hipLaunchKernelGGL((quant_rows_kernel<uint16_t, false>), rgrid, dim3(256), 0, dev->stream,
+                                   (const uint16_t *)x, x8, scales, nullptr, (int)N, (int)D, rows);
+        }
+    } else if (smooth) {
         if (dtype == ARHIP_F32)
             hipLaunchKernelGGL((quant_blocks_kernel<float, true>), qgrid, dim3(256), 0, dev->stream,
                                (const float *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk);

@@ -48,10 +48,13 @@ class SageWorkload:
     """SageAttention INT8 forward: Q ~ N(0,1), K = N(0,1) + per-(head,channel) bias ~ N(0, sigma),
     V ~ N(0,1); all three stored as bf16; O bf16."""
 
-    def __init__(self, dev, B, H, S, D, causal, sigma, outliers, cfg, bq=128, bk=64):
+    def __init__(self, dev, B, H, S, D, causal, sigma, outliers, cfg, bq=128, bk=64, f32_io=False):
         self.dev, self.B, self.H, self.S, self.D, self.causal = dev, B, H, S, D, causal
         self.bq, self.bk = bq, bk
-        self.name = "sage_int8_b%d_h%d_s%d_d%d%s" % (B, H, S, D, "_causal" if causal else "")
+        # f32_io: the reference's own convention (f32 tensors in, f32 out, per-row scales, no smoothing)
+        self.f32_io = f32_io
+        self.name = "sage_int8_b%d_h%d_s%d_d%d%s%s" % (B, H, S, D, "_causal" if causal else "",
+                                                        "_f32io_rowscales" if f32_io else "")
         n = B * H * S * D
         base = 1000 * cfg
         q = synth.normal(base + 1, (B, H, S, D))
@@ -65,12 +68,18 @@ class SageWorkload:
                     hit = synth.uniform(seed, m, o) < outliers
                     flat[o:o + m][hit] *= np.float32(20.0)
         self.host = {"q": q, "k": k}
-        self.dq = dev.from_numpy(synth.to_bf16_bits(q))
-        self.dk = dev.from_numpy(synth.to_bf16_bits(k))
         v = synth.normal(base + 3, (B, H, S, D))
         self.host["v"] = v
-        self.dv = dev.from_numpy(synth.to_bf16_bits(v))
-        self.do = dev.alloc(n * 2)
+        if f32_io:
+            self.dq, self.dk, self.dvf = dev.from_numpy(q), dev.from_numpy(k), dev.from_numpy(v)
+            self.dv = dev.alloc(n * 2)
+            self.do = dev.alloc(n * 4)
+        else:
+            self.dq = dev.from_numpy(synth.to_bf16_bits(q))
+            self.dk = dev.from_numpy(synth.to_bf16_bits(k))
+            self.dvf = None
+            self.dv = dev.from_numpy(synth.to_bf16_bits(v))
+            self.do = dev.alloc(n * 2)
         self.q8, self.k8 = dev.alloc(n), dev.alloc(n)
         self.sq = dev.alloc(B * H * ((S + bq - 1) // bq) * 4)
         self.sk = dev.alloc(B * H * ((S + bk - 1) // bk) * 4)
@@ -84,11 +93,14 @@ class SageWorkload:
 
     def step(self):
         d, B, H, S, D = self.dev, self.B, self.H, self.S, self.D
-        d.sage_quant(self.dq, self.q8, self.sq, B, H, S, D, self.bq, BF16, wait=False)
-        d.sage_quant(self.dk, self.k8, self.sk, B, H, S, D, self.bk, BF16, mean=self.mean, workspace=self.ws,
-                     smooth=True, wait=False)
+        io = F32 if self.f32_io else BF16
+        d.sage_quant(self.dq, self.q8, self.sq, B, H, S, D, self.bq, io, wait=False)
+        d.sage_quant(self.dk, self.k8, self.sk, B, H, S, D, self.bk, io, mean=self.mean, workspace=self.ws,
+                     smooth=not self.f32_io, wait=False)
+        if self.f32_io:
+            d.cast_bf16(self.dvf, self.dv, B * H * S * D, wait=False)
         d.sage_fwd(self.q8, self.k8, self.sq, self.sk, self.dv, self.do, B, H, H, S, D, self.bq, self.bk,
-                   out_dtype=BF16, causal=self.causal, wait=False)
+                   out_dtype=io, causal=self.causal, wait=False)
 
     def roofline(self, secs):
         half = self.ops / 2.0
@@ -100,8 +112,9 @@ class SageWorkload:
                 "frac_of_mixed_int8_bf16_bound": t_min / secs}
 
     def free(self):
-        for b in (self.dq, self.dk, self.dv, self.do, self.q8, self.k8, self.sq, self.sk, self.mean, self.ws):
-            b.free()
+        for b in (self.dq, self.dk, self.dv, self.dvf, self.do, self.q8, self.k8, self.sq, self.sk, self.mean, self.ws):
+            if b is not None:
+                b.free()
 
 
 class FlashWorkload:
@@ -213,7 +226,19 @@ def build_workload(dev, name):
         return FlashWorkload(dev, 4, 32, 2048, 128, True, BF16, cfg=3, kv_lens=True)
     if name == "vit_f32":
         return FlashWorkload(dev, 1, 12, 197, 64, False, F32, cfg=1)
+    # the shape the reference publishes its own kernel times on (B8 H6 N789 D64, PERFORMANCE.md:314-317)
+    if name == "ref_bf16":
+        return FlashWorkload(dev, 8, 6, 789, 64, False, BF16, cfg=7)
+    if name == "ref_f32":
+        return FlashWorkload(dev, 8, 6, 789, 64, False, F32, cfg=7)
+    if name == "ref_sage":
+        return SageWorkload(dev, 8, 6, 789, 64, False, 0.0, 0.0, cfg=7, bq=1, bk=1, f32_io=True)
     raise SystemExit("unknown workload %r" % name)
+
+
+# The reference's published kernel times for that shape, on an RTX 3060 (not comparable hardware;
+# reported next to ours for orientation only): PERFORMANCE.md:314-317.
+REFERENCE_RTX3060_MS = {"ref_f32": 7.0, "ref_bf16": 0.53, "ref_sage": 1.26}
 
 
 def main():
@@ -222,7 +247,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="sage",
-                    choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32", "flash_long"])
+                    choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32", "flash_long", "ref_bf16",
+                             "ref_f32", "ref_sage"])
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="one step of the workload plus one plain 1 GiB copy kernel and nothing else: "
@@ -252,18 +278,22 @@ def main():
     log(json.dumps(res))
     cpu = None
     if not args.no_cpu:
-        heads = {"sage": 2, "sage_causal_long": 1, "decoder": 16, "vit": 96, "vit_f32": 12, "flash_long": 2}[args.workload]
+        heads = {"sage": 2, "sage_causal_long": 1, "decoder": 16, "vit": 96, "vit_f32": 12, "flash_long": 2}.get(
+            args.workload, 48)
         cpu = cpu_baseline(w, heads)
         log(json.dumps(cpu))
     w.free()
 
     secondary = []
     if not args.no_secondary:
-        for name in ("vit", "decoder", "flash_long", "vit_f32", "sage", "sage_causal_long"):
+        for name in ("vit", "decoder", "flash_long", "vit_f32", "sage", "sage_causal_long", "ref_bf16", "ref_f32",
+                     "ref_sage"):
             if name == args.workload:
                 continue
             sw = build_workload(dev, name)
-            r = measure(dev, sw, max(args.steps, 20) if name.startswith("vit") else args.steps, args.warmup)
+            r = measure(dev, sw, max(args.steps, 20) if sw.S < 1024 else args.steps, args.warmup)
+            if name in REFERENCE_RTX3060_MS:
+                r["reference_kernel_ms_rtx3060"] = REFERENCE_RTX3060_MS[name]
             sw.free()
             log(json.dumps(r))
             secondary.append(r)

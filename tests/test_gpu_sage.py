@@ -121,3 +121,15 @@ def test_zero_block_and_outliers(dev):
     assert k8[0, 0, 70, 5] == 127
     want = oracle.sage(q8, k8, sq, sk, v, 128, 64)
     assert np.abs(r["out"] - want).max() < 4e-3
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_per_row_scales_with_smoothing(dev, D):
+    """Block size 1 (the reference's granularity) combined with this build's K smoothing."""
+    B, Hq, Hkv, N = 2, 4, 2, 333
+    q, k, v = _inputs(B, Hq, Hkv, N, D)
+    r = run_sage(dev, q, k, v, 1, 1, smooth=True)
+    q8, sq, k8, sk = _check_bits(r, q, k, v, 1, 1, True)
+    want = oracle.sage(q8, k8, sq, sk, v, 1, 1)
+    err = float(np.abs(r["out"] - want).max())
+    assert err < 4e-3
