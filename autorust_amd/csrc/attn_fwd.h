@@ -71,6 +71,9 @@ struct AttnParams {
     int32_t *dbg;            // MODE_I8 debug: [32][64] raw logits
     int dbg_bh, dbg_qt, dbg_kt;
     int Hq, Hkv, N;
+    // element strides of q / k,v / o: [batch, head, token]; the channel stride is 1.
+    // Dense [B,H,N,D] is {H*N*D, N*D, D}; token-major [B,N,H,D] is {N*H*D, D, H*D}.
+    long qs[3], ks[3], os[3];
     int bq, bk;
     int bk_tile_shift;  // log2(bk / 64) when the K scales are tile-uniform
     int nq;        // query tiles per head
@@ -198,14 +201,17 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
     // tiles this wave takes part in: under the causal mask, none past its last query
     const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / BK + 1) : ntiles;
 
-    const unsigned char *kbase = (const unsigned char *)p.k + (size_t)kv_bh * N * D * QK_BYTES;
-    const uint16_t *vbase = p.v + (size_t)kv_bh * N * D;
+    const size_t kv_off = (size_t)b * p.ks[0] + (size_t)kvh * p.ks[1];
+    const size_t k_rs = (size_t)p.ks[2];  // elements between consecutive tokens of K / V
+    const unsigned char *kbase = (const unsigned char *)p.k + kv_off * QK_BYTES;
+    const uint16_t *vbase = p.v + kv_off;
 
     // ---- Q operand, resident in registers for the whole kernel.  Rows past N
     // read row N-1: their results are never stored. ----
     uint4 qreg[KSTEPS];
     {
-        const unsigned char *qb = (const unsigned char *)p.q + ((size_t)bh * N + (size_t)min(q_row, N - 1)) * D * QK_BYTES;
+        const unsigned char *qb = (const unsigned char *)p.q +
+                                  ((size_t)b * p.qs[0] + (size_t)head * p.qs[1] + (size_t)min(q_row, N - 1) * p.qs[2]) * QK_BYTES;
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) qreg[s] = *(const uint4 *)(qb + s * 32 + h * 16);
     }
@@ -225,9 +231,9 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
                 const int row = c / K_CPR, col = c % K_CPR;
                 const int gr = k0 + row;
                 if (full) {
-                    kst[slot][j] = *(const uint4 *)(kbase + (size_t)gr * (D * QK_BYTES) + col * 16);
+                    kst[slot][j] = *(const uint4 *)(kbase + (size_t)gr * k_rs * QK_BYTES + col * 16);
                 } else {
-                    uint4 val = *(const uint4 *)(kbase + (size_t)min(gr, kend - 1) * (D * QK_BYTES) + col * 16);
+                    uint4 val = *(const uint4 *)(kbase + (size_t)min(gr, kend - 1) * k_rs * QK_BYTES + col * 16);
                     if (gr >= kend) val = make_uint4(0, 0, 0, 0);
                     kst[slot][j] = val;
                 }
@@ -240,9 +246,9 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
                 const int row = c / V_CPR, col = c % V_CPR;
                 const int gr = k0 + row;
                 if (full) {
-                    vst[slot][j] = *(const uint4 *)(vbase + (size_t)gr * D + col * 8);
+                    vst[slot][j] = *(const uint4 *)(vbase + (size_t)gr * k_rs + col * 8);
                 } else {
-                    uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * D + col * 8);
+                    uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * k_rs + col * 8);
                     if (gr >= kend) val = make_uint4(0, 0, 0, 0);
                     vst[slot][j] = val;
                 }
@@ -525,7 +531,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
     const float l_tot = xhalf_sum(l_run);
     const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
     if (q_row < N) {
-        const size_t obase = ((size_t)bh * N + q_row) * D;
+        const size_t obase = (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)q_row * p.os[2];
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll

@@ -79,13 +79,45 @@ static int pick_waves(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bo
     return nw;
 }
 
+static void dense_strides(long s[3], int64_t H, int64_t N, int64_t D)
+{
+    s[0] = (long)(H * N * D);
+    s[1] = (long)(N * D);
+    s[2] = (long)D;
+}
+
 extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, const void *v, void *o,
                                const float *mask, const int32_t *kv_len,
                                int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
                                int causal, int dtype, float scale, int wait, double *secs)
 {
+    long qs[3], ks[3];
+    dense_strides(qs, Hq, N, D);
+    dense_strides(ks, Hkv, N, D);
+    const int64_t q64[3] = {qs[0], qs[1], qs[2]}, k64[3] = {ks[0], ks[1], ks[2]};
+    return arhip_flash_fwd_strided(dev, q, k, v, o, q64, k64, q64, mask, kv_len, B, Hq, Hkv, N, D, causal, dtype, scale,
+                                   wait, secs);
+}
+
+extern "C" int arhip_flash_fwd_strided(arhip_device *dev, const void *q, const void *k, const void *v, void *o,
+                                       const int64_t q_strides[3], const int64_t kv_strides[3], const int64_t o_strides[3],
+                                       const float *mask, const int32_t *kv_len,
+                                       int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                                       int causal, int dtype, float scale, int wait, double *secs)
+{
     if (int rc = check_common("arhip_flash_fwd", dev, q, k, v, o, mask, B, Hq, Hkv, N, D)) return rc;
     ARHIP_REQUIRE(dtype == ARHIP_F32 || dtype == ARHIP_BF16, "arhip_flash_fwd: dtype %d", dtype);
+    ARHIP_REQUIRE(q_strides && kv_strides && o_strides, "arhip_flash_fwd_strided: null strides");
+    {
+        // rows must stay 16-byte aligned and must not overlap: every stride a multiple of 8 elements,
+        // the token stride at least D
+        const int64_t *all[3] = {q_strides, kv_strides, o_strides};
+        for (int t = 0; t < 3; ++t)
+            for (int i = 0; i < 3; ++i)
+                ARHIP_REQUIRE(all[t][i] >= 0 && all[t][i] % 8 == 0 && (i != 2 || all[t][i] >= D),
+                              "arhip_flash_fwd_strided: stride %lld (multiples of 8 elements, token stride >= D)",
+                              (long long)all[t][i]);
+    }
     ARHIP_HIP(hipSetDevice(dev->ordinal));
     arhip_call_timer t{dev, wait, secs};
     t.kernel = (dtype == ARHIP_F32) ? ARHIP_K_FLASH_F32 : ARHIP_K_FLASH_BF16;
@@ -95,6 +127,11 @@ extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, 
         fp.q = (const float *)q; fp.k = (const float *)k; fp.v = (const float *)v; fp.o = (float *)o;
         fp.mask = mask; fp.kv_len = kv_len;
         fp.Hq = (int)Hq; fp.Hkv = (int)Hkv; fp.N = (int)N;
+        for (int i = 0; i < 3; ++i) {
+            fp.qs[i] = (long)q_strides[i];
+            fp.ks[i] = (long)kv_strides[i];
+            fp.os[i] = (long)o_strides[i];
+        }
         // 4 waves (128 queries) per workgroup when that still fills the chip, else 1 wave
         const int nw = (B * Hq * ((N + 127) / 128) >= 2 * (int64_t)dev->cus) ? 4 : 1;
         fp.nq = (int)((N + nw * 32 - 1) / (nw * 32));
@@ -120,6 +157,11 @@ extern "C" int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, 
     p.q = q; p.k = k; p.v = (const uint16_t *)v; p.o = o;
     p.mask = mask; p.kv_len = kv_len;
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
+    for (int i = 0; i < 3; ++i) {
+        p.qs[i] = (long)q_strides[i];
+        p.ks[i] = (long)kv_strides[i];
+        p.os[i] = (long)o_strides[i];
+    }
     p.bq = p.bk = 1;
     p.scale = scale;
     const bool c = causal != 0, hm = mask != nullptr;
@@ -173,6 +215,9 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
     p.mask = mask; p.kv_len = kv_len;
     p.sq = sq; p.sk = sk;
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
+    dense_strides(p.qs, Hq, N, D);
+    dense_strides(p.ks, Hkv, N, D);
+    dense_strides(p.os, Hq, N, D);
     p.bq = (int)bq; p.bk = (int)bk;
     p.scale = scale;
     const bool dbg = dbg_logits != nullptr;

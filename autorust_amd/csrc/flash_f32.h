@@ -31,6 +31,7 @@ struct FlashF32Params {
     const float *mask;      // additive [N,N] or null
     const int32_t *kv_len;  // [B] or null
     int Hq, Hkv, N, nq;
+    long qs[3], ks[3], os[3];  // element strides [batch, head, token] of q / k,v / o (channel stride 1)
     float scale;
 };
 
@@ -55,7 +56,6 @@ __global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params
     int qt = blockIdx.x - bh * p.nq;
     if (CAUSAL) qt = p.nq - 1 - qt;
     const int b = bh / p.Hq, head = bh - b * p.Hq;
-    const int kv_bh = b * p.Hkv + head / (p.Hq / p.Hkv);
     const int N = p.N;
     const int qblk = qt * BQ;
     const int wq0 = qblk + wave * 32;
@@ -71,13 +71,16 @@ __global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params
     const int ntiles = (kend + F32_BK - 1) / F32_BK;
     const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / F32_BK + 1) : ntiles;
 
-    const float *kp = p.k + (size_t)kv_bh * N * D;
-    const float *vp = p.v + (size_t)kv_bh * N * D;
+    const int kvh = head / (p.Hq / p.Hkv);
+    const size_t kv_off = (size_t)b * p.ks[0] + (size_t)kvh * p.ks[1];
+    const size_t k_rs = (size_t)p.ks[2];
+    const float *kp = p.k + kv_off;
+    const float *vp = p.v + kv_off;
 
     // Q: this lane's half of its query row (rows past N read row N-1; never stored)
     float qr[HALF];
     {
-        const float *qp = p.q + ((size_t)bh * N + min(q_row, N - 1)) * D + h * HALF;
+        const float *qp = p.q + (size_t)b * p.qs[0] + (size_t)head * p.qs[1] + (size_t)min(q_row, N - 1) * p.qs[2] + h * HALF;
 #pragma unroll
         for (int s = 0; s < HALF; s += 4) {
             const float4 x = *(const float4 *)(qp + s);
@@ -102,8 +105,8 @@ __global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params
             const int gr = k0 + row;
             float4 kx = make_float4(0.f, 0.f, 0.f, 0.f), vx = kx;
             if (gr < kend) {
-                kx = *(const float4 *)(kp + (size_t)gr * D + col);
-                vx = *(const float4 *)(vp + (size_t)gr * D + col);
+                kx = *(const float4 *)(kp + (size_t)gr * k_rs + col);
+                vx = *(const float4 *)(vp + (size_t)gr * k_rs + col);
             }
             *(float4 *)&ks[row * KROW + col] = kx;
             *(float4 *)&vs[row * D + col] = vx;
@@ -168,7 +171,7 @@ __global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
     if (q_row < N) {
-        float *op = p.o + ((size_t)bh * N + q_row) * D;
+        float *op = p.o + (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)q_row * p.os[2];
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll

@@ -139,6 +139,18 @@ class Device:
                                        scale, int(wait), ctypes.byref(s)))
         return s.value if wait else None
 
+    def flash_fwd_strided(self, q, k, v, o, q_strides, kv_strides, o_strides, B, Hq, Hkv, N, D, dtype, mask=None,
+                          kv_len=None, causal=False, scale=None, wait=True):
+        """Element strides {batch, head, token} per tensor; see include/arhip.h."""
+        scale = float(1.0 / np.sqrt(np.float32(D))) if scale is None else float(scale)
+        arr = lambda t: (ctypes.c_int64 * 3)(*[int(x) for x in t])
+        s = ctypes.c_double()
+        check(self.lib.arhip_flash_fwd_strided(self.handle, self._ptr(q), self._ptr(k), self._ptr(v), self._ptr(o),
+                                               arr(q_strides), arr(kv_strides), arr(o_strides), self._ptr(mask),
+                                               self._ptr(kv_len), B, Hq, Hkv, N, D, int(causal), dtype, scale,
+                                               int(wait), ctypes.byref(s)))
+        return s.value if wait else None
+
     def sage_quant_workspace(self, B, H, N, D):
         return self.lib.arhip_sage_quant_workspace(B, H, N, D)
 

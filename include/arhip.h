@@ -127,6 +127,20 @@ int arhip_flash_fwd(arhip_device *dev, const void *q, const void *k, const void 
                     int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
                     int causal, int dtype, float scale, int wait, double *secs);
 
+/* arhip_flash_fwd_strided: the same kernels on strided tensors.  Strides are in elements,
+ *   {batch, head, token}; the channel stride is 1.  Dense [B,H,N,D] is {H*N*D, N*D, D};
+ *   the token-major layout the projections produce, [B,N,H,D], is {N*H*D, D, H*D}.
+ *   This is the caller-side fusion the reference lists as missing: its transformer block
+ *   copies q/k/v into [B,H,S,hs] before the kernel and the result back
+ *   (src/models/transformer.rs:286-299); with strides both copies disappear (pass the
+ *   projection output as is, and ask for o in [B,N,H*D]).
+ *   Every stride must be a multiple of 8 elements, the token stride >= D. */
+int arhip_flash_fwd_strided(arhip_device *dev, const void *q, const void *k, const void *v, void *o,
+                            const int64_t q_strides[3], const int64_t kv_strides[3], const int64_t o_strides[3],
+                            const float *mask, const int32_t *kv_len,
+                            int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                            int causal, int dtype, float scale, int wait, double *secs);
+
 /* arhip_sage_quant: the quantiser of the Sage kernel hoisted into a pre-pass
  *   (the reference quantises inside the attention kernel, K once per query
  *   block: src/runtime/cuda_flash_sage.rs:201-223, 248-278).

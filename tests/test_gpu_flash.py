@@ -123,3 +123,32 @@ def test_bf16_is_deterministic(dev):
     a = run_flash(dev, q, k, v, BF16)
     b = run_flash(dev, q, k, v, BF16)
     assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [BF16, F32])
+@pytest.mark.parametrize("D,N", [(64, 197), (128, 300), (128, 1100)])
+def test_token_major_layout_is_the_same_function(dev, dtype, D, N):
+    """Strided entry point: q/k/v as the projections produce them, [B, N, H, D], and the output
+    written as [B, N, H*D] (what src/models/transformer.rs:286-299 reaches with two copies)
+    must equal the dense [B, H, N, D] call bit for bit."""
+    from gpu_util import Bufs
+    B, Hq, Hkv = 2, 4, 2
+    q, k, v = synth.normal(901, (B, Hq, N, D)), synth.normal(902, (B, Hkv, N, D)), synth.normal(903, (B, Hkv, N, D))
+    dense = run_flash(dev, q, k, v, dtype, causal=True)
+    conv = (lambda t: synth.to_bf16_bits(t)) if dtype == BF16 else (lambda t: t.astype(np.float32))
+    es = 2 if dtype == BF16 else 4
+    with Bufs(dev) as bufs:
+        tq, tk, tv = (bufs.put(conv(np.ascontiguousarray(t.transpose(0, 2, 1, 3)))) for t in (q, k, v))
+        to = bufs.new(q.size * es)
+        dev.flash_fwd_strided(tq, tk, tv, to, (N * Hq * D, D, Hq * D), (N * Hkv * D, D, Hkv * D), (N * Hq * D, D, Hq * D),
+                              B, Hq, Hkv, N, D, dtype, causal=True)
+        raw = to.copyout(np.uint16 if dtype == BF16 else np.float32, (B, N, Hq, D))
+    got = (synth.from_bf16_bits(raw) if dtype == BF16 else raw).transpose(0, 2, 1, 3)
+    assert np.array_equal(got, dense)
+    # strides that would misalign rows are rejected
+    with pytest.raises(_lib.ArhipError):
+        d = dev.alloc(64)
+        try:
+            dev.flash_fwd_strided(d, d, d, d, (N * D, D, D + 4), (N * D, D, D), (N * D, D, D), 1, 1, 1, N, D, dtype)
+        finally:
+            d.free()
