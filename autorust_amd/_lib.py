@@ -52,6 +52,10 @@ SIGNATURES = {
                                         ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), ctypes.POINTER(c_int64),
                                         c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                         c_int, c_int, c_float, c_int, _pd]),
+    "arhip_flash_fwd_lse": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                    ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), ctypes.POINTER(c_int64),
+                                    c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                    c_int, c_int, c_float, c_int, _pd]),
     "arhip_sage_quant_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "arhip_sage_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),

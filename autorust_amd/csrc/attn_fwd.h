@@ -68,6 +68,7 @@ struct AttnParams {
     const int32_t *kv_len;   // [B] or null
     const float *sq;         // MODE_I8: [B,Hq,ceil(N/bq)]
     const float *sk;         // MODE_I8: [B,Hkv,ceil(N/bk)]
+    float *lse;              // optional [B,Hq,N]: log-sum-exp of the scaled, masked logits (natural log)
     int32_t *dbg;            // MODE_I8 debug: [32][64] raw logits
     int dbg_bh, dbg_qt, dbg_kt;
     int Hq, Hkv, N;
@@ -530,8 +531,13 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
     // ---- normalise and store: acc * (l > 0 ? 1/l : 0), cuda_flash_bf16.rs:414-426 ----
     const float l_tot = xhalf_sum(l_run);
     const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+    if (p.lse != nullptr && h == 0 && q_row < N) {
+        // LSE = m + log(l) in natural units (src/runtime/cuda_flash_train.rs:141); m_run is kept in
+        // the exp2 domain, so LSE = (m_run + log2 l) * ln 2
+        p.lse[(size_t)bh * N + q_row] = (l_tot > 0.f) ? (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : NEG_SENTINEL;
+    }
     if (q_row < N) {
-        const size_t obase = (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)q_row * p.os[2];
+        const size_t obase =(size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)q_row * p.os[2];
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll

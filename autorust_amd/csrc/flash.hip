@@ -64,7 +64,7 @@ static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bo
 // Tiling variants = waves (of 32 queries) per workgroup.
 //   1  32 queries per workgroup: short sequences, spreads the heads over the chip
 //   4  128 queries
-//   8  256 queries, two waves per SIMD running one phase apart (long sequences)
+//   8  256 queries, two waves per SIMD (long sequences)
 static int pick_waves(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bool special)
 {
     // masks, per-key scales and the debug export are built for 4 waves (and 1 at D = 64) only
@@ -105,7 +105,18 @@ extern "C" int arhip_flash_fwd_strided(arhip_device *dev, const void *q, const v
                                        int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
                                        int causal, int dtype, float scale, int wait, double *secs)
 {
+    return arhip_flash_fwd_lse(dev, q, k, v, o, nullptr, q_strides, kv_strides, o_strides, mask, kv_len, B, Hq, Hkv, N, D,
+                               causal, dtype, scale, wait, secs);
+}
+
+extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void *k, const void *v, void *o, float *lse,
+                                   const int64_t q_strides[3], const int64_t kv_strides[3], const int64_t o_strides[3],
+                                   const float *mask, const int32_t *kv_len,
+                                   int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                                   int causal, int dtype, float scale, int wait, double *secs)
+{
     if (int rc = check_common("arhip_flash_fwd", dev, q, k, v, o, mask, B, Hq, Hkv, N, D)) return rc;
+    ARHIP_REQUIRE(lse == nullptr || (reinterpret_cast<uintptr_t>(lse) & 3u) == 0, "arhip_flash_fwd_lse: lse must be 4-byte aligned");
     ARHIP_REQUIRE(dtype == ARHIP_F32 || dtype == ARHIP_BF16, "arhip_flash_fwd: dtype %d", dtype);
     ARHIP_REQUIRE(q_strides && kv_strides && o_strides, "arhip_flash_fwd_strided: null strides");
     {
@@ -125,7 +136,7 @@ extern "C" int arhip_flash_fwd_strided(arhip_device *dev, const void *q, const v
     if (dtype == ARHIP_F32) {
         FlashF32Params fp;
         fp.q = (const float *)q; fp.k = (const float *)k; fp.v = (const float *)v; fp.o = (float *)o;
-        fp.mask = mask; fp.kv_len = kv_len;
+        fp.mask = mask; fp.kv_len = kv_len; fp.lse = lse;
         fp.Hq = (int)Hq; fp.Hkv = (int)Hkv; fp.N = (int)N;
         for (int i = 0; i < 3; ++i) {
             fp.qs[i] = (long)q_strides[i];
@@ -155,7 +166,7 @@ extern "C" int arhip_flash_fwd_strided(arhip_device *dev, const void *q, const v
 
     AttnParams p = {};
     p.q = q; p.k = k; p.v = (const uint16_t *)v; p.o = o;
-    p.mask = mask; p.kv_len = kv_len;
+    p.mask = mask; p.kv_len = kv_len; p.lse = lse;
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
     for (int i = 0; i < 3; ++i) {
         p.qs[i] = (long)q_strides[i];

@@ -30,6 +30,7 @@ struct FlashF32Params {
     float *o;
     const float *mask;      // additive [N,N] or null
     const int32_t *kv_len;  // [B] or null
+    float *lse;             // optional [B,Hq,N]: m + log(l), src/runtime/cuda_flash_train.rs:141
     int Hq, Hkv, N, nq;
     long qs[3], ks[3], os[3];  // element strides [batch, head, token] of q / k,v / o (channel stride 1)
     float scale;
@@ -170,6 +171,8 @@ __global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+    if (p.lse != nullptr && h == 0 && q_row < N)
+        p.lse[(size_t)bh * N + q_row] = (l_tot > 0.f) ? m_run + logf(l_tot) : -1e30f;
     if (q_row < N) {
         float *op = p.o + (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)q_row * p.os[2];
 #pragma unroll

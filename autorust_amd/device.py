@@ -151,6 +151,19 @@ class Device:
                                                int(wait), ctypes.byref(s)))
         return s.value if wait else None
 
+    def flash_fwd_lse(self, q, k, v, o, lse, B, Hq, Hkv, N, D, dtype, mask=None, kv_len=None, causal=False,
+                      scale=None, wait=True):
+        """Dense [B,H,N,D] tensors; also writes lse [B,Hq,N] (f32)."""
+        scale = float(1.0 / np.sqrt(np.float32(D))) if scale is None else float(scale)
+        arr = lambda t: (ctypes.c_int64 * 3)(*[int(x) for x in t])
+        qs, ks = (Hq * N * D, N * D, D), (Hkv * N * D, N * D, D)
+        s = ctypes.c_double()
+        check(self.lib.arhip_flash_fwd_lse(self.handle, self._ptr(q), self._ptr(k), self._ptr(v), self._ptr(o),
+                                           self._ptr(lse), arr(qs), arr(ks), arr(qs), self._ptr(mask),
+                                           self._ptr(kv_len), B, Hq, Hkv, N, D, int(causal), dtype, scale,
+                                           int(wait), ctypes.byref(s)))
+        return s.value if wait else None
+
     def sage_quant_workspace(self, B, H, N, D):
         return self.lib.arhip_sage_quant_workspace(B, H, N, D)
 

@@ -141,6 +141,16 @@ int arhip_flash_fwd_strided(arhip_device *dev, const void *q, const void *k, con
                             int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
                             int causal, int dtype, float scale, int wait, double *secs);
 
+/* arhip_flash_fwd_lse: arhip_flash_fwd_strided that also writes, when lse != NULL, the
+ *   log-sum-exp of the scaled, masked logits of every query row, f32 [B,Hq,N] (natural log;
+ *   -1e30 for a row without visible keys): the statistic the reference's training forward
+ *   saves as LSE = m + log(l) (src/runtime/cuda_flash_train.rs:5-11,141) for its backward. */
+int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void *k, const void *v, void *o, float *lse,
+                        const int64_t q_strides[3], const int64_t kv_strides[3], const int64_t o_strides[3],
+                        const float *mask, const int32_t *kv_len,
+                        int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                        int causal, int dtype, float scale, int wait, double *secs);
+
 /* arhip_sage_quant: the quantiser of the Sage kernel hoisted into a pre-pass
  *   (the reference quantises inside the attention kernel, K once per query
  *   block: src/runtime/cuda_flash_sage.rs:201-223, 248-278).

@@ -123,6 +123,28 @@ def sdpa_f64(q, k, v, mask=None, causal=False, kv_len=None, rows=None, scale=Non
     return _heads(lib().ar_head_sdpa_f64, q, k, v, mask, causal, kv_len, rows, (ctypes.c_double(scale),))
 
 
+def lse_f64(q, k, mask=None, causal=False, kv_len=None, rows=None, scale=None):
+    """log-sum-exp of the scaled, masked logits per query row: [B, H, rows] (float64 inside)."""
+    q, k = _f32(q), _f32(k)
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    group = Hq // Hkv
+    scale = 1.0 / np.sqrt(D) if scale is None else scale
+    if mask is not None:
+        mask = np.ascontiguousarray(np.broadcast_to(_f32(mask), (B, Hq, N, N)))
+    kv_len = np.full(B, -1, np.int32) if kv_len is None else np.ascontiguousarray(kv_len, np.int32)
+    if rows is not None:
+        rows = np.ascontiguousarray(rows, dtype=np.int32)
+    nrows = N if rows is None else len(rows)
+    out = np.empty((B, Hq, nrows), dtype=np.float32)
+    for b in range(B):
+        for h in range(Hq):
+            m = None if mask is None else mask[b, h]
+            lib().ar_head_lse_f64(_p(q[b, h], _f32p), _p(k[b, h // group], _f32p), _p(m, _f32p), N, D, int(causal),
+                                  int(kv_len[b]), ctypes.c_double(scale), _p(rows, _i32p), nrows, _p(out[b, h], _f32p))
+    return out
+
+
 def flash_f32(q, k, v, mask=None, causal=False, kv_len=None, rows=None, scale=None, bq=64, bk=32):
     """fp32 exact-mode FA2 kernel restated (src/runtime/cuda_flash.rs:53-141)."""
     scale = np.float32(1.0) / np.sqrt(np.float32(q.shape[-1])) if scale is None else scale

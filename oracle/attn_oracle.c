@@ -24,6 +24,7 @@
  *   ar_head_sdpa_f32/f64  the six reference-held vectors of
  *                         tests/attention_golden.rs (tolerance of
  *                         tests/nn_attention.rs:20), torch's CPU SDPA, fp64.
+ *   ar_head_lse_f64       scipy.special.logsumexp / torch.logsumexp (library).
  *   ar_head_flash_f32     equals SDPA by the online-softmax identity; special
  *                         cases by brute force (fully masked row -> mean of V).
  *   ar_head_bf16          bf16 RNE against torch.bfloat16 casts; equals
@@ -173,6 +174,38 @@ void ar_head_sdpa_f64(const float *q, const float *k, const float *v, const floa
                 out[(size_t)r * D + t] = (float)(acc / sum);
             }
         }
+        free(s);
+    }
+}
+
+/* Log-sum-exp of the masked, scaled logits of every evaluated row, in binary64:
+ * lse[r] = log(sum_j exp(s_rj)), the statistic the reference's training forward saves as
+ * LSE = m + log(l) (src/runtime/cuda_flash_train.rs:5-11,141).  A row without any visible
+ * key gets the finite sentinel -1e30 like there. */
+void ar_head_lse_f64(const float *q, const float *k, const float *mask,
+                     int N, int D, int causal, int kv_len, double scale,
+                     const int *rows, int nrows, float *lse)
+{
+    const int L = kvn(kv_len, N);
+#pragma omp parallel for schedule(dynamic, 4)
+    for (int r = 0; r < nrows; ++r) {
+        const int i = row_of(rows, r);
+        double mx = -INFINITY;
+        double *s = (double *)malloc(sizeof(double) * (size_t)N);
+        for (int j = 0; j < N; ++j) {
+            double x = -INFINITY;
+            if (!(causal && j > i) && j < L) {
+                double dot = 0.0;
+                for (int t = 0; t < D; ++t) dot += (double)q[(size_t)i * D + t] * (double)k[(size_t)j * D + t];
+                x = dot * scale;
+                if (mask) x += (double)mask[(size_t)i * N + j];
+            }
+            s[j] = x;
+            if (x > mx) mx = x;
+        }
+        double sum = 0.0;
+        for (int j = 0; j < N; ++j) sum += exp(s[j] - mx);
+        lse[r] = (mx > -INFINITY) ? (float)(mx + log(sum)) : AR_NEG;
         free(s);
     }
 }

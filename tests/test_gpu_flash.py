@@ -152,3 +152,30 @@ def test_token_major_layout_is_the_same_function(dev, dtype, D, N):
             dev.flash_fwd_strided(d, d, d, d, (N * D, D, D + 4), (N * D, D, D), (N * D, D, D), 1, 1, 1, N, D, dtype)
         finally:
             d.free()
+
+
+@pytest.mark.parametrize("dtype,tol", [(F32, 2e-5), (BF16, 2e-2)])
+@pytest.mark.parametrize("D,N", [(64, 197), (128, 700)])
+def test_log_sum_exp_output(dev, dtype, tol, D, N):
+    """The statistic of the reference's training forward (LSE = m + log l,
+    src/runtime/cuda_flash_train.rs:141) against the float64 log-sum-exp; the attention
+    output itself must be unchanged by asking for it."""
+    from gpu_util import Bufs
+    B, Hq, Hkv = 2, 4, 2
+    q, k, v = synth.normal(911, (B, Hq, N, D)), synth.normal(912, (B, Hkv, N, D)), synth.normal(913, (B, Hkv, N, D))
+    kv_len = np.array([N, N // 3], np.int32)
+    plain = run_flash(dev, q, k, v, dtype, kv_len=kv_len, causal=True)
+    conv = (lambda t: synth.to_bf16_bits(t)) if dtype == BF16 else (lambda t: t.astype(np.float32))
+    es = 2 if dtype == BF16 else 4
+    with Bufs(dev) as bufs:
+        dq, dk, dv = (bufs.put(conv(t)) for t in (q, k, v))
+        do, dl, dk_len = bufs.new(q.size * es), bufs.new(B * Hq * N * 4), bufs.put(kv_len)
+        dev.flash_fwd_lse(dq, dk, dv, do, dl, B, Hq, Hkv, N, D, dtype, kv_len=dk_len, causal=True)
+        raw = do.copyout(np.uint16 if dtype == BF16 else np.float32, q.shape)
+        lse = dl.copyout(np.float32, (B, Hq, N))
+    got = synth.from_bf16_bits(raw) if dtype == BF16 else raw
+    assert np.array_equal(got, plain)
+    qq, kk = (oracle.bf16_round(q), oracle.bf16_round(k)) if dtype == BF16 else (q, k)
+    want = oracle.lse_f64(qq, kk, kv_len=kv_len, causal=True)
+    err = float(np.abs(lse - want).max())
+    assert err <= tol

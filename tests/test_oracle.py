@@ -270,3 +270,15 @@ def test_cpu_baseline_matches_oracle():
         want = oracle.sdpa_f64(q, k, v, causal=causal)
         assert threads >= 1
         assert (np.abs(out - want) / np.maximum(np.abs(want), 1)).max() <= 1e-5
+
+
+def test_log_sum_exp_against_scipy():
+    import scipy.special as sp
+    B, Hq, Hkv, N, D = 1, 4, 2, 45, 64
+    q, k = synth.normal(81, (B, Hq, N, D)), synth.normal(82, (B, Hkv, N, D))
+    s = np.einsum("bhid,bhjd->bhij", q.astype(np.float64), np.repeat(k, 2, 1).astype(np.float64)) / np.sqrt(D)
+    s = np.where(np.tril(np.ones((N, N), bool)), s, -np.inf)
+    s[:, :, :, 30:] = -np.inf                      # kv_len = 30
+    want = sp.logsumexp(s, axis=-1)
+    got = oracle.lse_f64(q, k, causal=True, kv_len=np.array([30], np.int32))
+    assert np.abs(got - want).max() < 1e-5
