@@ -10,9 +10,11 @@
 //           the operand layout the second product needs: O^T = V^T . P^T, again
 //           with one query per lane (the softmax rescale is a per-lane scalar).
 //   tiles : BK = 64 keys per step, K and V staged through LDS by the whole
-//           workgroup: 128-bit global loads issued one tile ahead into
-//           registers, written to the other LDS stage after the math; one
-//           barrier per tile.
+//           workgroup (two stages, one barrier per tile) and two tiles ahead of
+//           the math: in the middle of the iteration that computes tile i, tile
+//           i+1 goes from registers to the stage tile i-1 vacated, and the
+//           128-bit global loads of tile i+2 are issued.  Sequences of at most
+//           256 keys are brought into LDS in one go instead (SMALL).
 //   blocks: inside a tile the online softmax advances 32 keys at a time and the
 //           wave alternates between the matrix pipe and the vector ALU; every
 //           LDS fragment is requested one phase before the MFMAs that use it.
