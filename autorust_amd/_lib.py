@@ -41,6 +41,10 @@ SIGNATURES = {
     "arhip_timer_stop": (c_int, [c_void_p, _pd]),
     "arhip_kprof_enable": (c_int, [c_void_p, c_int]),
     "arhip_kprof_collect": (c_int, [c_void_p, c_int, _pd, ctypes.POINTER(ctypes.c_uint64)]),
+    "arhip_graph_begin": (c_int, [c_void_p]),
+    "arhip_graph_end": (c_int, [c_void_p, ctypes.POINTER(c_void_p)]),
+    "arhip_graph_launch": (c_int, [c_void_p, c_void_p, c_int, _pd]),
+    "arhip_graph_destroy": (c_int, [c_void_p, c_void_p]),
     "arhip_module_load": (c_int, [c_void_p, c_void_p, c_size_t, ctypes.POINTER(c_void_p)]),
     "arhip_launch": (c_int, [c_void_p, c_void_p, c_char_p, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint),
                              ctypes.POINTER(c_void_p), c_int, ctypes.POINTER(c_int64), ctypes.POINTER(c_int), c_int,

@@ -31,6 +31,7 @@ struct arhip_device {
     bool prof = false;
     std::vector<prof_entry> prof_log;
     std::vector<hipEvent_t> prof_pool;
+    bool capturing = false;  // between arhip_graph_begin and arhip_graph_end
 };
 
 // Records a message for arhip_last_error() and returns `code`.

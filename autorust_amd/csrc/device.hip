@@ -49,6 +49,10 @@ static int prof_event(arhip_device *dev, hipEvent_t *e)
 
 int arhip_call_timer::begin()
 {
+    if (dev->capturing) {
+        if (wait) return arhip_fail(ARHIP_EINVAL, "a launch that waits cannot be recorded into a graph (pass wait = 0)");
+        return ARHIP_OK;
+    }
     if (dev->prof && kernel >= 0) {
         if (int rc = prof_event(dev, &p0)) return rc;
         if (int rc = prof_event(dev, &p1)) return rc;
@@ -61,6 +65,7 @@ int arhip_call_timer::begin()
 int arhip_call_timer::end()
 {
     ARHIP_HIP(hipGetLastError());
+    if (dev->capturing) return ARHIP_OK;
     if (p0) {
         ARHIP_HIP(hipEventRecord(p1, dev->stream));
         dev->prof_log.push_back({kernel, p0, p1});
@@ -295,6 +300,58 @@ extern "C" int arhip_kprof_collect(arhip_device *dev, int kernel, double *total_
     dev->prof_log.swap(keep);
     if (total_secs) *total_secs = tot;
     if (launches) *launches = n;
+    return ARHIP_OK;
+}
+
+// Launch graphs: the device-side counterpart of the reference's captured replay (Session capture
+// + `Jit::replay`, src/engine/jit.rs:186-195).  Typed launches issued with wait = 0 between begin
+// and end are recorded from the handle's stream into a HIP graph instead of running; launching
+// the graph replays them in order with one submission.  Nothing in this library records a
+// memset into a graph (buffers are cleared with a fill kernel).
+extern "C" int arhip_graph_begin(arhip_device *dev)
+{
+    ARHIP_DEV(dev);
+    ARHIP_REQUIRE(!dev->capturing, "arhip_graph_begin: a capture is already open");
+    ARHIP_HIP(hipStreamSynchronize(dev->stream));
+    ARHIP_HIP(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
+    dev->capturing = true;
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_graph_end(arhip_device *dev, void **graph_exec)
+{
+    ARHIP_DEV(dev);
+    ARHIP_REQUIRE(dev->capturing && graph_exec, "arhip_graph_end: no capture is open (or null out pointer)");
+    dev->capturing = false;
+    hipGraph_t g = nullptr;
+    ARHIP_HIP(hipStreamEndCapture(dev->stream, &g));
+    hipGraphExec_t ex = nullptr;
+    hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return arhip_fail(ARHIP_EHIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    *graph_exec = ex;
+    return ARHIP_OK;
+}
+
+extern "C" int arhip_graph_launch(arhip_device *dev, void *graph_exec, int wait, double *secs)
+{
+    ARHIP_DEV(dev);
+    ARHIP_REQUIRE(graph_exec && !dev->capturing, "arhip_graph_launch: null graph or capture still open");
+    arhip_call_timer t{dev, wait, secs};
+    if (int rc = t.begin()) return rc;
+    ARHIP_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, dev->stream));
+    return t.end();
+}
+
+extern "C" int arhip_graph_destroy(arhip_device *dev, void *graph_exec)
+{
+    ARHIP_DEV(dev);
+    if (!graph_exec) return ARHIP_OK;
+    ARHIP_HIP(hipStreamSynchronize(dev->stream));
+    ARHIP_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
     return ARHIP_OK;
 }
 

@@ -103,6 +103,23 @@ class Device:
         check(self.lib.arhip_kprof_collect(self.handle, kernel, ctypes.byref(s), ctypes.byref(n)))
         return s.value, n.value
 
+    # ---- launch graphs ----
+    def graph_begin(self):
+        check(self.lib.arhip_graph_begin(self.handle))
+
+    def graph_end(self):
+        g = ctypes.c_void_p()
+        check(self.lib.arhip_graph_end(self.handle, ctypes.byref(g)))
+        return g.value
+
+    def graph_launch(self, graph, wait=True):
+        s = ctypes.c_double()
+        check(self.lib.arhip_graph_launch(self.handle, graph, int(wait), ctypes.byref(s)))
+        return s.value if wait else None
+
+    def graph_destroy(self, graph):
+        check(self.lib.arhip_graph_destroy(self.handle, graph))
+
     # ---- generic launch (run_host_kernel) ----
     def module_load(self, image):
         m = ctypes.c_void_p()

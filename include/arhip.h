@@ -89,6 +89,17 @@ int arhip_timer_stop(arhip_device *dev, double *secs); /* records, waits, return
 int arhip_kprof_enable(arhip_device *dev, int on);
 int arhip_kprof_collect(arhip_device *dev, int kernel, double *total_secs, uint64_t *launches);
 
+/* ---- launch graphs: captured replay (`Session::capture_host` + `Jit::replay`,
+ *      src/engine/session.rs:138-146, src/engine/jit.rs:186-195) as one device submission.
+ *      Between begin and end, launches on this handle issued with wait = 0 are recorded, not
+ *      run; arhip_graph_launch replays them in order.  Buffers are captured by address: a replay
+ *      reads and writes the same memory as the recorded calls.  Allocation, copies and calls
+ *      that wait are not allowed inside a capture. ---- */
+int arhip_graph_begin(arhip_device *dev);
+int arhip_graph_end(arhip_device *dev, void **graph_exec);
+int arhip_graph_launch(arhip_device *dev, void *graph_exec, int wait, double *secs);
+int arhip_graph_destroy(arhip_device *dev, void *graph_exec);
+
 /* ---- generic host-kernel launch: `Compiled::run_host_kernel`,
  *      src/runtime/device.rs:383-402; argument encoding of
  *      src/runtime/ops_cuda.rs:930-1019 (`CudaProgram::call`) ----
