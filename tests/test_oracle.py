@@ -262,6 +262,82 @@ def test_sage_reference_properties():
     assert np.abs(approx - exact).max() < 0.5
 
 
+def _sage_inputs(seed, B, Hq, Hkv, N, D, bq, bk):
+    q = synth.normal(seed, (B, Hq, N, D))
+    k = synth.normal(seed + 1, (B, Hkv, N, D)) + 3 * synth.normal(seed + 3, (1, Hkv, 1, D))
+    v = synth.normal(seed + 2, (B, Hkv, N, D))
+    q8, sq = oracle.quant_blocks(q, bq)
+    k8, sk = oracle.quant_blocks(k, bk, sub=oracle.k_mean(k))
+    return q8, k8, sq, sk, v
+
+
+@pytest.mark.parametrize("bq,bk", [(1, 1), (128, 64), (32, 16)])
+@pytest.mark.parametrize("causal,use_mask,kv_len,hkv", [
+    (False, False, None, 2), (True, False, None, 2), (False, True, None, 2), (False, False, 100, 2),
+    (True, True, 77, 1), (True, False, 131, 4)])
+def test_sage_reference_against_torch_ops(bq, bk, causal, use_mask, kv_len, hkv):
+    """Every branch and rounding point of the quantised-attention emulation
+    (tests/sage_int8.rs:33-76, src/runtime/cuda_flash_sage.rs:315-340), re-derived with torch
+    tensor ops: integer matmul, the dequantisation factor in the kernel's order, additive mask,
+    causal triangle, key length, fp32 softmax numerator, bf16 P and V, division by the sum of the
+    unrounded probabilities."""
+    torch = pytest.importorskip("torch")
+    B, Hq, N, D = 1, 4, 150, 64
+    q8, k8, sq, sk, v = _sage_inputs(91, B, Hq, hkv, N, D, bq, bk)
+    mask = synth.normal(95, (N, N)).astype(np.float32) if use_mask else None
+    scale = np.float32(1.0) / np.sqrt(np.float32(D))
+    rep = Hq // hkv
+    bf = lambda t: t.to(torch.bfloat16).to(torch.float32)
+    tq = torch.from_numpy(q8).to(torch.int64)
+    tk = torch.from_numpy(np.repeat(k8, rep, 1)).to(torch.int64)
+    acc = tq @ tk.transpose(-1, -2)                                   # exact integers
+    fq = torch.from_numpy(np.repeat(sq, bq, -1)[..., :N])             # scale of row i: sq[i // bq]
+    fk = torch.from_numpy(np.repeat(np.repeat(sk, rep, 1), bk, -1)[..., :N])
+    a = (fq[..., :, None] * fk[..., None, :]) * torch.tensor(scale)   # (sq * sk) * scale, fp32
+    s = acc.to(torch.float32) * a
+    if mask is not None:
+        s = s + torch.from_numpy(mask)
+    dead = torch.zeros(N, N, dtype=torch.bool)
+    if causal:
+        dead |= torch.ones(N, N, dtype=torch.bool).triu(1)
+    if kv_len is not None:
+        dead[:, kv_len:] = True
+    s = s.masked_fill(dead, float("-inf"))
+    p = torch.exp(s - s.max(-1, keepdim=True).values)
+    tv = bf(torch.from_numpy(np.repeat(v, rep, 1)))
+    want = ((bf(p).double() @ tv.double()).float() / p.sum(-1, keepdim=True)).numpy()
+    kl = None if kv_len is None else np.array([kv_len], np.int32)
+    got = oracle.sage(q8, k8, sq, sk, v, bq, bk, mask=mask, causal=causal, kv_len=kl)
+    # fp32 output: only summation order and libm-vs-torch exp differ (a dropped bf16 rounding of P
+    # or V moves the result by ~1e-3, a wrong mask edge by O(0.1))
+    assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+    got_b = oracle.sage(q8, k8, sq, sk, v, bq, bk, mask=mask, causal=causal, kv_len=kl, round_out=True)
+    assert np.array_equal(got_b, oracle.bf16_round(got))
+
+
+def test_sage_reference_closed_forms():
+    B, Hq, Hkv, N, D, bq, bk = 1, 2, 2, 96, 64, 32, 16
+    q8, k8, sq, sk, v = _sage_inputs(101, B, Hq, Hkv, N, D, bq, bk)
+    full = oracle.sage(q8, k8, sq, sk, v, bq, bk, causal=True)
+    # a key length is the truncated problem (L a multiple of both block sizes keeps the scale
+    # indices aligned); rows at or past L still attend to keys < L only
+    L = 64
+    cut = oracle.sage(q8[:, :, :L], k8[:, :, :L], sq[:, :, :L // bq], sk[:, :, :L // bk], v[:, :, :L], bq, bk)
+    got = oracle.sage(q8, k8, sq, sk, v, bq, bk, kv_len=np.array([L], np.int32))
+    assert np.array_equal(got[:, :, :L], cut)
+    # a row subset is the same rows of the full result
+    rows = np.array([0, 1, 31, 32, 63, 95], np.int32)
+    assert np.array_equal(oracle.sage(q8, k8, sq, sk, v, bq, bk, causal=True, rows=rows), full[:, :, rows])
+    # causal row 0 sees key 0 only: the output is bf16(v[0]) whatever the logits are
+    assert np.array_equal(full[:, :, 0], oracle.bf16_round(v[:, :, 0]))
+    # a mask of -inf above the diagonal is the causal flag
+    tri = np.where(np.triu(np.ones((N, N), bool), 1), -np.inf, 0).astype(np.float32)
+    assert np.array_equal(oracle.sage(q8, k8, sq, sk, v, bq, bk, mask=tri), full)
+    # a constant added to every logit of a row cancels (up to fp32 rounding of s + c)
+    shifted = oracle.sage(q8, k8, sq, sk, v, bq, bk, causal=True, mask=np.full((N, N), 0.5, np.float32))
+    assert np.abs(shifted - full).max() < 1e-4
+
+
 def test_cpu_baseline_matches_oracle():
     B, H, N, D = 1, 3, 197, 64
     q, k, v = synth.normal(71, (B, H, N, D)), synth.normal(72, (B, H, N, D)), synth.normal(73, (B, H, N, D))
