@@ -97,8 +97,7 @@ def test_decoder_bf16_causal_key_lengths(dev):
     assert steps <= 3
 
 
-def _sage_config(dev, B, H, N, D, causal, sigma, outliers, seed, rows_per_head_extra=()):
-    bq, bk = 128, 64
+def _sage_config(dev, B, H, N, D, causal, sigma, outliers, seed, rows_per_head_extra=(), bq=128, bk=64, light=False):
     q = synth.normal(seed + 1, (B, H, N, D))
     k = synth.normal(seed + 2, (B, H, N, D))
     k += np.float32(sigma) * synth.normal(seed + 4, (1, H, 1, D))
@@ -112,6 +111,7 @@ def _sage_config(dev, B, H, N, D, causal, sigma, outliers, seed, rows_per_head_e
                 hit = synth.uniform(sd, m, o) < outliers
                 flat[o:o + m][hit] *= np.float32(20.0)
     nqb, nkb = N // bq, N // bk
+    rows = _rows(N, extra=rows_per_head_extra)
     with Bufs(dev) as bufs:
         dq, dk = bufs.put(synth.to_bf16_bits(q)), bufs.put(synth.to_bf16_bits(k))
         dv = bufs.put(synth.to_bf16_bits(v))
@@ -127,20 +127,23 @@ def _sage_config(dev, B, H, N, D, causal, sigma, outliers, seed, rows_per_head_e
         g_q8, g_k8 = q8.copyout(np.int8, q.shape), k8.copyout(np.int8, k.shape)
         g_sq, g_sk = sq.copyout(np.float32, (B, H, nqb)), sk.copyout(np.float32, (B, H, nkb))
         g_mean = mean.copyout(np.float32, (B, H, D))
-        # raw int32 logits of one tile (on/below the diagonal) through the debug export
-        dbg = bufs.new(32 * 64 * 4)
         sel = (B * H - 1, (N - 1) // 32, ((N - 1) // 64) // 2)
-        o32 = bufs.new(q.size * 4, zero=False)
-        dev.sage_fwd(q8, k8, sq, sk, dv, o32, B, H, H, N, D, bq, bk, out_dtype=F32, causal=causal, dbg_logits=dbg,
-                     dbg_sel=sel)
-        logits = dbg.copyout(np.int32, (32, 64))
-        o32.free()
-        # V = 1 -> 1 for every row
-        ones = bufs.put(np.full(q.size, 0x3F80, np.uint16))
-        dev.sage_fwd(q8, k8, sq, sk, ones, do, B, H, H, N, D, bq, bk, out_dtype=BF16, causal=causal)
-        unit = synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
-    err = max_abs(unit, 1.0)
-    assert err <= 2.0 ** -7
+        logits = unit = None
+        if not light:
+            # raw int32 logits of one tile (on/below the diagonal) through the debug export
+            dbg = bufs.new(32 * 64 * 4)
+            o32 = bufs.new(q.size * 4, zero=False)
+            dev.sage_fwd(q8, k8, sq, sk, dv, o32, B, H, H, N, D, bq, bk, out_dtype=F32, causal=causal, dbg_logits=dbg,
+                         dbg_sel=sel)
+            logits = dbg.copyout(np.int32, (32, 64))
+            o32.free()
+            # V = 1 -> 1 for every row
+            ones = bufs.put(np.full(q.size, 0x3F80, np.uint16))
+            dev.sage_fwd(q8, k8, sq, sk, ones, do, B, H, H, N, D, bq, bk, out_dtype=BF16, causal=causal)
+            unit = synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+    if unit is not None:
+        err = max_abs(unit, 1.0)
+        assert err <= 2.0 ** -7
 
     # quantised tensors, scales and the K mean: bit-exact on the full tensors
     qb, kb = oracle.bf16_round(q), oracle.bf16_round(k)
@@ -152,38 +155,68 @@ def _sage_config(dev, B, H, N, D, causal, sigma, outliers, seed, rows_per_head_e
     assert all(ok.values()), ok
     b, h = divmod(sel[0], H)
     i0, j0 = sel[1] * 32, sel[2] * 64
-    logits_ok = np.array_equal(logits, oracle.logits_i32(w_q8[b, h], w_k8[b, h], i0, i0 + 32, j0, j0 + 64))
-    assert logits_ok
+    if logits is not None:
+        logits_ok = np.array_equal(logits, oracle.logits_i32(w_q8[b, h], w_k8[b, h], i0, i0 + 32, j0, j0 + 64))
+        assert logits_ok
 
-    rows = _rows(N, extra=rows_per_head_extra)
     want = oracle.sage(w_q8, w_k8, w_sq, w_sk, v, bq, bk, causal=causal, rows=rows, round_out=True)
     truth = oracle.sdpa_f64(q, k, v, causal=causal, rows=rows)
-    return got[:, :, rows], want, truth, rows
+    # What the quantiser itself answers: float64 attention on the dequantised tensors q8*sq and
+    # k8*sk (the subtracted K mean shifts every logit of a row by the same amount and cancels).
+    # The difference between this and `truth` is the quantiser's error; the difference between
+    # the kernel and this is the kernel's (bf16 P, V and output).
+    qd = w_q8[:, :, rows].astype(np.float32) * np.repeat(w_sq, bq, -1)[:, :, rows, None]
+    kd = w_k8.astype(np.float32)
+    kd *= np.repeat(w_sk, bk, -1)[..., None]
+    qfull = np.zeros((B, H, N, D), np.float32)
+    qfull[:, :, rows] = qd
+    dequant = oracle.sdpa_f64(qfull, kd, v, causal=causal, rows=rows)
+    return got[:, :, rows], want, truth, dequant
 
 
 def test_sage_int8_s8192(dev):
     """configs[3]: B=4 H=32 S=8192 D=128, K bias sigma 3, Q blocks of 128, K blocks of 64, smoothing."""
-    got, want, truth, _ = _sage_config(dev, 4, 32, 8192, 128, False, 3.0, 0.0, 4000)
+    got, want, truth, dequant = _sage_config(dev, 4, 32, 8192, 128, False, 3.0, 0.0, 4000)
     steps = bf16_ulps(got, want)                  # the kernel against the emulation of its own arithmetic
     assert steps <= 3
     err = max_abs(got, truth)
     assert err <= 2e-2
+    assert max_rel1(got, dequant) <= 2e-2
+
+
+def _within(got, truth, tol=2e-2):
+    return float((np.abs(got - truth) <= tol).mean())
 
 
 def test_sage_int8_causal_long_context(dev):
-    """configs[4]: B=1 H=64 S=32768 D=128 causal, K bias sigma 5, 1% of Q/K entries x20."""
-    got, want, truth, rows = _sage_config(dev, 1, 64, 32768, 128, True, 5.0, 0.01, 5000, rows_per_head_extra=(4096, 16383))
+    """configs[4]: B=1 H=64 S=32768 D=128 causal, K bias sigma 5, 1% of Q/K entries x20.
+
+    The <= 2e-2 bound against the exact result is NOT met on this configuration, by the kernel
+    and by the CPU emulation alike: the x20 outliers stretch the int8 range of every block they
+    fall in and make the logits so large that the softmax is nearly one-hot, so one quantisation
+    step flips the winning key.  The test makes that attribution explicit: the kernel must be
+    within 2e-2 of the float64 attention of the DEQUANTISED tensors everywhere (so whatever is
+    missing against the exact result is the prescribed quantiser's), and the shortfall against
+    the exact result is pinned as a stated fraction, not hidden behind a median."""
+    cfg = (dev, 1, 64, 32768, 128, True, 5.0, 0.01, 5000)
+    got, want, truth, dequant = _sage_config(*cfg, rows_per_head_extra=(4096, 16383))
     steps = bf16_ulps(got, want)                  # the kernel against the emulation of its own arithmetic
     assert steps <= 3
-    # Against the exact result: nowhere may the kernel be worse than the emulation by more than
-    # the bf16 output step.
-    err_g = np.abs(got - truth).max(axis=(0, 1, 3))
-    err_w = np.abs(want - truth).max(axis=(0, 1, 3))
-    worse = float((err_g - err_w).max())
-    assert worse <= 1.6e-2
-    # Measured on this configuration: median 3.4e-3, 63 % of the sampled outputs within 2e-2,
-    # maximum 4.66 -- for the kernel and for the emulation alike.  The x20 outliers make the
-    # logits so large that the softmax is nearly one-hot, and an int8 step then flips the winner:
-    # that error belongs to the quantiser the configuration prescribes, not to the kernel.
-    med = float(np.median(np.abs(got - truth)))
-    assert med <= 2e-2
+    assert max_rel1(got, dequant) <= 2e-2         # the kernel against the quantiser's own answer
+    assert max_rel1(want, dequant) <= 2e-2
+    frac_blocks = _within(got, truth)
+    worst = max_abs(got, truth)
+    print("cfg5 per-block (128/64): %.3f of sampled outputs within 2e-2 of the exact result, median %.2e, max %.2f"
+          % (frac_blocks, float(np.median(np.abs(got - truth))), worst))
+    # measured: 0.63 within the bound, median 3.4e-3, maximum 4.66 (an output is a convex
+    # combination of V rows, so the error is bounded by 2 max|v|)
+    assert frac_blocks >= 0.55 and worst <= 2 * 5.7
+    assert abs(_within(want, truth) - frac_blocks) <= 0.01   # the emulation misses it just the same
+    # the reference's own granularity (one scale per row / per key, cuda_flash_sage.rs:209-222)
+    got1, want1, truth1, dequant1 = _sage_config(*cfg, rows_per_head_extra=(4096, 16383), bq=1, bk=1, light=True)
+    assert bf16_ulps(got1, want1) <= 3
+    assert max_rel1(got1, dequant1) <= 2e-2
+    frac_rows = _within(got1, truth1)
+    print("cfg5 per-row (1/1): %.3f within 2e-2, median %.2e, max %.2f"
+          % (frac_rows, float(np.median(np.abs(got1 - truth1))), max_abs(got1, truth1)))
+    assert frac_rows >= frac_blocks - 0.02        # finer scales do not hurt; they do not reach the bound either
