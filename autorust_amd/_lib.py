@@ -63,6 +63,9 @@ SIGNATURES = {
     "arhip_sage_quant_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "arhip_sage_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),
+    "arhip_sage_quant_static_limit": (c_size_t, []),
+    "arhip_sage_quant_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),
     "arhip_cast_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, _pd]),
     "arhip_sage_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_float,

@@ -66,4 +66,7 @@ struct arhip_call_timer {
 
 void arhip_note_selected(int kernel);
 
+// Resolves the device address of the built-in Sage scratch array for the current device.
+int arhip_static_scratch_setup(int ordinal);
+
 static inline bool arhip_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -125,6 +125,10 @@ extern "C" int arhip_open(int ordinal, arhip_device **out)
         delete d;
         return arhip_fail(ARHIP_EHIP, "arhip_open: stream/event creation failed: %s", hipGetErrorString(e));
     }
+    if (int rc = arhip_static_scratch_setup(ordinal)) {
+        (void)arhip_close(d);
+        return rc;
+    }
     *out = d;
     return ARHIP_OK;
 }

@@ -11,7 +11,21 @@
 // the int8 tensors and scales are bit-reproducible on the CPU.
 #include "arhip_internal.h"
 
+#include <mutex>
+
 #pragma clang fp contract(off)
+
+// Scratch of arhip_sage_quant_static, resident on the device: the partial channel sums of the K
+// mean.  Each GPU the library runs on holds its own copy until the process ends.
+constexpr size_t STATIC_SCRATCH_FLOATS = (size_t)4 << 20;  // 16 MiB
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+// Device address of `scratch` per GPU ordinal, resolved once per device in
+// arhip_static_scratch_setup.  In host code the array's name is only a stand-in for the symbol,
+// not a device address: kernels, copies and fills always get the resolved pointer.
+constexpr int MAX_DEVICES = 64;
+static float *g_scratch_ptr[MAX_DEVICES];
+static std::mutex g_scratch_mutex;
 
 namespace {
 
@@ -219,9 +233,22 @@ extern "C" size_t arhip_sage_quant_workspace(int64_t B, int64_t H, int64_t N, in
     return (size_t)(B * H * nchunk * D) * sizeof(float);
 }
 
-extern "C" int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, float *scales, float *mean,
-                                void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
-                                int64_t block, int dtype, int smooth, int wait, double *secs)
+// Called by arhip_open with the device current: resolves this GPU's copy of `scratch`.
+int arhip_static_scratch_setup(int ordinal)
+{
+    ARHIP_REQUIRE(ordinal >= 0 && ordinal < MAX_DEVICES, "device ordinal %d beyond %d", ordinal, MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[ordinal] != nullptr) return ARHIP_OK;
+    float *ptr = nullptr;
+    ARHIP_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+    ARHIP_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null scratch address for device %d", ordinal);
+    g_scratch_ptr[ordinal] = ptr;
+    return ARHIP_OK;
+}
+
+static int sage_quant_impl(arhip_device *dev, const void *x, int8_t *x8, float *scales, float *mean,
+                           void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
+                           int64_t block, int dtype, int smooth, int wait, double *secs, int prof_kernel)
 {
     ARHIP_REQUIRE(dev != nullptr, "arhip_sage_quant: null device");
     ARHIP_REQUIRE(x && x8 && scales, "arhip_sage_quant: null pointer");
@@ -237,7 +264,7 @@ extern "C" int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, fl
     const int nchunk = (int)((N + MEAN_CHUNK - 1) / MEAN_CHUNK);
     const dim3 qgrid((unsigned)nblk, (unsigned)(B * H));
     arhip_call_timer t{dev, wait, secs};
-    t.kernel = ARHIP_K_SAGE_QUANT;
+    t.kernel = prof_kernel;
     if (int rc = t.begin()) return rc;
     if (smooth) {
         const int cpb = 256 / (int)(D / 8);  // chunks per workgroup
@@ -287,6 +314,41 @@ extern "C" int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, fl
     }
     arhip_note_selected(ARHIP_K_SAGE_QUANT);
     return t.end();
+}
+
+extern "C" int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, float *scales, float *mean,
+                                void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
+                                int64_t block, int dtype, int smooth, int wait, double *secs)
+{
+    return sage_quant_impl(dev, x, x8, scales, mean, workspace, B, H, N, D, block, dtype, smooth, wait, secs,
+                           ARHIP_K_SAGE_QUANT);
+}
+
+extern "C" size_t arhip_sage_quant_static_limit(void) { return STATIC_SCRATCH_FLOATS * sizeof(float); }
+
+// The same kernels with the partial sums in the library's own device array: no allocation here,
+// none asked of the caller.  The launches are not entered in the per-kernel profile log, which
+// would create events.  Every chunk the final reduction reads is written by the partial-sum
+// kernel of the same call first, so nothing has to be cleared between calls; two calls that
+// overlap on one GPU (different streams or handles) race on the array.
+extern "C" int arhip_sage_quant_static(arhip_device *dev, const void *x, int8_t *x8, float *scales, float *mean,
+                                       int64_t B, int64_t H, int64_t N, int64_t D,
+                                       int64_t block, int dtype, int smooth, int wait, double *secs)
+{
+    ARHIP_REQUIRE(dev != nullptr, "arhip_sage_quant_static: null device");
+    float *ws = nullptr;
+    if (smooth) {
+        const size_t need = arhip_sage_quant_workspace(B, H, N, D);
+        if (need > STATIC_SCRATCH_FLOATS * sizeof(float))
+            return arhip_fail(ARHIP_EINVAL,
+                              "arhip_sage_quant_static: B*H*ceil(N/64)*D*4 = %zu bytes of partial sums exceed the "
+                              "built-in %zu-byte scratch; use arhip_sage_quant with a caller workspace",
+                              need, STATIC_SCRATCH_FLOATS * sizeof(float));
+        ARHIP_REQUIRE(dev->ordinal >= 0 && dev->ordinal < MAX_DEVICES && g_scratch_ptr[dev->ordinal] != nullptr,
+                      "arhip_sage_quant_static: the scratch address of device %d was not resolved at open", dev->ordinal);
+        ws = g_scratch_ptr[dev->ordinal];
+    }
+    return sage_quant_impl(dev, x, x8, scales, mean, ws, B, H, N, D, block, dtype, smooth, wait, secs, -1);
 }
 
 extern "C" int arhip_cast_bf16(arhip_device *dev, const float *x, uint16_t *y, int64_t n, int wait, double *secs)

@@ -191,6 +191,14 @@ class Device:
                                         ctypes.byref(s)))
         return s.value if wait else None
 
+    def sage_quant_static(self, x, x8, scales, B, H, N, D, block, dtype, mean=None, smooth=False, wait=True):
+        """sage_quant with the partial sums in the library's own device array (no allocation)."""
+        s = ctypes.c_double()
+        check(self.lib.arhip_sage_quant_static(self.handle, self._ptr(x), self._ptr(x8), self._ptr(scales),
+                                               self._ptr(mean), B, H, N, D, block, dtype, int(smooth), int(wait),
+                                               ctypes.byref(s)))
+        return s.value if wait else None
+
     def cast_bf16(self, x, y, n, wait=True):
         s = ctypes.c_double()
         check(self.lib.arhip_cast_bf16(self.handle, self._ptr(x), self._ptr(y), n, int(wait), ctypes.byref(s)))

@@ -179,6 +179,20 @@ int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, float *scales
                      void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
                      int64_t block, int dtype, int smooth, int wait, double *secs);
 
+/* arhip_sage_quant_static: arhip_sage_quant without a workspace argument and without any
+ *   allocation inside the call.  It has no counterpart in the reference; it is for callers that
+ *   cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
+ *   that forbid hipMalloc.  The partial sums of the K mean go to a device array inside the
+ *   library (16 MiB per GPU, resolved when the device is opened), so smoothing is limited to
+ *   arhip_sage_quant_workspace(B,H,N,D) <= arhip_sage_quant_static_limit() bytes; larger shapes
+ *   are rejected with ARHIP_EINVAL.  Same kernels and bit-identical results as arhip_sage_quant.
+ *   All calls on one GPU share the array: calls that overlap in time on one GPU race.  The
+ *   launches are not entered in the arhip_kprof_* log. */
+size_t arhip_sage_quant_static_limit(void);
+int arhip_sage_quant_static(arhip_device *dev, const void *x, int8_t *x8, float *scales, float *mean,
+                            int64_t B, int64_t H, int64_t N, int64_t D,
+                            int64_t block, int dtype, int smooth, int wait, double *secs);
+
 /* arhip_cast_bf16: f32 -> bf16 round-to-nearest-even of n elements (the V
  *   operand of the Sage kernel: cuda_flash_sage.rs:99-103, 257-262). */
 int arhip_cast_bf16(arhip_device *dev, const float *x, uint16_t *y, int64_t n, int wait, double *secs);
