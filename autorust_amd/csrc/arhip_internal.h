@@ -32,6 +32,7 @@ struct arhip_device {
     std::vector<prof_entry> prof_log;
     std::vector<hipEvent_t> prof_pool;
     bool capturing = false;  // between arhip_graph_begin and arhip_graph_end
+    int attn_waves = 0;      // ARHIP_ATTN_WAVES at open (0: choose by shape)
 };
 
 // Records a message for arhip_last_error() and returns `code`.

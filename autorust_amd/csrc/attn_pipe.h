@@ -1,0 +1,450 @@
+// Fused attention forward for long sequences on gfx950: the software-pipelined variant of
+// attn_fwd_kernel (attn_fwd.h) for launches without an additive mask, per-key scales or the
+// logits export.  Same arithmetic, same MFMA decomposition (S^T = K . Q^T, one query per lane,
+// O^T += V^T . P^T), different plumbing:
+//
+//   HBM -> LDS   K and V tiles of 64 keys go straight to LDS (buffer_load ... lds, 16 bytes per
+//                lane, no registers in between), four stages deep, so a tile is requested two
+//                iterations before its first use.  Rows past the last visible key come back as
+//                zeros from the buffer bounds check; nothing is clamped or branched on.
+//   LDS layout   A transfer writes 64 x 16 bytes to consecutive addresses, so rows cannot be padded.
+//                Rows are cut into 64-byte pieces and stored [piece][row][64 B]; inside a block of
+//                16 rows the four 16-byte chunks of a row are permuted with chunk ^= (row / 4) % 4.
+//                The permutation is applied to the SOURCE address a lane fetches, and the operand
+//                reads (ds_read_b128 for K, ds_read_b64_tr_b16 for V^T) then hit 16 distinct
+//                16-byte bank groups per 16 lanes.
+//   wave stream  A wave issues in order, and a matrix instruction keeps the matrix pipe busy for
+//                8 passes during which the wave may issue independent vector instructions.  The
+//                instruction stream therefore interleaves the two pipes itself, one 32-key block
+//                ahead:
+//                  R1(j)  S = K(j+1) . Q^T         (MFMA)
+//                  R2(j)  O^T += V(j)^T . P(j)^T   (MFMA)  |  P(j+1) = exp2(S c - m), row sum,
+//                                                             bf16 pack                  (VALU)
+//                V(j) fragments are requested at the start of R1(j), K(j+2) fragments at its end.
+//                Carried from block to block: P(j) packed, its row sum, the K(j+1) fragments.
+//   reference    lazy exponent reference as in attn_fwd.h; it is checked right after R2, while S
+//                still holds the raw logits (the rare case recomputes P from them).
+//   masked tiles (causal diagonal, key-length edge) run block by block without look-ahead.
+//
+// 8 waves of 32 queries per workgroup, two waves per SIMD.
+#pragma once
+
+#include "attn_fwd.h"
+
+namespace arhip {
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
+template <int N>
+__device__ __forceinline__ void wait_vmem_le()
+{
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <int D, bool CAUSAL, int MODE, bool OUT_F32>
+__global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
+{
+    constexpr int NW = 8;
+    constexpr int BQ = NW * 32;
+    constexpr int QK_BYTES = (MODE == MODE_I8) ? 1 : 2;
+    constexpr int KP = D * QK_BYTES / 64;  // 64-byte pieces per K row
+    constexpr int VP = D * 2 / 64;         // 64-byte pieces per V row
+    constexpr int K_TILE = KP * 4096;      // [piece][64 rows][64 B]
+    constexpr int V_TILE = VP * 4096;
+    constexpr int STAGE = K_TILE + V_TILE;
+    constexpr int NSTAGE = 4;
+    constexpr int XFERS = (KP + VP) * 4;          // 1 KB transfers per tile
+    constexpr int XPW = (XFERS + NW - 1) / NW;    // at most this many per wave
+    constexpr int XPW_MIN = XFERS / NW;           // at least this many per wave
+    constexpr int KSTEPS = (MODE == MODE_I8) ? D / 32 : D / 16;
+    constexpr int DB = D / 32;
+    static_assert(KP >= 1 && XFERS >= NW, "tile too small for 8 waves");
+
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[NSTAGE * STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int i32 = lane & 31;
+    const int h = lane >> 5;
+
+    // workgroup -> (head, query tile), as in attn_fwd_kernel
+    int wg = blockIdx.x;
+    int bh, qt;
+    if (CAUSAL && p.lpt) {
+        const int nbh = p.total / p.nq;
+        qt = p.nq - 1 - wg / nbh;
+        bh = wg % nbh;
+    } else {
+        if ((p.total & 7) == 0) wg = (wg & 7) * (p.total >> 3) + (wg >> 3);
+        bh = wg / p.nq;
+        qt = wg - bh * p.nq;
+        if (CAUSAL) qt = p.nq - 1 - qt;
+    }
+    const int b = bh / p.Hq;
+    const int head = bh - b * p.Hq;
+    const int kvh = head / (p.Hq / p.Hkv);
+    const int kv_bh = b * p.Hkv + kvh;
+    const int N = p.N;
+    const int qblk = qt * BQ;
+    const int wq0 = qblk + wave * 32;
+    const int q_row = wq0 + i32;
+
+    int kvl = N;
+    if (p.kv_len) {
+        kvl = p.kv_len[b];
+        kvl = kvl < 0 ? 0 : (kvl > N ? N : kvl);
+    }
+    int kend = kvl;
+    if (CAUSAL) kend = min(kend, min(N, qblk + BQ));
+    const int ntiles = (kend + BK - 1) / BK;
+    const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / BK + 1) : ntiles;
+
+    // ---- buffer resources over this head's K and V: offsets past kend rows read as zero ----
+    const size_t kv_off = (size_t)b * p.ks[0] + (size_t)kvh * p.ks[1];
+    const uint32_t k_rowb = (uint32_t)p.ks[2] * QK_BYTES;  // bytes between consecutive keys
+    const uint32_t v_rowb = (uint32_t)p.ks[2] * 2;
+    // raw buffer descriptor: base address, stride 0, size in bytes, 32-bit untyped data
+    auto make_rsrc = [](const void *base, uint32_t bytes) __attribute__((always_inline)) -> i32x4 {
+        const uint64_t a = (uint64_t)(uintptr_t)base;
+        i32x4 r;
+        r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+        r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32) & 0xffff);
+        r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+        r[3] = 0x00020000;
+        return r;
+    };
+    const i32x4 k_rsrc = make_rsrc((const unsigned char *)p.k + kv_off * QK_BYTES, (uint32_t)kend * k_rowb);
+    const i32x4 v_rsrc = make_rsrc(p.v + kv_off, (uint32_t)kend * v_rowb);
+
+    // transfer x of a tile (x = wave + 8 j): rows 16 g .. 16 g + 15 of piece pc of K (x < 4 KP) or V;
+    // lane l fetches row 16 g + l / 4, chunk (l % 4) ^ ((l / 16) % 4) of that piece
+    uint32_t xoff[XPW];
+#pragma unroll
+    for (int j = 0; j < XPW; ++j) {
+        const int x = wave + NW * j;
+        const bool is_k = x < KP * 4;
+        const int xl = is_k ? x : x - KP * 4;
+        const int pc = xl >> 2, g = xl & 3;
+        const int r = lane >> 2;
+        const int c = (lane & 3) ^ ((r >> 2) & 3);
+        xoff[j] = (uint32_t)(16 * g + r) * (is_k ? k_rowb : v_rowb) + pc * 64 + c * 16;
+    }
+    // The transfers are written as inline assembly on purpose: the compiler makes every LDS read
+    // wait for all outstanding transfers it knows of (it cannot tell the stages apart), which
+    // would put the whole memory latency in front of every tile.  Here the waits are explicit
+    // (wait_vmem_le before the barrier that publishes a tile).  m0 holds the LDS destination;
+    // one wait state is required between writing m0 and the transfer.
+    auto issue_tile = [&](int tile, int stage) __attribute__((always_inline)) {
+        const uint32_t dst = (uint32_t)(uintptr_t)(lds_ptr_t)lds + stage * STAGE;
+#pragma unroll
+        for (int j = 0; j < XPW; ++j) {
+            const int x = wave + NW * j;
+            if (XFERS % NW == 0 || x < XFERS) {
+                // the tile offset goes into the per-lane offset: the scalar offset operand of a
+                // buffer access is not covered by the bounds check
+                const bool is_k = x < KP * 4;
+                const uint32_t off = xoff[j] + (uint32_t)tile * BK * (is_k ? k_rowb : v_rowb);
+                const i32x4 rsrc = is_k ? k_rsrc : v_rsrc;
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                             :
+                             : "s"(dst + x * 1024), "v"(off), "s"(rsrc)
+                             : "memory", "m0");
+            }
+        }
+    };
+
+    uint4 qreg[KSTEPS];  // Q operand (loaded in the prologue below)
+
+    // ---- LDS operand addresses (relative to a stage) ----
+    // K fragment of step st: row 32 blk + i32, bytes 32 st + 16 h .. +15, i.e. piece st / 2, chunk
+    // 2 (st % 2) + h, stored at chunk position (2 (st % 2) + h) ^ ((i32 / 4) % 4)
+    const int k_t = h ^ ((i32 >> 2) & 3);
+    const int k_row = (i32 & 15) * 64 + (i32 >> 4) * 1024;
+    const int k_addr[2] = {k_row + k_t * 16, k_row + (k_t ^ 2) * 16};
+    // V^T fragment: this lane's corner of the transposing reads is key row 4 h + (lane % 16) / 4
+    // (+ 8 for the second read), channels 16 ((lane / 16) % 2) + 4 (lane % 4) .. + 3 of a 32-channel
+    // block, i.e. chunk 2 ((lane / 16) % 2) + (lane % 4) / 2, byte 8 (lane % 2) inside it
+    const int v_r0 = 4 * h + ((lane & 15) >> 2);
+    const int v_c = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+    const int v_addr[2] = {K_TILE + v_r0 * 64 + (v_c ^ h) * 16 + (lane & 1) * 8,
+                           K_TILE + (v_r0 + 8) * 64 + (v_c ^ (h + 2)) * 16 + (lane & 1) * 8};
+
+    typedef typename std::conditional<MODE == MODE_I8, i32x16, f32x16>::type acc_t;
+    f32x16 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+    float m_run = NEG_SENTINEL;
+    float l_run = 0.f;
+    float sq_lane = 1.f;
+    const int nkb = (MODE == MODE_I8) ? (N + p.bk - 1) / p.bk : 0;
+    if (MODE == MODE_I8) {
+        const int nqb = (N + p.bq - 1) / p.bq;
+        sq_lane = p.sq[(size_t)bh * nqb + min(q_row, N - 1) / p.bq];
+    }
+    const float c_scale = p.scale * LOG2E;
+    const int last_tile = (N - 1) / BK;
+    // exponent factor of the keys of tile t: scale log2(e), times sq sk for int8
+    // (s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322)
+    auto tile_c = [&](int t) __attribute__((always_inline)) -> float {
+        if constexpr (MODE == MODE_I8) {
+            const float f = p.sk[(size_t)kv_bh * nkb + (min(t, last_tile) >> p.bk_tile_shift)];
+            return ((sq_lane * f) * p.scale) * LOG2E;
+        } else {
+            return c_scale;
+        }
+    };
+
+    uint4 kf[KSTEPS];
+    uint2 vf[DB][2][2];
+    auto load_kf = [&](const unsigned char *st, int blk) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+            kf[s] = *(const uint4 *)(st + k_addr[s & 1] + (s >> 1) * 4096 + blk * 2048);
+    };
+    auto load_vf = [&](const unsigned char *st, int blk) __attribute__((always_inline)) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                vf[db][ks][0] = lds_read_tr16(st + v_addr[0] + db * 4096 + (blk * 2 + ks) * 1024);
+                vf[db][ks][1] = lds_read_tr16(st + v_addr[1] + db * 4096 + (blk * 2 + ks) * 1024);
+            }
+    };
+    auto mfma_qk = [&]() __attribute__((always_inline)) -> acc_t {
+        acc_t s;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0;
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            if constexpr (MODE == MODE_I8)
+                s = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kf[st]), __builtin_bit_cast(i32x4, qreg[st]), s, 0, 0, 0);
+            else
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s, 0, 0, 0);
+        }
+        return s;
+    };
+    auto mfma_pv = [&](const uint4 (&pb)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const uint4 a = make_uint4(vf[db][ks][0].x, vf[db][ks][0].y, vf[db][ks][1].x, vf[db][ks][1].y);
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                                   __builtin_bit_cast(bf16x8, pb[ks]), oacc[db], 0, 0, 0);
+            }
+    };
+    auto row_sum = [&](const float (&x)[16]) __attribute__((always_inline)) {
+        // over the unrounded probabilities (src/runtime/cuda_flash_bf16.rs:365-377)
+        float rs0 = (x[0] + x[1]) + (x[2] + x[3]), rs1 = (x[8] + x[9]) + (x[10] + x[11]);
+        rs0 += (x[4] + x[5]) + (x[6] + x[7]);
+        rs1 += (x[12] + x[13]) + (x[14] + x[15]);
+        return rs0 + rs1;
+    };
+    auto pack = [&](const float (&x)[16], uint4 (&pb)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            pb[ks].x = pack_bf16x2(x[ks * 8 + 0], x[ks * 8 + 1]);
+            pb[ks].y = pack_bf16x2(x[ks * 8 + 2], x[ks * 8 + 3]);
+            pb[ks].z = pack_bf16x2(x[ks * 8 + 4], x[ks * 8 + 5]);
+            pb[ks].w = pack_bf16x2(x[ks * 8 + 6], x[ks * 8 + 7]);
+        }
+    };
+    auto move_reference = [&](float mx) __attribute__((always_inline)) {
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+    };
+    // probabilities of an unmasked block against the current reference, the scale folded into the
+    // exponent; row sum over the unrounded values (src/runtime/cuda_flash_bf16.rs:365-377); bf16
+    // pack in the B-operand layout.  Done in two halves of 8 keys so that only 8 values are live.
+    auto exp_pack = [&](const acc_t &s, float c, uint4 (&pb)[2], float &rs) __attribute__((always_inline)) {
+        float half[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            float x[8];
+#pragma unroll
+            for (int r = 0; r < 8; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[ks * 8 + r], c, -m_run));
+            half[ks] = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+            pb[ks].x = pack_bf16x2(x[0], x[1]);
+            pb[ks].y = pack_bf16x2(x[2], x[3]);
+            pb[ks].z = pack_bf16x2(x[4], x[5]);
+            pb[ks].w = pack_bf16x2(x[6], x[7]);
+        }
+        rs = half[0] + half[1];
+    };
+    // The row sum bounds the largest probability (max <= sum <= 16 max): a sum that is too large, or
+    // not finite (the first block, or a jump of the maximum), moves the reference and redoes the
+    // block.  Rare, so the raw logits are not kept for it: they are recomputed from the K block,
+    // which is still in LDS (block blk of stage st).
+    auto fix_reference = [&](const unsigned char *st, int blk, float c, uint4 (&pb)[2], float &rs) __attribute__((always_inline)) {
+        acc_t s;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0;
+#pragma unroll
+        for (int q = 0; q < KSTEPS; ++q) {
+            const uint4 kt = *(const uint4 *)(st + k_addr[q & 1] + (q >> 1) * 4096 + blk * 2048);
+            if constexpr (MODE == MODE_I8)
+                s = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kt), __builtin_bit_cast(i32x4, qreg[q]), s, 0, 0, 0);
+            else
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kt), __builtin_bit_cast(bf16x8, qreg[q]), s, 0, 0, 0);
+        }
+        float mx = max3((float)s[0], (float)s[1], (float)s[2]);
+#pragma unroll
+        for (int r = 3; r < 15; r += 2) mx = max3(mx, (float)s[r], (float)s[r + 1]);
+        mx = xhalf_max(fmaxf(mx, (float)s[15])) * c;
+        move_reference(mx);
+        exp_pack(s, c, pb, rs);
+    };
+    // a block with masked keys (causal diagonal, key-length edge), no look-ahead
+    auto masked_block = [&](const unsigned char *st, int blk, int k0, float c) __attribute__((always_inline)) {
+        load_kf(st, blk);
+        load_vf(st, blk);
+        const acc_t s = mfma_qk();
+        float x[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = k0 + blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            float xv = (float)s[r] * c;
+            if (key >= kend || (CAUSAL && key > q_row)) xv = NEG_SENTINEL;
+            x[r] = xv;
+        }
+        float mx = max3(x[0], x[1], x[2]);
+#pragma unroll
+        for (int r = 3; r < 15; r += 2) mx = max3(mx, x[r], x[r + 1]);
+        mx = xhalf_max(fmaxf(mx, x[15]));
+        if (__any(mx > m_run + LAZY_TAU)) move_reference(mx);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_run);
+        l_run += row_sum(x);
+        uint4 pb[2];
+        pack(x, pb);
+        mfma_pv(pb);
+    };
+
+    constexpr int SG_MFMA = 0x008, SG_VALU = 0x402, SG_DSR = 0x100;  // sched_group_barrier classes
+    uint4 pb[2];     // P of the block about to be multiplied with V
+    float rs = 0.f;  // its row sum
+    // One pipelined block j: V(j) is block vb of stage sv; K(j+1), whose fragments are in kf, is block
+    // qb of stage sq; the K fragments requested at the end are block kb of stage sk (block j + 2);
+    // c_next is the exponent factor of block j + 1, whose probabilities are dropped when keep is
+    // false (it lies past this wave's unmasked tiles).
+    auto pipe_block = [&](const unsigned char *sv, int vb, const unsigned char *sq, int qb, const unsigned char *sk, int kb,
+                          float c_next, bool keep) __attribute__((always_inline)) {
+        // ---- R1 ----
+        load_vf(sv, vb);
+        const acc_t s = mfma_qk();
+        l_run += rs;
+        load_kf(sk, kb);
+        __builtin_amdgcn_sched_group_barrier(SG_DSR, DB * 4, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, KSTEPS, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DSR, KSTEPS, 0);
+        ARHIP_FENCE();
+        // ---- R2 ----
+        mfma_pv(pb);
+        uint4 pn[2];
+        exp_pack(s, c_next, pn, rs);
+        constexpr int NV = (MODE == MODE_I8) ? 72 : 56;  // vector instructions of exp_pack
+        constexpr int PER = (NV + DB * 2 - 3) / (DB * 2 - 2);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);
+#pragma unroll
+        for (int i = 0; i < DB * 2 - 2; ++i) {
+            __builtin_amdgcn_sched_group_barrier(SG_VALU, PER, 0);
+            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        }
+        ARHIP_FENCE();
+        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)) && keep, 0)) fix_reference(sq, qb, c_next, pn, rs);
+        pb[0] = pn[0];
+        pb[1] = pn[1];
+    };
+
+    // ---- prologue: tiles 0..2 on their way, tiles 0 and 1 visible ----
+    // The pipelined loop covers the tiles in which no key is masked for ANY wave of the workgroup
+    // (all full tiles; under the causal mask those before the workgroup's first query), so that
+    // every wave runs the same code between barriers.  The remaining tiles (at most 4 on the causal
+    // diagonal, or the last partial one) go block by block with the masks applied.
+    const int npipe = CAUSAL ? min(kend / BK, qblk / BK) : kend / BK;
+    issue_tile(0, 0);
+    issue_tile(1, 1);
+    issue_tile(2, 2);
+    // Q operand, resident in registers.  Everything in flight is awaited here once, Q included, so
+    // that no wait for a global load is left inside the loops.
+    {
+        const unsigned char *qb = (const unsigned char *)p.q +
+                                  ((size_t)b * p.qs[0] + (size_t)head * p.qs[1] + (size_t)min(q_row, N - 1) * p.qs[2]) * QK_BYTES;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) qreg[s] = *(const uint4 *)(qb + s * 32 + h * 16);
+    }
+
+    wait_vmem_le<0>();
+    __syncthreads();
+    if (npipe > 0) {
+        load_kf(lds, 0);
+        const acc_t s = mfma_qk();
+        load_kf(lds, 1);
+        const float c0 = tile_c(0);
+        exp_pack(s, c0, pb, rs);
+        if (__any(!(rs <= 16.0f * LAZY_LIMIT))) fix_reference(lds, 0, c0, pb, rs);
+    }
+
+#pragma clang loop unroll(disable)
+    for (int it = 0; it < npipe; ++it) {
+        const unsigned char *st_cur = lds + (it & 3) * STAGE;
+        const unsigned char *st_nxt = lds + ((it + 1) & 3) * STAGE;
+        // tile it + 3 goes to the stage tile it - 1 vacated at the last barrier
+        issue_tile(it + 3, (it + 3) & 3);
+        const float c_cur = tile_c(it), c_nxt = tile_c(it + 1);
+        pipe_block(st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, true);
+        pipe_block(st_cur, 1, st_nxt, 0, st_nxt, 1, c_nxt, it + 1 < npipe);
+        wait_vmem_le<XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
+        __syncthreads();
+    }
+#pragma clang loop unroll(disable)
+    for (int it = npipe; it < ntiles; ++it) {
+        const unsigned char *st_cur = lds + (it & 3) * STAGE;
+        issue_tile(it + 3, (it + 3) & 3);
+        if (it < my_tiles) {
+            const float c_cur = tile_c(it);
+            masked_block(st_cur, 0, it * BK, c_cur);
+            masked_block(st_cur, 1, it * BK, c_cur);
+        }
+        wait_vmem_le<XPW_MIN>();
+        __syncthreads();
+    }
+
+    // ---- normalise and store: acc * (l > 0 ? 1/l : 0), cuda_flash_bf16.rs:414-426 ----
+    const float l_tot = xhalf_sum(l_run);
+    const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
+    if (p.lse != nullptr && h == 0 && q_row < N) {
+        p.lse[(size_t)bh * N + q_row] = (l_tot > 0.f) ? (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : NEG_SENTINEL;
+    }
+    if (q_row < N) {
+        const size_t obase = (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)q_row * p.os[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int gg = 0; gg < 4; ++gg) {
+                const int d = db * 32 + 8 * gg + 4 * h;
+                const float o0 = oacc[db][4 * gg + 0] * inv, o1 = oacc[db][4 * gg + 1] * inv;
+                const float o2 = oacc[db][4 * gg + 2] * inv, o3 = oacc[db][4 * gg + 3] * inv;
+                if (OUT_F32) {
+                    *(float4 *)((float *)p.o + obase + d) = make_float4(o0, o1, o2, o3);
+                } else {
+                    uint2 w;
+                    w.x = pack_bf16x2(o0, o1);
+                    w.y = pack_bf16x2(o2, o3);
+                    *(uint2 *)((uint16_t *)p.o + obase + d) = w;
+                }
+            }
+    }
+}
+
+}  // namespace arhip

@@ -6,6 +6,7 @@
 #include "arhip_internal.h"
 
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 
 static thread_local std::string g_last_error;
@@ -116,6 +117,7 @@ extern "C" int arhip_open(int ordinal, arhip_device **out)
     d->ordinal = ordinal;
     d->arch = arch;
     d->cus = prop.multiProcessorCount;
+    if (const char *e = getenv("ARHIP_ATTN_WAVES")) d->attn_waves = atoi(e);
     hipError_t e = hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&d->ev0);
     if (e == hipSuccess) e = hipEventCreate(&d->ev1);

@@ -6,9 +6,9 @@
 // (src/runtime/cuda_flash_sage.rs:452-485).
 #include "arhip_internal.h"
 #include "attn_fwd.h"
+#include "attn_pipe.h"
 #include "flash_f32.h"
 
-#include <cstdlib>
 
 using namespace arhip;
 
@@ -61,6 +61,22 @@ static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bo
         hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
 }
 
+// The software-pipelined long-sequence kernel (8 waves, no additive mask, tile-uniform K scales).
+template <int D, int MODE, bool OUT_F32>
+static void launch_pipe(hipStream_t stream, const AttnParams &p, bool causal)
+{
+    const dim3 grid((unsigned)p.total), block(512);
+    if (causal) hipLaunchKernelGGL((attn_pipe_kernel<D, true, MODE, OUT_F32>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_pipe_kernel<D, false, MODE, OUT_F32>), grid, block, 0, stream, p);
+}
+
+// The pipelined kernel addresses K and V through 32-bit buffer offsets (rows of one head, plus the
+// tiles it requests past the end).
+static bool pipe_addressable(int64_t N, int64_t kv_token_stride, int64_t elem_bytes)
+{
+    return (N + 5 * 64) * kv_token_stride * elem_bytes < ((int64_t)1 << 31);
+}
+
 // Tiling variants = waves (of 32 queries) per workgroup.
 //   1  32 queries per workgroup: short sequences, spreads the heads over the chip
 //   4  128 queries
@@ -72,10 +88,9 @@ static int pick_waves(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bo
     if (D == 64 && heads * ((N + 127) / 128) < 2 * (int64_t)dev->cus) nw = 1;
     else if (special) nw = 4;
     else nw = (heads * ((N + 255) / 256) >= 2 * (int64_t)dev->cus) ? 8 : 4;
-    if (const char *e = getenv("ARHIP_ATTN_WAVES")) {  // tuning aid; results do not depend on it
-        const int w = atoi(e);
-        if ((w == 1 || w == 4 || w == 8) && !special && (w != 1 || D == 64)) nw = w;
-    }
+    // ARHIP_ATTN_WAVES (read once when the device is opened) is a tuning aid; results do not depend on it
+    const int w = dev->attn_waves;
+    if ((w == 1 || w == 4 || w == 8) && !special && (w != 1 || D == 64)) nw = w;
     return nw;
 }
 
@@ -176,12 +191,13 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
     p.bq = p.bk = 1;
     p.scale = scale;
     const bool c = causal != 0, hm = mask != nullptr;
-    const int nw = pick_waves(dev, B * Hq, N, D, hm);
+    int nw = pick_waves(dev, B * Hq, N, D, hm);
+    if (nw == 8 && !pipe_addressable(N, kv_strides[2], 2)) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;  // few workgroups per CU: balance them globally
     if (int rc = t.begin()) return rc;
-    if (N <= 256 && !hm && B * Hq * ((N + 127) / 128) <= 4 * (int64_t)dev->cus && !getenv("ARHIP_ATTN_WAVES")) {
+    if (N <= 256 && !hm && B * Hq * ((N + 127) / 128) <= 4 * (int64_t)dev->cus && dev->attn_waves == 0) {
         // short sequence: bring all of K/V into LDS at once (128 queries per workgroup)
         p.nq = (int)((N + 127) / 128);
         p.total = (int)(p.nq * B * Hq);
@@ -196,10 +212,10 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
     } else if (D == 64) {
         if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
         else if (nw == 4) launch_attn<64, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
-        else launch_attn<64, 8, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm);
+        else launch_pipe<64, MODE_BF16, false>(dev->stream, p, c);
     } else {
         if (nw == 4) launch_attn<128, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
-        else launch_attn<128, 8, MODE_BF16, false, false, false, false>(dev->stream, p, c, hm);
+        else launch_pipe<128, MODE_BF16, false>(dev->stream, p, c);
     }
     arhip_note_selected(ARHIP_K_FLASH_BF16);
     return t.end();
@@ -241,6 +257,7 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
     p.bk_tile_shift = shift;
     int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg);
     if (nw == 1) nw = 4;
+    if (nw == 8 && !pipe_addressable(N, D, 2)) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;
@@ -266,7 +283,8 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
             else SAGE_V(DD, 4, false, true, false);                                                    \
         } else if (per_key) SAGE_V(DD, 4, true, false, true);                                          \
         else if (nw == 4) SAGE_V(DD, 4, false, false, true);                                           \
-        else SAGE_V(DD, 8, false, false, false);                                                       \
+        else if (f32o) launch_pipe<DD, MODE_I8, true>(dev->stream, p, c);                              \
+        else launch_pipe<DD, MODE_I8, false>(dev->stream, p, c);                                       \
     } while (0)
     if (D == 64) SAGE_D(64);
     else SAGE_D(128);
