@@ -20,8 +20,9 @@
 //                  R1(j)  S = K(j+1) . Q^T         (MFMA)
 //                  R2(j)  O^T += V(j)^T . P(j)^T   (MFMA)  |  P(j+1) = exp2(S c - m), row sum,
 //                                                             bf16 pack                  (VALU)
-//                V(j) fragments are requested at the start of R1(j), K(j+2) fragments at its end.
-//                Carried from block to block: P(j) packed, its row sum, the K(j+1) fragments.
+//                Every fragment register is refilled right after the MFMA that read it: K(j+2)
+//                behind the S^T MFMAs of R1(j), V(j+1) behind the O^T MFMAs of R2(j).
+//                Carried from block to block: P(j) packed, its row sum, the K(j+1) and V(j) fragments.
 //   reference    lazy exponent reference as in attn_fwd.h; it is checked right after R2, while S
 //                still holds the raw logits (the rare case recomputes P from them).
 //   masked tiles (causal diagonal, key-length edge) run block by block without look-ahead.
@@ -40,6 +41,16 @@ template <int N>
 __device__ __forceinline__ void wait_vmem_le()
 {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// f(integral_constant<int, A>) ... f(integral_constant<int, B - 1>), unrolled at compile time
+template <int A, int B, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (A < B) {
+        f(std::integral_constant<int, A>{});
+        static_for<A + 1, B>(f);
+    }
 }
 
 template <int D, bool CAUSAL, int MODE, bool OUT_F32>
@@ -187,14 +198,37 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
     }
     const float c_scale = p.scale * LOG2E;
     const int last_tile = (N - 1) / BK;
-    // exponent factor of the keys of tile t: scale log2(e), times sq sk for int8
-    // (s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322)
-    auto tile_c = [&](int t) __attribute__((always_inline)) -> float {
+    // int8: the K scales of 64 consecutive tiles sit in one register (lane l holds tile 64 g + l),
+    // for the current group of tiles and the next one; a tile's scale is then a v_readlane away.
+    // (A scalar load per tile would share its counter with the LDS reads and, returning out of
+    // order, force every LDS wait in the loop down to "everything has returned".)
+    float skv_cur = 1.f, skv_nxt = 1.f;
+    auto load_sk_group = [&](int g) __attribute__((always_inline)) -> float {
+        const int t = min(g * 64 + lane, last_tile);
+        return p.sk[(size_t)kv_bh * nkb + (t >> p.bk_tile_shift)];
+    };
+    // exponent factor of the keys of tile t (in the group of tile `it` or the next one): scale log2(e),
+    // times sq sk for int8 (s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322)
+    auto tile_c = [&](int t, int it) __attribute__((always_inline)) -> float {
         if constexpr (MODE == MODE_I8) {
-            const float f = p.sk[(size_t)kv_bh * nkb + (min(t, last_tile) >> p.bk_tile_shift)];
+            const int a = __builtin_amdgcn_readlane(__float_as_int(skv_cur), t & 63);
+            const int bnext = __builtin_amdgcn_readlane(__float_as_int(skv_nxt), t & 63);
+            const float f = __int_as_float(((t >> 6) == (it >> 6)) ? a : bnext);
             return ((sq_lane * f) * p.scale) * LOG2E;
         } else {
             return c_scale;
+        }
+    };
+    // called at the top of iteration it: moves to the next group of 64 tiles when it begins.  The
+    // wait makes the new vector's arrival explicit (once per 64 tiles) so that no wait for it is
+    // left at its uses.
+    auto advance_sk_group = [&](int it) __attribute__((always_inline)) {
+        if constexpr (MODE == MODE_I8) {
+            if ((it & 63) == 0 && it > 0) {
+                skv_cur = skv_nxt;
+                skv_nxt = load_sk_group((it >> 6) + 1);
+                wait_vmem_le<0>();
+            }
         }
     };
 
@@ -330,37 +364,91 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
         mfma_pv(pb);
     };
 
-    constexpr int SG_MFMA = 0x008, SG_VALU = 0x402, SG_DSR = 0x100;  // sched_group_barrier classes
     uint4 pb[2];     // P of the block about to be multiplied with V
     float rs = 0.f;  // its row sum
-    // One pipelined block j: V(j) is block vb of stage sv; K(j+1), whose fragments are in kf, is block
-    // qb of stage sq; the K fragments requested at the end are block kb of stage sk (block j + 2);
-    // c_next is the exponent factor of block j + 1, whose probabilities are dropped when keep is
-    // false (it lies past this wave's unmasked tiles).
+    // The softmax of an unmasked block as a list of single vector instructions, so that they can be
+    // dealt out between the matrix instructions by hand.  Per half of 8 keys: [convert (int8 only)]
+    // 8 x fma(s, c, -m), 8 x exp2, 7 adds (row sum of the unrounded values), 4 bf16 packs.
+    constexpr int SM_CVT = (MODE == MODE_I8) ? 8 : 0;
+    constexpr int SM_HALF = SM_CVT + 8 + 8 + 7 + 4;
+    constexpr int SM_OPS = 2 * SM_HALF;
+    float sm_t[8], sm_x[8], sm_a[6], sm_half[2];
+    auto sm_op = [&](auto ic, const acc_t &s, float c, uint4 (&pn)[2]) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int ks = i / SM_HALF, k = i % SM_HALF;
+        if constexpr (k < SM_CVT) {
+            sm_t[k] = (float)s[ks * 8 + k];
+        } else if constexpr (k < SM_CVT + 8) {
+            constexpr int r = k - SM_CVT;
+            sm_t[r] = __builtin_fmaf((MODE == MODE_I8) ? sm_t[r] : (float)s[ks * 8 + r], c, -m_run);
+        } else if constexpr (k < SM_CVT + 16) {
+            constexpr int r = k - SM_CVT - 8;
+            sm_x[r] = __builtin_amdgcn_exp2f(sm_t[r]);
+        } else if constexpr (k < SM_CVT + 23) {
+            constexpr int a = k - SM_CVT - 16;  // ((x0+x1)+(x2+x3)) + ((x4+x5)+(x6+x7))
+            if constexpr (a < 4) sm_a[a] = sm_x[2 * a] + sm_x[2 * a + 1];
+            else if constexpr (a < 6) sm_a[a] = sm_a[2 * (a - 4)] + sm_a[2 * (a - 4) + 1];
+            else sm_half[ks] = sm_a[4] + sm_a[5];
+        } else {
+            constexpr int j = k - SM_CVT - 23;
+            const uint32_t w = pack_bf16x2(sm_x[2 * j], sm_x[2 * j + 1]);
+            if constexpr (j == 0) pn[ks].x = w;
+            else if constexpr (j == 1) pn[ks].y = w;
+            else if constexpr (j == 2) pn[ks].z = w;
+            else pn[ks].w = w;
+        }
+    };
+
+    // One pipelined block j.  On entry kf holds the K(j+1) fragments and vf the V(j) fragments, both
+    // requested during block j-1.  Every fragment register is refilled right after the MFMA that
+    // read it: K(j+2) (block kb of stage sk) behind the S^T MFMAs, V(j+1) (block vb of stage sv)
+    // behind the O^T MFMAs, so each LDS read has a whole region to arrive.  K(j+1) itself is block qb
+    // of stage sq (needed again only when the exponent reference moves).  c_next is the exponent
+    // factor of block j + 1, whose probabilities are dropped when keep is false (it lies past the
+    // pipelined tiles).  The instruction order below IS the schedule: the fences keep the compiler
+    // from moving anything across them, and the wave issues in order.
     auto pipe_block = [&](const unsigned char *sv, int vb, const unsigned char *sq, int qb, const unsigned char *sk, int kb,
                           float c_next, bool keep) __attribute__((always_inline)) {
-        // ---- R1 ----
-        load_vf(sv, vb);
-        const acc_t s = mfma_qk();
-        l_run += rs;
-        load_kf(sk, kb);
-        __builtin_amdgcn_sched_group_barrier(SG_DSR, DB * 4, 0);
-        __builtin_amdgcn_sched_group_barrier(SG_MFMA, KSTEPS, 0);
-        __builtin_amdgcn_sched_group_barrier(SG_DSR, KSTEPS, 0);
-        ARHIP_FENCE();
-        // ---- R2 ----
-        mfma_pv(pb);
-        uint4 pn[2];
-        exp_pack(s, c_next, pn, rs);
-        constexpr int NV = (MODE == MODE_I8) ? 72 : 56;  // vector instructions of exp_pack
-        constexpr int PER = (NV + DB * 2 - 3) / (DB * 2 - 2);
-        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);
+        // ---- R1: S^T = K(j+1) . Q^T ----
+        acc_t s;
 #pragma unroll
-        for (int i = 0; i < DB * 2 - 2; ++i) {
-            __builtin_amdgcn_sched_group_barrier(SG_VALU, PER, 0);
-            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
-        }
+        for (int r = 0; r < 16; ++r) s[r] = 0;
+        l_run += rs;
         ARHIP_FENCE();
+#pragma unroll
+        for (int st = 0; st < KSTEPS; ++st) {
+            if constexpr (MODE == MODE_I8)
+                s = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kf[st]), __builtin_bit_cast(i32x4, qreg[st]), s, 0, 0, 0);
+            else
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s, 0, 0, 0);
+            ARHIP_FENCE();
+            kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
+            ARHIP_FENCE();
+        }
+        // ---- R2: O^T += V(j)^T . P(j)^T, and P(j+1) from S on the vector ALU ----
+        uint4 pn[2];
+        constexpr int SLOTS = DB * 2 - 2;  // S is not ready under the first two MFMAs
+        static_for<0, DB * 2>([&](auto gi) __attribute__((always_inline)) {
+            constexpr int g = decltype(gi)::value;
+            constexpr int db = g / 2, ks = g % 2;
+            const uint4 a = make_uint4(vf[db][ks][0].x, vf[db][ks][0].y, vf[db][ks][1].x, vf[db][ks][1].y);
+            oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                               __builtin_bit_cast(bf16x8, pb[ks]), oacc[db], 0, 0, 0);
+            ARHIP_FENCE();
+            if constexpr (g >= 2) {
+                constexpr int lo = (g - 2) * SM_OPS / SLOTS, hi = (g - 1) * SM_OPS / SLOTS;
+                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(ic, s, c_next, pn); });
+            }
+            if constexpr (ks == 1) {
+#pragma unroll
+                for (int k2 = 0; k2 < 2; ++k2) {
+                    vf[db][k2][0] = lds_read_tr16(sv + v_addr[0] + db * 4096 + (vb * 2 + k2) * 1024);
+                    vf[db][k2][1] = lds_read_tr16(sv + v_addr[1] + db * 4096 + (vb * 2 + k2) * 1024);
+                }
+            }
+            ARHIP_FENCE();
+        });
+        rs = sm_half[0] + sm_half[1];
         if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)) && keep, 0)) fix_reference(sq, qb, c_next, pn, rs);
         pb[0] = pn[0];
         pb[1] = pn[1];
@@ -384,13 +472,18 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
         for (int s = 0; s < KSTEPS; ++s) qreg[s] = *(const uint4 *)(qb + s * 32 + h * 16);
     }
 
+    if constexpr (MODE == MODE_I8) {
+        skv_cur = load_sk_group(0);
+        skv_nxt = load_sk_group(1);
+    }
     wait_vmem_le<0>();
     __syncthreads();
     if (npipe > 0) {
         load_kf(lds, 0);
         const acc_t s = mfma_qk();
         load_kf(lds, 1);
-        const float c0 = tile_c(0);
+        load_vf(lds, 0);
+        const float c0 = tile_c(0, 0);
         exp_pack(s, c0, pb, rs);
         if (__any(!(rs <= 16.0f * LAZY_LIMIT))) fix_reference(lds, 0, c0, pb, rs);
     }
@@ -401,9 +494,10 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
         const unsigned char *st_nxt = lds + ((it + 1) & 3) * STAGE;
         // tile it + 3 goes to the stage tile it - 1 vacated at the last barrier
         issue_tile(it + 3, (it + 3) & 3);
-        const float c_cur = tile_c(it), c_nxt = tile_c(it + 1);
-        pipe_block(st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, true);
-        pipe_block(st_cur, 1, st_nxt, 0, st_nxt, 1, c_nxt, it + 1 < npipe);
+        advance_sk_group(it);
+        const float c_cur = tile_c(it, it), c_nxt = tile_c(it + 1, it);
+        pipe_block(st_cur, 1, st_cur, 1, st_nxt, 0, c_cur, true);
+        pipe_block(st_nxt, 0, st_nxt, 0, st_nxt, 1, c_nxt, it + 1 < npipe);
         wait_vmem_le<XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
         __syncthreads();
     }
@@ -411,8 +505,9 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
     for (int it = npipe; it < ntiles; ++it) {
         const unsigned char *st_cur = lds + (it & 3) * STAGE;
         issue_tile(it + 3, (it + 3) & 3);
+        advance_sk_group(it);
         if (it < my_tiles) {
-            const float c_cur = tile_c(it);
+            const float c_cur = tile_c(it, it);
             masked_block(st_cur, 0, it * BK, c_cur);
             masked_block(st_cur, 1, it * BK, c_cur);
         }
