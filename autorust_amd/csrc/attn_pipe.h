@@ -17,14 +17,15 @@
 //                8 passes during which the wave may issue independent vector instructions.  The
 //                instruction stream therefore interleaves the two pipes itself, one 32-key block
 //                ahead:
-//                  R1(j)  S = K(j+1) . Q^T         (MFMA)
-//                  R2(j)  O^T += V(j)^T . P(j)^T   (MFMA)  |  P(j+1) = exp2(S c - m), row sum,
-//                                                             bf16 pack                  (VALU)
+//                  R1(j)  S(j+1) = K(j+1) . Q^T    (MFMA)  |  second part of the softmax of S(j)  (VALU)
+//                  R2(j)  O^T += V(j)^T . P(j)^T   (MFMA)  |  first part of the softmax of S(j+1)
+//                softmax = exp2(S c - m), row sum, bf16 pack, dealt out one instruction at a time
 //                Every fragment register is refilled right after the MFMA that read it: K(j+2)
 //                behind the S^T MFMAs of R1(j), V(j+1) behind the O^T MFMAs of R2(j).
-//                Carried from block to block: P(j) packed, its row sum, the K(j+1) and V(j) fragments.
-//   reference    lazy exponent reference as in attn_fwd.h; it is checked right after R2, while S
-//                still holds the raw logits (the rare case recomputes P from them).
+//                Carried from block to block: the logits S(j) with their softmax half done, the
+//                K(j+1) and V(j) fragments.
+//   reference    lazy exponent reference as in attn_fwd.h; it is checked between R1 and R2 (the
+//                rare case recomputes the block's logits from K, which is still in LDS).
 //   masked tiles (causal diagonal, key-length edge) run block by block without look-ahead.
 //
 // 8 waves of 32 queries per workgroup, two waves per SIMD.
@@ -399,35 +400,46 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
         }
     };
 
-    // One pipelined block j.  On entry kf holds the K(j+1) fragments and vf the V(j) fragments, both
-    // requested during block j-1.  Every fragment register is refilled right after the MFMA that
-    // read it: K(j+2) (block kb of stage sk) behind the S^T MFMAs, V(j+1) (block vb of stage sv)
-    // behind the O^T MFMAs, so each LDS read has a whole region to arrive.  K(j+1) itself is block qb
-    // of stage sq (needed again only when the exponent reference moves).  c_next is the exponent
-    // factor of block j + 1, whose probabilities are dropped when keep is false (it lies past the
-    // pipelined tiles).  The instruction order below IS the schedule: the fences keep the compiler
-    // from moving anything across them, and the wave issues in order.
-    auto pipe_block = [&](const unsigned char *sv, int vb, const unsigned char *sq, int qb, const unsigned char *sk, int kb,
-                          float c_next, bool keep) __attribute__((always_inline)) {
-        // ---- R1: S^T = K(j+1) . Q^T ----
-        acc_t s;
+    // One pipelined block j.  On entry kf holds the K(j+1) fragments and vf the V(j) fragments (both
+    // requested during block j-1), s_old the logits of block j with the first SM_SPLIT softmax
+    // instructions already done.
+    //   R1  S^T(j+1) = K(j+1) . Q^T into s_new     |  rest of the softmax of block j  -> P(j), row sum
+    //   --  reference check for block j (rare: recompute P(j) from K(j), block cb of stage sc)
+    //   R2  O^T += V(j)^T . P(j)^T                  |  first SM_SPLIT softmax instructions of block j+1
+    // Every fragment register is refilled right after the MFMA that read it: K(j+2) (block kb of
+    // stage sk) in R1, V(j+1) (block vb of stage sv) in R2, so each LDS read has a whole region to
+    // arrive.  c_cur / c_next are the exponent factors of blocks j and j+1.  The instruction order
+    // below IS the schedule: the fences keep the compiler from moving anything across them, and
+    // the wave issues in order.  Past the last pipelined block the look-ahead works on whatever
+    // the next LDS stage holds; those results are never used.
+    constexpr int R2_SLOTS = DB * 2 - 2;  // S is not ready under the first two O^T MFMAs
+    constexpr int SM_SPLIT = (MODE == MODE_I8) ? (SM_OPS * R2_SLOTS) / (R2_SLOTS + KSTEPS) : SM_HALF;
+    uint4 pn[2];  // P of the block whose softmax is in progress
+    auto pipe_block = [&](acc_t &s_old, acc_t &s_new, const unsigned char *sc, int cb, const unsigned char *sv, int vb,
+                          const unsigned char *sk, int kb, float c_cur, float c_next) __attribute__((always_inline)) {
+        // ---- R1 ----
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0;
-        l_run += rs;
+        for (int r = 0; r < 16; ++r) s_new[r] = 0;
         ARHIP_FENCE();
-#pragma unroll
-        for (int st = 0; st < KSTEPS; ++st) {
+        static_for<0, KSTEPS>([&](auto si) __attribute__((always_inline)) {
+            constexpr int st = decltype(si)::value;
             if constexpr (MODE == MODE_I8)
-                s = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kf[st]), __builtin_bit_cast(i32x4, qreg[st]), s, 0, 0, 0);
+                s_new = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kf[st]), __builtin_bit_cast(i32x4, qreg[st]), s_new, 0, 0, 0);
             else
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s, 0, 0, 0);
+                s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s_new, 0, 0, 0);
             ARHIP_FENCE();
+            constexpr int lo = SM_SPLIT + st * (SM_OPS - SM_SPLIT) / KSTEPS, hi = SM_SPLIT + (st + 1) * (SM_OPS - SM_SPLIT) / KSTEPS;
+            static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(ic, s_old, c_cur, pn); });
             kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
             ARHIP_FENCE();
-        }
-        // ---- R2: O^T += V(j)^T . P(j)^T, and P(j+1) from S on the vector ALU ----
-        uint4 pn[2];
-        constexpr int SLOTS = DB * 2 - 2;  // S is not ready under the first two MFMAs
+        });
+        rs = sm_half[0] + sm_half[1];
+        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(sc, cb, c_cur, pn, rs);
+        l_run += rs;
+        pb[0] = pn[0];
+        pb[1] = pn[1];
+        ARHIP_FENCE();
+        // ---- R2 ----
         static_for<0, DB * 2>([&](auto gi) __attribute__((always_inline)) {
             constexpr int g = decltype(gi)::value;
             constexpr int db = g / 2, ks = g % 2;
@@ -436,8 +448,8 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
                                                                __builtin_bit_cast(bf16x8, pb[ks]), oacc[db], 0, 0, 0);
             ARHIP_FENCE();
             if constexpr (g >= 2) {
-                constexpr int lo = (g - 2) * SM_OPS / SLOTS, hi = (g - 1) * SM_OPS / SLOTS;
-                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(ic, s, c_next, pn); });
+                constexpr int lo = (g - 2) * SM_SPLIT / R2_SLOTS, hi = (g - 1) * SM_SPLIT / R2_SLOTS;
+                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(ic, s_new, c_next, pn); });
             }
             if constexpr (ks == 1) {
 #pragma unroll
@@ -448,10 +460,6 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
             }
             ARHIP_FENCE();
         });
-        rs = sm_half[0] + sm_half[1];
-        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)) && keep, 0)) fix_reference(sq, qb, c_next, pn, rs);
-        pb[0] = pn[0];
-        pb[1] = pn[1];
     };
 
     // ---- prologue: tiles 0..2 on their way, tiles 0 and 1 visible ----
@@ -478,14 +486,16 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
     }
     wait_vmem_le<0>();
     __syncthreads();
+    acc_t s_a, s_b;  // logits of the even / odd block of a tile
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s_a[r] = s_b[r] = 0;
     if (npipe > 0) {
         load_kf(lds, 0);
-        const acc_t s = mfma_qk();
+        s_a = mfma_qk();
         load_kf(lds, 1);
         load_vf(lds, 0);
         const float c0 = tile_c(0, 0);
-        exp_pack(s, c0, pb, rs);
-        if (__any(!(rs <= 16.0f * LAZY_LIMIT))) fix_reference(lds, 0, c0, pb, rs);
+        static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(ic, s_a, c0, pn); });
     }
 
 #pragma clang loop unroll(disable)
@@ -496,8 +506,8 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
         issue_tile(it + 3, (it + 3) & 3);
         advance_sk_group(it);
         const float c_cur = tile_c(it, it), c_nxt = tile_c(it + 1, it);
-        pipe_block(st_cur, 1, st_cur, 1, st_nxt, 0, c_cur, true);
-        pipe_block(st_nxt, 0, st_nxt, 0, st_nxt, 1, c_nxt, it + 1 < npipe);
+        pipe_block(s_a, s_b, st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, c_cur);
+        pipe_block(s_b, s_a, st_cur, 1, st_nxt, 0, st_nxt, 1, c_cur, c_nxt);
         wait_vmem_le<XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
         __syncthreads();
     }
