@@ -10,6 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libarhip.so")
 PROBES_PATH = os.path.join(_HERE, "probes.hsaco")
+KERNELS_PATH = os.path.join(_HERE, "attn_kernels.hsaco")
 
 OK, EINVAL, EUNSUPPORTED, EHIP, ENODEVICE = 0, -1, -2, -3, -4
 F32, BF16 = 0, 1

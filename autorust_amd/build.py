@@ -14,16 +14,17 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libarhip.so")
 PROBES = os.path.join(HERE, "probes.hsaco")
+KERNELS = os.path.join(HERE, "attn_kernels.hsaco")  # the named entry points (csrc/attn_entry.hip)
 HOST_LIB = os.path.join(HERE, "libautorust_host.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 SOURCES = ["device.hip", "flash.hip", "sage_quant.hip"]
-HEADERS = ["arhip_internal.h", "attn_fwd.h", "attn_pipe.h", "flash_f32.h", os.path.join("..", "..", "include", "arhip.h")]
+HEADERS = ["arhip_internal.h", "attn_fwd.h", "attn_pipe.h", "flash_f32.h", "sage_quant_kernels.h", os.path.join("..", "..", "include", "arhip.h")]
 
 # -packed-fp32-ops off: packed fp32 VALU instructions are not used by this build.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wall", "-Wno-unused-function",
+         "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
          # loop strength reduction multiplies the address registers of the tile loop and spills them
          "-mllvm", "-disable-lsr"]
 
@@ -76,6 +77,9 @@ def build(force=False, verbose=False):
     if force or _newer(HOST_LIB, host_deps):
         _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", HOST_LIB] + host_srcs +
              ["-L" + HERE, "-larhip", "-Wl,-rpath,$ORIGIN"])
+    entry_src = os.path.join(CSRC, "attn_entry.hip")
+    if force or _newer(KERNELS, [entry_src] + [os.path.join(CSRC, h) for h in HEADERS]):
+        _run([HIPCC] + FLAGS + ["-Wno-inline-asm", "--genco", entry_src, "-o", KERNELS])
     probe_src = os.path.join(CSRC, "probes.hip")
     if os.path.exists(probe_src) and (force or _newer(PROBES, [probe_src])):
         _run([HIPCC] + FLAGS + ["--genco", probe_src, "-o", PROBES])

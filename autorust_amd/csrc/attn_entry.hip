@@ -1,0 +1,245 @@
+// The fused-attention kernels as a loadable gfx950 code object with named entry points, for hosts
+// that launch kernels the way the reference does: `HostCall{src, name, signature, bufs, global,
+// local, vals}` -> `Compiled::run_host_kernel` -> `Prog::call` (src/engine/session.rs:210-256,
+// src/runtime/device.rs:383-402), i.e. hipModuleLoadData + hipModuleLaunchKernel
+// (arhip_module_load + arhip_launch).  Arguments are device pointers followed by 32-bit scalars,
+// in the reference's order:
+//     (Q, K, V, O, M,  N, head_dim, causal, has_mask, hq, hkv)
+//     vals = [n, head_dim, causal, has_mask, hq, hkv]          src/runtime/cuda_flash_bf16.rs:226-231,550-599
+// M is read only when has_mask != 0 (the reference passes O as a dummy, cuda_flash.rs:233-240).
+// Tensors are dense [B, H, N, D]; B follows from the grid (grid.y = B * hq); the scale is
+// 1/sqrt(head_dim) (the reference hard-codes 0.125 for its only head_dim, 64).
+//
+//   entry               block      grid                      covers
+//   ar_flash_f32        [256,1,1]  [ceil(n/128), B*hq, 1]    fp32 exact (cuda_flash.rs)
+//   ar_flash_bf16       [256,1,1]  [ceil(n/128), B*hq, 1]    bf16 (cuda_flash_bf16.rs), any mask
+//   ar_flash_bf16_long  [512,1,1]  [ceil(n/256), B*hq, 1]    bf16 pipelined, has_mask must be 0
+//   ar_flash_sage       [256,1,1]  [ceil(n/128), B*hq, 1]    int8 (cuda_flash_sage.rs), any mask, any
+//                                                            block sizes incl. per-row scales; O f32
+//   ar_flash_sage_long  [512,1,1]  [ceil(n/256), B*hq, 1]    int8 pipelined: has_mask 0, bk = 64 * 2^n
+// The Sage entries take pre-quantised operands (the quantiser is the pre-pass below, not part of
+// the attention kernel as in the reference):
+//     (Q8, K8, V, O, M, SQ, SK,  N, head_dim, causal, has_mask, hq, hkv, bq, bk [, out_f32])
+// head_dim must be 64 or 128; any other value makes the kernel return without writing.
+// The *_long entries address K and V with 32-bit byte offsets: (N + 320) * head_dim * 2 < 2^31.
+#include "attn_fwd.h"
+#include "attn_pipe.h"
+#include "flash_f32.h"
+// last: it switches floating-point contraction off for the rest of the file
+#include "sage_quant_kernels.h"
+
+using namespace arhip;
+
+namespace {
+
+__device__ __forceinline__ int linear_wg() { return (int)(blockIdx.y * gridDim.x + blockIdx.x); }
+
+__device__ __forceinline__ void dense(long s[3], int H, int N, int D)
+{
+    s[0] = (long)H * N * D;
+    s[1] = (long)N * D;
+    s[2] = D;
+}
+
+// AttnParams of a dense launch whose grid is [query tiles, B * hq, 1]
+__device__ __forceinline__ AttnParams dense_params(const void *q, const void *k, const void *v, void *o, const float *m,
+                                                   int N, int D, int has_mask, int hq, int hkv)
+{
+    AttnParams p = {};
+    p.q = q; p.k = k; p.v = (const uint16_t *)v; p.o = o;
+    p.mask = has_mask ? m : nullptr;
+    p.Hq = hq; p.Hkv = hkv; p.N = N;
+    dense(p.qs, hq, N, D);
+    dense(p.ks, hkv, N, D);
+    dense(p.os, hq, N, D);
+    p.bq = p.bk = 1;
+    p.nq = (int)gridDim.x;
+    p.total = (int)(gridDim.x * gridDim.y);
+    p.lpt = p.total <= 16 * 256;  // few workgroups per compute unit: order them longest first
+    p.scale = 1.0f / __builtin_sqrtf((float)D);
+    return p;
+}
+
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_f32(const float *Q, const float *K, const float *V, float *O,
+                                                                const float *M, int N, int head_dim, int causal,
+                                                                int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<128>()];
+    FlashF32Params p = {};
+    p.q = Q; p.k = K; p.v = V; p.o = O;
+    p.mask = has_mask ? M : nullptr;
+    p.Hq = hq; p.Hkv = hkv; p.N = N;
+    p.nq = (int)gridDim.x;
+    dense(p.qs, hq, N, head_dim);
+    dense(p.ks, hkv, N, head_dim);
+    dense(p.os, hq, N, head_dim);
+    p.scale = 1.0f / __builtin_sqrtf((float)head_dim);
+    const int wg = linear_wg();
+    if (head_dim == 64) {
+        if (causal) flash_f32_body<64, 4, true>(p, lds, wg);
+        else flash_f32_body<64, 4, false>(p, lds, wg);
+    } else if (head_dim == 128) {
+        if (causal) flash_f32_body<128, 4, true>(p, lds, wg);
+        else flash_f32_body<128, 4, false>(p, lds, wg);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                 uint16_t *O, const float *M, int N, int head_dim, int causal,
+                                                                 int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_BF16, false>()];
+    AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, has_mask, hq, hkv);
+    const int wg = linear_wg();
+#define AR_BF16(DD)                                                                                       \
+    do {                                                                                                  \
+        if (has_mask) {                                                                                   \
+            if (causal) attn_fwd_body<DD, 4, true, true, MODE_BF16, false, false, false>(p, lds, wg);     \
+            else attn_fwd_body<DD, 4, false, true, MODE_BF16, false, false, false>(p, lds, wg);           \
+        } else {                                                                                          \
+            if (causal) attn_fwd_body<DD, 4, true, false, MODE_BF16, false, false, false>(p, lds, wg);    \
+            else attn_fwd_body<DD, 4, false, false, MODE_BF16, false, false, false>(p, lds, wg);          \
+        }                                                                                                 \
+    } while (0)
+    if (head_dim == 64) AR_BF16(64);
+    else if (head_dim == 128) AR_BF16(128);
+#undef AR_BF16
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                      uint16_t *O, const float *M, int N, int head_dim,
+                                                                      int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_BF16>()];
+    if (has_mask) return;  // this entry has no additive mask: the host picks ar_flash_bf16 for those
+    AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, 0, hq, hkv);
+    const int wg = linear_wg();
+    if (head_dim == 64) {
+        if (causal) attn_pipe_body<64, true, MODE_BF16, false>(p, lds, wg);
+        else attn_pipe_body<64, false, MODE_BF16, false>(p, lds, wg);
+    } else if (head_dim == 128) {
+        if (causal) attn_pipe_body<128, true, MODE_BF16, false>(p, lds, wg);
+        else attn_pipe_body<128, false, MODE_BF16, false>(p, lds, wg);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_sage(const int8_t *Q8, const int8_t *K8, const uint16_t *V, float *O,
+                                                                 const float *M, const float *SQ, const float *SK, int N,
+                                                                 int head_dim, int causal, int has_mask, int hq, int hkv,
+                                                                 int bq, int bk)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_I8, true>()];
+    AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, has_mask, hq, hkv);
+    p.sq = SQ; p.sk = SK;
+    p.bq = bq; p.bk = bk;
+    // K scales that are uniform over a 64-key tile (bk = 64 * 2^n) are a scalar per tile; any other
+    // block size, the reference's per-key scales (bk = 1) included, stages the tile's scales in LDS
+    int shift = 0;
+    while ((64 << shift) < bk) ++shift;
+    const bool per_key = (64 << shift) != bk;
+    p.bk_tile_shift = shift;
+    const int wg = linear_wg();
+#define AR_SAGE(DD, PK)                                                                                 \
+    do {                                                                                                \
+        if (has_mask) {                                                                                 \
+            if (causal) attn_fwd_body<DD, 4, true, true, MODE_I8, PK, true, false>(p, lds, wg);         \
+            else attn_fwd_body<DD, 4, false, true, MODE_I8, PK, true, false>(p, lds, wg);               \
+        } else {                                                                                        \
+            if (causal) attn_fwd_body<DD, 4, true, false, MODE_I8, PK, true, false>(p, lds, wg);        \
+            else attn_fwd_body<DD, 4, false, false, MODE_I8, PK, true, false>(p, lds, wg);              \
+        }                                                                                               \
+    } while (0)
+    if (head_dim == 64) {
+        if (per_key) AR_SAGE(64, true);
+        else AR_SAGE(64, false);
+    } else if (head_dim == 128) {
+        if (per_key) AR_SAGE(128, true);
+        else AR_SAGE(128, false);
+    }
+#undef AR_SAGE
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
+                                                                      void *O, const float *M, const float *SQ, const float *SK,
+                                                                      int N, int head_dim, int causal, int has_mask, int hq,
+                                                                      int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8>()];
+    int shift = 0;
+    while ((64 << shift) < bk) ++shift;
+    if (has_mask || (64 << shift) != bk) return;  // ar_flash_sage covers those
+    AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, 0, hq, hkv);
+    p.sq = SQ; p.sk = SK;
+    p.bq = bq; p.bk = bk;
+    p.bk_tile_shift = shift;
+    const int wg = linear_wg();
+#define AR_SAGE_LONG(DD)                                                                  \
+    do {                                                                                  \
+        if (out_f32) {                                                                    \
+            if (causal) attn_pipe_body<DD, true, MODE_I8, true>(p, lds, wg);              \
+            else attn_pipe_body<DD, false, MODE_I8, true>(p, lds, wg);                    \
+        } else {                                                                          \
+            if (causal) attn_pipe_body<DD, true, MODE_I8, false>(p, lds, wg);             \
+            else attn_pipe_body<DD, false, MODE_I8, false>(p, lds, wg);                   \
+        }                                                                                 \
+    } while (0)
+    if (head_dim == 64) AR_SAGE_LONG(64);
+    else if (head_dim == 128) AR_SAGE_LONG(128);
+#undef AR_SAGE_LONG
+}
+
+// ---- Sage pre-pass (the quantiser the reference runs inside its attention kernel,
+// src/runtime/cuda_flash_sage.rs:201-223,248-278, hoisted into passes of its own) ----
+// x [B*H, N, D] f32 or bf16; block [256,1,1] for all of them.
+//   ar_sage_kmean_partial_*  grid [ceil(ceil(N/64) / (256/(D/8))), B*H, 1]   part [B*H, ceil(N/64), D]
+//   ar_sage_kmean_final      grid [B*H, 1, 1], block [D,1,1]                 mean [B*H, D]
+//   ar_sage_quant_blocks_*   grid [ceil(N/blk), B*H, 1]                      x8, scales [B*H, ceil(N/blk)]
+//   ar_sage_quant_rows_*     grid [ceil(B*H*N / (256/(D/8))), 1, 1]          x8, scales [B*H*N]
+//   ar_cast_bf16             grid [min(ceil(n/256), 16384), 1, 1]            y bf16
+// smooth != 0 subtracts mean[bh][d] first (K smoothing).
+extern "C" __global__ void __launch_bounds__(256) ar_sage_kmean_partial_f32(const float *x, float *part, int N, int D, int nchunk)
+{
+    k_mean_partial_body<float>(x, part, N, D, nchunk, blockIdx);
+}
+extern "C" __global__ void __launch_bounds__(256) ar_sage_kmean_partial_bf16(const uint16_t *x, float *part, int N, int D, int nchunk)
+{
+    k_mean_partial_body<uint16_t>(x, part, N, D, nchunk, blockIdx);
+}
+extern "C" __global__ void ar_sage_kmean_final(const float *part, float *mean, int N, int D, int nchunk)
+{
+    k_mean_final_body(part, mean, N, D, nchunk, blockIdx);
+}
+extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_blocks_f32(const float *x, int8_t *x8, float *scales,
+                                                                            const float *mean, int N, int D, int blk, int nblk,
+                                                                            int smooth)
+{
+    if (smooth) quant_blocks_body<float, true>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
+    else quant_blocks_body<float, false>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
+}
+extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_blocks_bf16(const uint16_t *x, int8_t *x8, float *scales,
+                                                                             const float *mean, int N, int D, int blk, int nblk,
+                                                                             int smooth)
+{
+    if (smooth) quant_blocks_body<uint16_t, true>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
+    else quant_blocks_body<uint16_t, false>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
+}
+extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_f32(const float *x, int8_t *x8, float *scales,
+                                                                          const float *mean, int N, int D, long rows_total,
+                                                                          int smooth)
+{
+    if (smooth) quant_rows_body<float, true>(x, x8, scales, mean, N, D, rows_total, blockIdx);
+    else quant_rows_body<float, false>(x, x8, scales, mean, N, D, rows_total, blockIdx);
+}
+extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_bf16(const uint16_t *x, int8_t *x8, float *scales,
+                                                                           const float *mean, int N, int D, long rows_total,
+                                                                           int smooth)
+{
+    if (smooth) quant_rows_body<uint16_t, true>(x, x8, scales, mean, N, D, rows_total, blockIdx);
+    else quant_rows_body<uint16_t, false>(x, x8, scales, mean, N, D, rows_total, blockIdx);
+}
+extern "C" __global__ void __launch_bounds__(256) ar_cast_bf16(const float *x, uint16_t *y, long n)
+{
+    cast_bf16_body(x, y, (size_t)n, blockIdx);
+}

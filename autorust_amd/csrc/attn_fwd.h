@@ -129,8 +129,19 @@ __device__ __forceinline__ uint2 lds_read_tr16(const unsigned char *p)
 // s_waitcnt vmcnt(0): all outstanding global loads of this wave have landed.
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// LDS bytes attn_fwd_body needs for a tiling variant
+template <int D, int NW, int MODE, bool PER_KEY, bool SMALL = false>
+constexpr int attn_fwd_lds_bytes()
+{
+    constexpr int QKB = (MODE == MODE_I8) ? 1 : 2;
+    return (SMALL ? 4 : 2) * (BK * (D * QKB + 16) + BK * (D * 2 + 64) + (PER_KEY ? BK * 4 : 0));
+}
+
+// The kernel body.  lds: attn_fwd_lds_bytes<...>() bytes of workgroup memory, 16-byte aligned;
+// wg_linear: this workgroup's index in [0, p.total) (the entry points below and the named entry
+// points of the loadable code object derive it from their grids).
 template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false>
-__global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd_kernel(const AttnParams p)
+__device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
     // SMALL: the whole sequence (at most 4 tiles) is brought into LDS up front, all global loads
     // in flight at once and a single barrier: short sequences are latency bound, not math bound.
@@ -157,7 +168,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
     static_assert(V_CHUNKS % T == 0 || V_CHUNKS < T, "V staging must divide evenly");
     static_assert(!PER_KEY || MODE == MODE_I8, "per-key scales belong to the int8 path");
 
-    __shared__ __attribute__((aligned(16))) unsigned char lds[NSTAGE * STAGE];
+    static_assert(NSTAGE * STAGE == attn_fwd_lds_bytes<D, NW, MODE, PER_KEY, SMALL>(), "LDS size bookkeeping");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -168,7 +179,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
     // Workgroup id -> (head, query tile).  Consecutive ids go to different XCDs
     // (8 of them, each with its own L2); give every XCD a contiguous range of
     // heads so that the query tiles sharing one head's K/V hit the same L2.
-    int wg = blockIdx.x;
+    int wg = wg_linear;
     int bh, qt;
     if (CAUSAL && p.lpt) {
         // Few workgroups per CU and very unequal ones (causal): longest-first over the whole
@@ -557,6 +568,13 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd
                 }
             }
     }
+}
+
+template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false>
+__global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd_kernel(const AttnParams p)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<D, NW, MODE, PER_KEY, SMALL>()];
+    attn_fwd_body<D, NW, CAUSAL, HAS_MASK, MODE, PER_KEY, OUT_F32, DBG, SMALL>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

@@ -54,8 +54,17 @@ __device__ __forceinline__ void static_for(F &&f)
     }
 }
 
+// LDS bytes attn_pipe_body needs: four stages of [piece][64 rows][64 B] K and V tiles
+template <int D, int MODE>
+constexpr int attn_pipe_lds_bytes()
+{
+    return 4 * 4096 * (D * ((MODE == MODE_I8) ? 1 : 2) / 64 + D * 2 / 64);
+}
+
+// The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
+// aligned; wg_linear: this workgroup's index in [0, p.total).
 template <int D, bool CAUSAL, int MODE, bool OUT_F32>
-__global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
+__device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
     constexpr int NW = 8;
     constexpr int BQ = NW * 32;
@@ -73,7 +82,7 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
     constexpr int DB = D / 32;
     static_assert(KP >= 1 && XFERS >= NW, "tile too small for 8 waves");
 
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[NSTAGE * STAGE];
+    static_assert(NSTAGE * STAGE == attn_pipe_lds_bytes<D, MODE>(), "LDS size bookkeeping");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -82,7 +91,7 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
     const int h = lane >> 5;
 
     // workgroup -> (head, query tile), as in attn_fwd_kernel
-    int wg = blockIdx.x;
+    int wg = wg_linear;
     int bh, qt;
     if (CAUSAL && p.lpt) {
         const int nbh = p.total / p.nq;
@@ -550,6 +559,13 @@ __global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
                 }
             }
     }
+}
+
+template <int D, bool CAUSAL, int MODE, bool OUT_F32>
+__global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<D, MODE>()];
+    attn_pipe_body<D, CAUSAL, MODE, OUT_F32>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

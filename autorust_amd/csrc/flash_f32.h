@@ -36,8 +36,17 @@ struct FlashF32Params {
     float scale;
 };
 
+// LDS floats flash_f32_body needs: one padded K tile and one V tile
+template <int D>
+constexpr int flash_f32_lds_floats()
+{
+    return F32_BK * (D + 4) + F32_BK * D;
+}
+
+// The kernel body.  lds: flash_f32_lds_floats<D>() floats of workgroup memory, 16-byte aligned;
+// wg_linear: this workgroup's index in [0, nq * B * Hq).
 template <int D, int NW, bool CAUSAL>
-__global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params p)
+__device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *lds, int wg_linear)
 {
     constexpr int T = NW * 64;
     constexpr int BQ = NW * 32;
@@ -48,13 +57,13 @@ __global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params
     constexpr int PER_THREAD = (CHUNKS + T - 1) / T;
     static_assert(CHUNKS % T == 0, "tile staging must divide evenly");
 
-    __shared__ __attribute__((aligned(16))) float ks[F32_BK * KROW];
-    __shared__ __attribute__((aligned(16))) float vs[F32_BK * D];
+    float *ks = lds;                  // [F32_BK][KROW]
+    float *vs = lds + F32_BK * KROW;  // [F32_BK][D]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i32 = lane & 31, h = lane >> 5;
-    const int bh = blockIdx.x / p.nq;
-    int qt = blockIdx.x - bh * p.nq;
+    const int bh = wg_linear / p.nq;
+    int qt = wg_linear - bh * p.nq;
     if (CAUSAL) qt = p.nq - 1 - qt;
     const int b = bh / p.Hq, head = bh - b * p.Hq;
     const int N = p.N;
@@ -184,6 +193,13 @@ __global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params
                                                   oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
             }
     }
+}
+
+template <int D, int NW, bool CAUSAL>
+__global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params p)
+{
+    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<D>()];
+    flash_f32_body<D, NW, CAUSAL>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

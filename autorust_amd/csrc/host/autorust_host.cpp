@@ -2,10 +2,14 @@
 // Everything computes through libarhip's C ABI; nothing here touches HIP directly.
 #include "autorust_host.h"
 
+#include <dlfcn.h>
+
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <fstream>
 #include <mutex>
 
 namespace autorust {
@@ -68,6 +72,69 @@ Device::~Device()
     arhip_close(dev_);
 }
 
+int Device::compute_units() const { return arhip_compute_units(dev_); }
+
+std::string attention_kernels_src()
+{
+    if (const char *e = getenv("AUTORUST_HIP_KERNELS")) return e;
+    Dl_info info;
+    if (dladdr((const void *)&attention_kernels_src, &info) && info.dli_fname) {
+        std::string p = info.dli_fname;
+        const size_t slash = p.rfind('/');
+        return (slash == std::string::npos ? std::string(".") : p.substr(0, slash)) + "/attn_kernels.hsaco";
+    }
+    return "attn_kernels.hsaco";
+}
+
+std::optional<double> Device::run_host_kernel(const std::string &src, const std::string &name,
+                                              const std::vector<std::pair<int64_t, DType>> &signature,
+                                              const std::vector<void *> &bufs, const int64_t global[3],
+                                              const std::optional<std::array<int64_t, 3>> &local,
+                                              const std::vector<int64_t> &vals, bool wait)
+{
+    // compile_cached: one load per code object and device (device.rs:239-251; the image itself is
+    // cached by content inside arhip_module_load as well)
+    auto it = modules_.find(src);
+    if (it == modules_.end()) {
+        std::ifstream f(src, std::ios::binary);
+        if (!f) throw std::runtime_error("TGERR: run_host_kernel: cannot read the code object " + src);
+        const std::vector<char> image((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+        void *mod = nullptr;
+        check(arhip_module_load(dev_, image.data(), image.size(), &mod));
+        it = modules_.emplace(src, mod).first;
+        if (getenv("AUTORUST_KERNEL_INFO"))  // ops_cuda.rs:902-918 prints per-kernel resources at load
+            std::fprintf(stderr, "[hip] loaded %s (%zu bytes) for %s\n", src.c_str(), image.size(), this->name().c_str());
+    }
+    if (!local) throw std::runtime_error("TGERR: run_host_kernel: " + name + " needs an explicit workgroup shape");
+    const size_t nb = bufs.size();
+    if (signature.size() != nb + vals.size())
+        throw std::runtime_error("TGERR: run_host_kernel: " + name + ": signature does not match bufs + vals");
+    std::vector<void *> ptrs(nb);
+    std::vector<int64_t> sv(vals.size());
+    std::vector<int> bits(vals.size());
+    for (size_t i = 0; i < signature.size(); ++i) {
+        const int64_t slot = signature[i].first;
+        if (slot < 0 || (size_t)slot >= signature.size() || (size_t)slot != i)
+            throw std::runtime_error("TGERR: run_host_kernel: " + name + ": slots must be 0..n-1 in order");
+        if (i < nb) {
+            ptrs[i] = bufs[i];
+        } else {
+            sv[i - nb] = vals[i - nb];
+            bits[i - nb] = signature[i].second == DType::Int64 ? 64 : 32;  // narrowed like ops_cuda.rs:943-990
+        }
+    }
+    unsigned g[3], l[3];
+    for (int i = 0; i < 3; ++i) {
+        g[i] = (unsigned)std::max<int64_t>(global[i], 0);       // negatives clamp to 0 (session.rs:241-251)
+        l[i] = (unsigned)std::max<int64_t>((*local)[i], 0);
+    }
+    double secs = 0.0;
+    check(arhip_launch(dev_, it->second, name.c_str(), g, l, ptrs.data(), (int)nb, sv.data(), bits.data(), (int)sv.size(),
+                       wait ? 1 : 0, &secs));
+    if (wait) return secs;
+    return std::nullopt;
+}
+
 void *Device::alloc(size_t bytes)
 {
     if (bytes == 0) return nullptr;
@@ -101,7 +168,17 @@ Storage::~Storage()
 
 // ---- tensors --------------------------------------------------------------------------
 
-static size_t esize(DType d) { return d == DType::BFloat16 ? 2 : 4; }
+static size_t esize(DType d)
+{
+    switch (d) {
+    case DType::BFloat16: return 2;
+    case DType::Int8: return 1;
+    case DType::Int64: return 8;
+    default: return 4;
+    }
+}
+
+size_t Tensor::nbytes() const { return (size_t)numel() * esize(dtype_); }
 
 int64_t Tensor::numel() const
 {
@@ -197,6 +274,8 @@ Kernel plan_fused(const std::vector<int64_t> &q, const std::vector<int64_t> &k, 
         if (mask_dtype != DType::Float32 || mask_shape->size() != 2 || (*mask_shape)[0] != n || (*mask_shape)[1] != n)
             return Kernel::None;
     }
+    // the launch grid is [query tiles, b*h, 1]: b*h must fit the y dimension of a grid
+    if (b <= 0 || h <= 0 || n <= 0 || b * h > 65535) return Kernel::None;
     const int dt = qd == DType::BFloat16 ? ARHIP_BF16 : ARHIP_F32;
     // Sage: the reference takes f32 tensors only (:411-414); bf16 tensors are accepted here too.
     const bool sage = quantized && st.tensor_cores && arhip_attn_supported(ARHIP_ATTN_SAGE, n, d, dt);
@@ -215,7 +294,31 @@ bool wants_fused(std::optional<AttentionKind> force, const Settings &st, double 
     return effective(requested) != AttentionKind::Sdpa && dropout_p == 0.0 && has_session;
 }
 
-uint64_t selections(Kernel k) { return k == Kernel::None ? 0 : arhip_selections((int)k); }
+static std::atomic<uint64_t> g_selected[3];
+
+uint64_t selections(Kernel k) { return k == Kernel::None ? 0 : g_selected[(int)k].load(std::memory_order_relaxed); }
+
+// Record a dispatch; one-time line under AUTORUST_ATTN_DEBUG (cuda_flash_bf16.rs:446-456,
+// cuda_flash_sage.rs:417-436).
+static void note_selected(Kernel k)
+{
+    static std::once_flag once[3];
+    static const char *what[3] = {"[attention] flash: fp32 exact, fp32 MFMA (gfx950)",
+                                  "[attention] flash: bf16 MFMA, software-pipelined for long sequences (gfx950)",
+                                  "[attention] sage: int8 MFMA for q.k^T, bf16 MFMA for p.v, K smoothing + block scales (gfx950)"};
+    g_selected[(int)k].fetch_add(1, std::memory_order_relaxed);
+    if (getenv("AUTORUST_ATTN_DEBUG")) note_once(once[(int)k], what[(int)k]);
+}
+
+void HostCall::exec() const
+{
+    if (bufs.empty()) throw std::runtime_error("TGERR: HostCall::exec: no buffers");
+    const auto &dev = bufs.front().device();   // the reference resolves `device` by name (session.rs:232)
+    if (dev->name() != device) throw std::runtime_error("TGERR: HostCall::exec: buffers live on " + dev->name() + ", not " + device);
+    std::vector<void *> ptrs;
+    for (const auto &b : bufs) ptrs.push_back(b.ptr());
+    dev->run_host_kernel(src, name, signature, ptrs, global, local, vals, true);
+}
 
 std::optional<Tensor> fused_attention(const Tensor &q, const Tensor &k, const Tensor &v, Session &sess, const Settings &st)
 {
@@ -226,6 +329,141 @@ std::optional<Tensor> fused_attention_kind(const Tensor &q, const Tensor &k, con
                                            Session &sess, const Settings &st)
 {
     return fused_attention_ex(q, k, v, nullptr, false, false, kind == AttentionKind::Sage, sess, st);
+}
+
+namespace {
+
+using Sig = std::vector<std::pair<int64_t, DType>>;
+
+// bufs first, then 32-bit scalars (64-bit where wide[i] is set)
+Sig make_sig(const std::vector<DType> &buf_types, size_t nvals, const std::vector<size_t> &wide = {})
+{
+    Sig s;
+    for (size_t i = 0; i < buf_types.size(); ++i) s.emplace_back((int64_t)i, buf_types[i]);
+    for (size_t i = 0; i < nvals; ++i) {
+        DType t = DType::Int32;
+        for (size_t w : wide)
+            if (w == i) t = DType::Int64;
+        s.emplace_back((int64_t)(buf_types.size() + i), t);
+    }
+    return s;
+}
+
+HostCall make_call(const std::shared_ptr<Device> &dev, const char *name, const std::vector<Tensor> &bufs,
+                   const std::vector<DType> &buf_types, std::array<int64_t, 3> global, std::array<int64_t, 3> local,
+                   const std::vector<int64_t> &vals, const std::vector<size_t> &wide = {})
+{
+    HostCall c;
+    c.device = dev->name();
+    c.src = attention_kernels_src();
+    c.name = name;
+    c.signature = make_sig(buf_types, vals.size(), wide);
+    c.bufs = bufs;
+    for (int i = 0; i < 3; ++i) c.global[i] = global[(size_t)i];
+    c.local = local;
+    c.vals = vals;
+    return c;
+}
+
+// The pipelined kernels want enough workgroups of 256 queries to fill the chip twice and address
+// K/V with 32-bit byte offsets.
+bool long_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int64_t n, int64_t d)
+{
+    return b * h * ((n + 255) / 256) >= 2 * (int64_t)dev->compute_units() && (n + 320) * d * 2 < ((int64_t)1 << 31);
+}
+
+}  // namespace
+
+std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
+                                           const Tensor &out, bool is_causal, Kernel kern, const Settings &st)
+{
+    const int64_t b = q.shape()[0], h = q.shape()[1], n = q.shape()[2], d = q.shape()[3], hk = k.shape()[1];
+    const auto dev = q.device();
+    const DType F = DType::Float32, BF = DType::BFloat16, I8 = DType::Int8;
+    const bool has_mask = attn_mask != nullptr;
+    // the mask slot always holds a buffer; without a mask it is `out` (cuda_flash.rs:233-240)
+    const Tensor mslot = has_mask ? *attn_mask : out;
+    const std::vector<int64_t> vals = {n, d, (int64_t)is_causal, (int64_t)has_mask, h, hk};  // cuda_flash_bf16.rs:550-561
+    std::vector<HostCall> calls;
+
+    if (kern == Kernel::FlashF32) {
+        calls.push_back(make_call(dev, "ar_flash_f32", {q, k, v, out, mslot}, {F, F, F, F, F}, {(n + 127) / 128, b * h, 1},
+                                  {256, 1, 1}, vals));
+        return calls;
+    }
+    if (kern == Kernel::FlashBf16) {
+        if (!has_mask && long_variant(dev, b, h, n, d))
+            calls.push_back(make_call(dev, "ar_flash_bf16_long", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
+                                      {(n + 255) / 256, b * h, 1}, {512, 1, 1}, vals));
+        else
+            calls.push_back(make_call(dev, "ar_flash_bf16", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
+                                      {(n + 127) / 128, b * h, 1}, {256, 1, 1}, vals));
+        return calls;
+    }
+
+    // ---- Sage: quantise Q, smooth + quantise K, (cast V), attention; scratch tensors ride in the
+    // HostCalls, so a replay finds them again and nothing is allocated then ----
+    const bool bf16_in = q.dtype() == DType::BFloat16;
+    const char *sfx = bf16_in ? "bf16" : "f32";
+    const DType X = bf16_in ? BF : F;
+    const int64_t bq = st.sage_block_q, bk = st.sage_block_k;
+    const int64_t nqb = (n + bq - 1) / bq, nkb = (n + bk - 1) / bk, nchunk = (n + 63) / 64;
+    Tensor q8 = Tensor::empty(dev, {b, h, n, d}, I8), k8 = Tensor::empty(dev, {b, hk, n, d}, I8);
+    Tensor sq = Tensor::empty(dev, {b, h, nqb}, F), sk = Tensor::empty(dev, {b, hk, nkb}, F);
+    Tensor mean = Tensor::empty(dev, {b, hk, d}, F);
+    const std::string part_name = std::string("ar_sage_kmean_partial_") + sfx;
+    const std::string rows_name = std::string("ar_sage_quant_rows_") + sfx, blocks_name = std::string("ar_sage_quant_blocks_") + sfx;
+    auto quant = [&](const Tensor &x, const Tensor &x8, const Tensor &sc, int64_t heads, int64_t blk, int64_t nblk, bool smooth) {
+        if (blk == 1) {
+            const int64_t rows = b * heads * n, rpb = 256 / (d / 8);
+            calls.push_back(make_call(dev, rows_name.c_str(), {x, x8, sc, mean}, {X, I8, F, F}, {(rows + rpb - 1) / rpb, 1, 1},
+                                      {256, 1, 1}, {n, d, rows, (int64_t)smooth}, {2}));
+        } else {
+            calls.push_back(make_call(dev, blocks_name.c_str(), {x, x8, sc, mean}, {X, I8, F, F}, {nblk, b * heads, 1},
+                                      {256, 1, 1}, {n, d, blk, nblk, (int64_t)smooth}));
+        }
+    };
+    quant(q, q8, sq, h, bq, nqb, false);
+    if (st.sage_smooth_k) {
+        Tensor part = Tensor::empty(dev, {b, hk, nchunk, d}, F);
+        const int64_t cpb = 256 / (d / 8);
+        calls.push_back(make_call(dev, part_name.c_str(), {k, part}, {X, F}, {(nchunk + cpb - 1) / cpb, b * hk, 1}, {256, 1, 1},
+                                  {n, d, nchunk}));
+        calls.push_back(make_call(dev, "ar_sage_kmean_final", {part, mean}, {F, F}, {b * hk, 1, 1}, {d, 1, 1}, {n, d, nchunk}));
+    }
+    quant(k, k8, sk, hk, bk, nkb, st.sage_smooth_k);
+    Tensor vb = v;
+    if (!bf16_in) {
+        vb = Tensor::empty(dev, {b, hk, n, d}, BF);
+        const int64_t nv = b * hk * n * d;
+        calls.push_back(make_call(dev, "ar_cast_bf16", {v, vb}, {F, BF}, {std::min<int64_t>((nv + 255) / 256, 16384), 1, 1},
+                                  {256, 1, 1}, {nv}, {0}));
+    }
+    std::vector<int64_t> svals = vals;
+    svals.push_back(bq);
+    svals.push_back(bk);
+    int shift = 0;
+    while (((int64_t)64 << shift) < bk) ++shift;
+    const bool tile_uniform = ((int64_t)64 << shift) == bk;
+    if (!has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
+        svals.push_back(bf16_in ? 0 : 1);  // out_f32
+        calls.push_back(make_call(dev, "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
+                                  {(n + 255) / 256, b * h, 1}, {512, 1, 1}, svals));
+    } else if (!bf16_in) {
+        calls.push_back(make_call(dev, "ar_flash_sage", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, F, F, F, F},
+                                  {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
+    } else {
+        // ar_flash_sage stores f32 (the reference's convention); bf16 tensors get their bf16 result
+        // through one more cast
+        Tensor o32 = Tensor::empty(dev, {b, h, n, d}, F);
+        const Tensor m2 = has_mask ? *attn_mask : o32;
+        calls.push_back(make_call(dev, "ar_flash_sage", {q8, k8, vb, o32, m2, sq, sk}, {I8, I8, BF, F, F, F, F},
+                                  {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
+        const int64_t no = b * h * n * d;
+        calls.push_back(make_call(dev, "ar_cast_bf16", {o32, out}, {F, BF}, {std::min<int64_t>((no + 255) / 256, 16384), 1, 1},
+                                  {256, 1, 1}, {no}, {0}));
+    }
+    return calls;
 }
 
 std::optional<Tensor> fused_attention_ex(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
@@ -242,66 +480,16 @@ std::optional<Tensor> fused_attention_ex(const Tensor &q, const Tensor &k, const
         note_once(sage_note, "[attention] sage: quantized attention is not available for this shape/settings: using the exact kernel");
     if (kern == Kernel::None) return std::nullopt;
 
-    const int64_t b = q.shape()[0], h = q.shape()[1], n = q.shape()[2], d = q.shape()[3], hk = k.shape()[1];
-    auto dev = q.device();
-    const float scale = 1.0f / std::sqrt((float)d);
-    // out: bf16 for bf16 tensors, f32 otherwise (:514-530); no host-side zero fill is needed,
-    // the kernels write every element
-    Tensor out = Tensor::empty(dev, {b, h, n, d}, q.dtype());
-    const Tensor mask = attn_mask ? *attn_mask : Tensor();
-
-    HostCall call;
-    call.device = dev->name();
-    call.global[0] = (n + 63) / 64;  // what the reference's launch would use (BQ = 64)
-    call.global[1] = b * h;
-    call.global[2] = 1;
-    call.vals = {n, d, (int64_t)is_causal, (int64_t)(attn_mask != nullptr), h, hk};
-    call.bufs = {q, k, v, out};
-    if (attn_mask) call.bufs.push_back(mask);
-    const float *mptr = attn_mask ? (const float *)mask.ptr() : nullptr;
-
-    if (kern == Kernel::Sage) {
-        call.name = "ar_flash_sage";
-        const int in_dt = q.dtype() == DType::BFloat16 ? ARHIP_BF16 : ARHIP_F32;
-        const int64_t bq = st.sage_block_q, bk = st.sage_block_k;
-        const bool smooth = st.sage_smooth_k;
-        call.run = [=]() {
-            arhip_device *hd = dev->handle();
-            const int64_t nq = b * h * n * d, nkv = b * hk * n * d;
-            const int64_t nqb = (n + bq - 1) / bq, nkb = (n + bk - 1) / bk;
-            // scratch from the free-list allocator: repeated calls do not reach hipMalloc
-            const size_t ws_bytes = arhip_sage_quant_workspace(b, hk, n, d);
-            void *q8 = dev->alloc((size_t)nq), *k8 = dev->alloc((size_t)nkv);
-            void *sq = dev->alloc((size_t)(b * h * nqb) * 4), *sk = dev->alloc((size_t)(b * hk * nkb) * 4);
-            void *mean = dev->alloc((size_t)(b * hk * d) * 4), *ws = dev->alloc(ws_bytes);
-            void *vb = in_dt == ARHIP_F32 ? dev->alloc((size_t)nkv * 2) : nullptr;
-            dev->check(arhip_sage_quant(hd, q.ptr(), (int8_t *)q8, (float *)sq, nullptr, nullptr, b, h, n, d, bq, in_dt, 0, 0, nullptr));
-            dev->check(arhip_sage_quant(hd, k.ptr(), (int8_t *)k8, (float *)sk, (float *)mean, ws, b, hk, n, d, bk, in_dt,
-                                        smooth ? 1 : 0, 0, nullptr));
-            const uint16_t *vptr = (const uint16_t *)v.ptr();
-            if (vb) {
-                dev->check(arhip_cast_bf16(hd, (const float *)v.ptr(), (uint16_t *)vb, nkv, 0, nullptr));
-                vptr = (const uint16_t *)vb;
-            }
-            dev->check(arhip_sage_fwd(hd, (const int8_t *)q8, (const int8_t *)k8, (const float *)sq, (const float *)sk, vptr,
-                                      out.ptr(), mptr, nullptr, b, h, hk, n, d, bq, bk, is_causal, in_dt, scale, nullptr,
-                                      nullptr, 1, nullptr));
-            dev->release(q8, (size_t)nq); dev->release(k8, (size_t)nkv);
-            dev->release(sq, (size_t)(b * h * nqb) * 4); dev->release(sk, (size_t)(b * hk * nkb) * 4);
-            dev->release(mean, (size_t)(b * hk * d) * 4); dev->release(ws, ws_bytes);
-            if (vb) dev->release(vb, (size_t)nkv * 2);
-        };
-    } else {
-        const int dt = kern == Kernel::FlashBf16 ? ARHIP_BF16 : ARHIP_F32;
-        call.name = kern == Kernel::FlashBf16 ? "ar_flash_bf16" : "ar_flash_f32";
-        call.run = [=]() {
-            dev->check(arhip_flash_fwd(dev->handle(), q.ptr(), k.ptr(), v.ptr(), out.ptr(), mptr, nullptr, b, h, hk, n, d,
-                                       is_causal, dt, scale, 1, nullptr));
-        };
+    const int64_t b = q.shape()[0], h = q.shape()[1], n = q.shape()[2], d = q.shape()[3];
+    // out: bf16 for bf16 tensors, f32 otherwise (:514-530); no host-side zero fill is needed, the
+    // kernels write every element
+    Tensor out = Tensor::empty(q.device(), {b, h, n, d}, q.dtype());
+    // Record the launches for replay and run them now (flash_attention.rs:696-701).
+    for (const HostCall &call : attention_host_calls(q, k, v, attn_mask, out, is_causal, kern, st)) {
+        sess.capture_host(call);
+        call.exec();
     }
-    // Record the launch for replay and run it now (flash_attention.rs:696-701).
-    sess.capture_host(call);
-    call.exec();
+    note_selected(kern);
     return out;
 }
 

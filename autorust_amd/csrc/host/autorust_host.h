@@ -18,8 +18,8 @@
 // std::nullopt and the caller takes its general (SDPA) path, which is outside this build.
 #pragma once
 
+#include <array>
 #include <cstdint>
-#include <functional>
 #include <map>
 #include <memory>
 #include <optional>
@@ -36,7 +36,8 @@ const char *name(AttentionKind k);                       // flash_attention.rs:7
 inline AttentionKind effective(AttentionKind k) { return k; }  // flash_attention.rs:744-746
 AttentionKind attention_kind_from_str(const std::string &s);   // settings.rs:209-213
 
-enum class DType { Float32 = 0, BFloat16 = 1, Other = 2 };
+// Other: anything else a tensor could be; Int8/Int32/Int64 only type scratch buffers and kernel scalars
+enum class DType { Float32 = 0, BFloat16 = 1, Other = 2, Int8 = 3, Int32 = 4, Int64 = 5 };
 
 struct Settings {
     AttentionKind attention = AttentionKind::Flash;  // AUTORUST_ATTN (default flash)
@@ -57,16 +58,33 @@ public:
     Device(const Device &) = delete;
     arhip_device *handle() const { return dev_; }
     std::string name() const { return ordinal_ == 0 ? "HIP" : "HIP:" + std::to_string(ordinal_); }
+    int compute_units() const;
     void *alloc(size_t bytes);   // reuses a cached block of the same size (<= 32 kept per size)
     void release(void *p, size_t bytes);
     uint64_t raw_allocs() const { return raw_allocs_; }
     void check(int rc) const;    // throws "TGERR: ..." on failure
+    // `Compiled::run_host_kernel` (src/runtime/device.rs:383-402) + `Prog::call`
+    // (src/runtime/ops_cuda.rs:930-1019): `src` names the code object (a file path; loaded once and
+    // cached like compile_cached does), arguments follow `signature`: slot < bufs.size() is that
+    // buffer's device pointer, any other slot is vals[slot - bufs.size()] narrowed to the width of
+    // its dtype.  global is the grid in workgroups, local the workgroup shape.  Returns the elapsed
+    // device seconds when wait is set.
+    std::optional<double> run_host_kernel(const std::string &src, const std::string &name,
+                                          const std::vector<std::pair<int64_t, DType>> &signature,
+                                          const std::vector<void *> &bufs, const int64_t global[3],
+                                          const std::optional<std::array<int64_t, 3>> &local,
+                                          const std::vector<int64_t> &vals, bool wait);
 private:
     arhip_device *dev_ = nullptr;
     int ordinal_;
     std::map<size_t, std::vector<void *>> free_;
+    std::map<std::string, void *> modules_;  // code object path -> loaded module
     uint64_t raw_allocs_ = 0;
 };
+
+// Path of the code object with the named attention kernels (autorust_amd/attn_kernels.hsaco):
+// $AUTORUST_HIP_KERNELS, else the file next to this library.
+std::string attention_kernels_src();
 
 struct Storage {  // OpaqueT: base pointer + size, views share it (buffer.rs:32-39)
     std::shared_ptr<Device> dev;
@@ -83,6 +101,7 @@ public:
     static Tensor from_slice(const std::shared_ptr<Device> &dev, const float *data, const std::vector<int64_t> &shape,
                              DType dtype);                       // tensor/mod.rs:1088
     static Tensor empty(const std::shared_ptr<Device> &dev, const std::vector<int64_t> &shape, DType dtype);
+    size_t nbytes() const;
     Tensor reshape(const std::vector<int64_t> &shape) const;     // view: shares storage
     std::vector<float> to_list() const;                          // tensor/mod.rs:695 (bf16 widened to f32)
     const std::vector<int64_t> &shape() const { return shape_; }
@@ -113,14 +132,16 @@ private:
 };
 
 // ---- captured launches ----------------------------------------------------------------
-struct HostCall {              // session.rs:210-256
+struct HostCall {              // session.rs:210-256, field for field
     std::string device;        // "HIP"
-    std::string name;          // kernel entry ("ar_flash_f32", "ar_flash_bf16", "ar_flash_sage")
-    std::vector<Tensor> bufs;  // held so that a replay can resolve them
-    int64_t global[3];         // grid the reference would launch: [ceil(n/BQ), b*h, 1]
-    std::vector<int64_t> vals; // [n, head_dim, causal, has_mask, hq, hkv]
-    std::function<void()> run; // the typed libarhip calls behind this launch
-    void exec() const { run(); }   // always waits, like session.rs:253
+    std::string src;           // the kernel "source": here the path of the gfx950 code object
+    std::string name;          // entry point ("ar_flash_f32", "ar_flash_bf16", "ar_flash_sage", ...)
+    std::vector<std::pair<int64_t, DType>> signature;  // (slot, dtype) argument list
+    std::vector<Tensor> bufs;  // buffers in slot order, held so that a replay can resolve them
+    int64_t global[3];         // launch grid
+    std::optional<std::array<int64_t, 3>> local;       // launch block
+    std::vector<int64_t> vals; // scalar arguments
+    void exec() const;         // run_host_kernel(..., wait = true), session.rs:230-255
 };
 
 class Session {                // session.rs:44-193 (the part the path touches)
@@ -136,6 +157,12 @@ private:
 
 // ---- dispatcher -----------------------------------------------------------------------
 enum class Kernel { None = -1, FlashF32 = ARHIP_K_FLASH_F32, FlashBf16 = ARHIP_K_FLASH_BF16, Sage = ARHIP_K_SAGE };
+
+// The launches one fused attention call consists of, in order (the pre-pass of the quantised
+// path first, the attention kernel last), without running them: the `host_call` builders of
+// src/runtime/cuda_flash{,_bf16,_sage}.rs (cuda_flash_bf16.rs:580-599).
+std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
+                                           const Tensor &out, bool is_causal, Kernel kern, const Settings &st);
 
 // The gates of fused_attention_ex without touching a device (flash_attention.rs:358-472):
 // which kernel would run, or Kernel::None (=> the caller's SDPA).

@@ -119,6 +119,24 @@ int arh_session_step_info(void *s, int i, char *name, int cap, int64_t *global3,
     for (int j = 0; j < 6 && j < (int)c.vals.size(); ++j) vals6[j] = c.vals[(size_t)j];
     return 0;
 }
+// the rest of a captured launch: code object path, workgroup shape, number of buffers / scalars,
+// and the (slot, dtype) signature as pairs
+int arh_session_step_detail(void *s, int i, char *src, int cap, int64_t *local3, int *nbufs, int *nvals, int64_t *sig_pairs,
+                            int sig_cap)
+{
+    auto *b = (SessionBox *)s;
+    if (i < 0 || i >= (int)b->steps.size()) return -1;
+    const HostCall &c = b->steps[(size_t)i];
+    std::strncpy(src, c.src.c_str(), (size_t)cap);
+    for (int j = 0; j < 3; ++j) local3[j] = c.local ? (*c.local)[(size_t)j] : -1;
+    *nbufs = (int)c.bufs.size();
+    *nvals = (int)c.vals.size();
+    for (int j = 0; j < (int)c.signature.size() && 2 * j + 1 < sig_cap; ++j) {
+        sig_pairs[2 * j] = c.signature[(size_t)j].first;
+        sig_pairs[2 * j + 1] = (int64_t)c.signature[(size_t)j].second;
+    }
+    return (int)c.signature.size();
+}
 int arh_session_replay(void *s)
 {
     return guard([&]() -> int {
@@ -143,6 +161,22 @@ void *arh_attention(void *q, void *k, void *v, void *mask, double dropout_p, int
         case 2: return new Tensor(tq.flash_attention_with(tk, tv, tm, dropout_p, is_causal != 0, *ss, s));
         default: return new Tensor(tq.sage_attention_with(tk, tv, tm, dropout_p, is_causal != 0, *ss, s));
         }
+    }, nullptr);
+}
+
+// fused_attention (kind < 0) / fused_attention_kind: the thin wrappers of
+// src/models/flash_attention.rs:292-320.  Returns NULL with an empty error when the kernels
+// decline (the reference's None).
+void *arh_fused_attention(void *q, void *k, void *v, int kind, void *sess, const arh_settings *st)
+{
+    g_err.clear();
+    return guard([&]() -> void * {
+        const Tensor &tq = *(Tensor *)q, &tk = *(Tensor *)k, &tv = *(Tensor *)v;
+        Session &ss = ((SessionBox *)sess)->sess;
+        const Settings s = to_settings(st);
+        std::optional<Tensor> r = kind < 0 ? fused_attention(tq, tk, tv, ss, s)
+                                           : fused_attention_kind(tq, tk, tv, (AttentionKind)kind, ss, s);
+        return r ? (void *)new Tensor(*r) : nullptr;
     }, nullptr);
 }
 

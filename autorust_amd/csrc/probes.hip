@@ -89,3 +89,49 @@ extern "C" __global__ void probe_copy(const uint4 *src, uint4 *dst, long n)
     const long stride = (long)gridDim.x * blockDim.x;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
 }
+
+// Sustained rate of the bf16 matrix instruction on operands taken from memory, with the shader
+// clock it ran at: 8 waves per workgroup issue independent 32x32x16 MFMAs back to back (8 distinct
+// A and B operands, 4 accumulators) and lane 0 of every workgroup records the shader-clock and
+// 100 MHz real-time ticks of the loop.  On random operands the chip lowers its clock to stay
+// inside its power limit, so this is the matrix rate a kernel can reach at best on real data.
+extern "C" __global__ void __launch_bounds__(512) probe_mfma_rate(const uint4 *src, float *out, long long *ticks, int iters)
+{
+    bf16x8 a[8], b[8];
+    for (int j = 0; j < 8; ++j) {
+        a[j] = __builtin_bit_cast(bf16x8, src[(threadIdx.x * 16 + j) & 8191]);
+        b[j] = __builtin_bit_cast(bf16x8, src[(threadIdx.x * 16 + 8 + j) & 8191]);
+    }
+    f32x16 o[4];
+    for (int n = 0; n < 4; ++n)
+        for (int r = 0; r < 16; ++r) o[n][r] = 0.f;
+    const long long t0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j], b[j], o[j & 3], 0, 0, 0);
+    }
+    const long long t1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+    float r = 0.f;
+    for (int n = 0; n < 4; ++n)
+        for (int i = 0; i < 16; ++i) r += o[n][i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = r;
+    if (threadIdx.x == 0) {
+        ticks[blockIdx.x * 2] = t1 - t0;
+        ticks[blockIdx.x * 2 + 1] = r1 - r0;
+    }
+}
+
+// Shader-clock sampler: one wave that, `samples` times, sleeps for a few microseconds and records
+// the shader-clock and real-time (100 MHz) ticks that went by.  Launched on a second stream next
+// to the kernel under test, it reports the clock that kernel actually ran at.
+extern "C" __global__ void probe_clock_sampler(long long *ticks, int samples, int naps)
+{
+    if (threadIdx.x != 0) return;
+    for (int i = 0; i < samples; ++i) {
+        const long long t0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+        for (int k = 0; k < naps; ++k) __builtin_amdgcn_s_sleep(127);
+        const long long t1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+        ticks[2 * i] = t1 - t0;
+        ticks[2 * i + 1] = r1 - r0;
+    }
+}

@@ -77,6 +77,10 @@ def host():
         for f in ("arh_session_free", "arh_session_begin_capture", "arh_session_end_capture", "arh_session_replay"):
             getattr(h, f).argtypes = [vp]
         h.arh_session_step_info.argtypes = [vp, ci, ctypes.c_char_p, ci, i64p, i64p]
+        h.arh_session_step_detail.argtypes = [vp, ci, ctypes.c_char_p, ci, i64p, ctypes.POINTER(ci), ctypes.POINTER(ci),
+                                              i64p, ci]
+        h.arh_fused_attention.restype = vp
+        h.arh_fused_attention.argtypes = [vp, vp, vp, ci, vp, ctypes.POINTER(Settings)]
         h.arh_attention.restype = vp
         h.arh_attention.argtypes = [vp, vp, vp, vp, ctypes.c_double, ci, ci, vp, ctypes.POINTER(Settings)]
         h.arh_plan_fused.argtypes = [i64p, ci, i64p, ci, i64p, ci, ci, ci, ci, i64p, ci, ci, ci, ci,
@@ -141,6 +145,16 @@ class Session:
             raise IndexError(i)
         return name.value.decode(), list(g), list(v)
 
+    def step_detail(self, i):
+        """(code object path, local[3], number of buffers, number of scalars, [(slot, dtype), ...])."""
+        src = ctypes.create_string_buffer(1024)
+        loc, nb, nv = (ctypes.c_int64 * 3)(), ctypes.c_int(), ctypes.c_int()
+        sig = (ctypes.c_int64 * 64)()
+        n = host().arh_session_step_detail(self.h, i, src, 1024, loc, ctypes.byref(nb), ctypes.byref(nv), sig, 64)
+        if n < 0:
+            raise IndexError(i)
+        return src.value.decode(), list(loc), nb.value, nv.value, [(sig[2 * j], sig[2 * j + 1]) for j in range(n)]
+
     def replay(self):
         if host().arh_session_replay(self.h) != 0:
             raise _err()
@@ -198,6 +212,19 @@ class Tensor:
 
     def sage_attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None):
         return self._call(3, k, v, mask, dropout_p, is_causal, sess, settings)
+
+
+def fused_attention(q, k, v, sess, kind=None, settings=None):
+    """`fused_attention` (kind None) / `fused_attention_kind`: a Tensor, or None when the fused
+    kernels decline (src/models/flash_attention.rs:292-320)."""
+    st = settings if settings is not None else Settings.default()
+    h = host().arh_fused_attention(q.h, k.h, v.h, -1 if kind is None else int(kind), sess.h, ctypes.byref(st))
+    if not h:
+        msg = host().arh_last_error()
+        if msg:
+            raise HostError(msg.decode("utf-8", "replace"))
+        return None
+    return Tensor(h)
 
 
 def plan_fused(q, k, v, qd=FLOAT32, kd=None, vd=None, mask=None, mask_dtype=FLOAT32, enable_gqa=False, quantized=False,

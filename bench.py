@@ -106,8 +106,9 @@ class SageWorkload:
         half = self.ops / 2.0
         t_min = half / (PEAK_INT8 * 1e12) + half / (PEAK_BF16 * 1e12)
         ach = self.ops / secs / 1e12
-        return {"bound": "mfma", "achieved": ach, "peak": PEAK_INT8, "unit": "TFLOP/s", "frac": ach / PEAK_INT8,
-                "traffic": MEASURED_TRAFFIC.get(self.name), "kernel": "attn_fwd_kernel<int8>", "launch_ms": secs * 1e3,
+        return {"bound": "mfma", "achieved": ach, "peak": PEAK_INT8, "unit": "TOP/s", "frac": ach / PEAK_INT8,
+                "traffic": MEASURED_TRAFFIC.get(self.name), "traffic_source": "rocprofv3 --pmc profile (profiles/), not this run",
+                "kernel": "attn_pipe_kernel<int8>", "launch_ms": secs * 1e3,
                 "ops_per_launch": self.ops, "peak_note": "dense int8 MFMA; half of the ops are bf16 (P.V)",
                 "frac_of_mixed_int8_bf16_bound": t_min / secs}
 
@@ -140,6 +141,11 @@ class FlashWorkload:
             self.kv_host = synth.randint(base + 5, B, S // 2, S)
             self.kv = dev.from_numpy(self.kv_host)
         self.ops = attn_ops(B, H, S, D, causal)
+        if kv_lens:
+            # visible (query, key) pairs: key j < L[b] and, under the causal mask, j <= i
+            q = np.arange(S, dtype=np.int64)
+            pairs = sum(int(np.minimum(q + 1, int(L)).sum()) if causal else S * int(L) for L in self.kv_host)
+            self.ops = 4.0 * H * D * pairs
         self.kernel = _lib.K_FLASH_BF16 if dtype == BF16 else _lib.K_FLASH_F32
         self.kernel_bytes = 4 * n * es
         self.dtype = tag
@@ -154,8 +160,8 @@ class FlashWorkload:
         if self.dt == BF16 and ai > PEAK_BF16 * 1e12 / (PEAK_HBM * 1e9):
             ach = self.ops / secs / 1e12
             return {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16, "unit": "TFLOP/s", "frac": ach / PEAK_BF16,
-                    "traffic": None, "kernel": "attn_fwd_kernel<bf16>", "launch_ms": secs * 1e3,
-                    "ops_per_launch": self.ops}
+                    "traffic": None, "kernel": "attn_pipe_kernel<bf16>" if self.S > 256 else "attn_fwd_kernel<bf16>",
+                    "launch_ms": secs * 1e3, "ops_per_launch": self.ops}
         ach = self.kernel_bytes / secs / 1e9
         return {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
                 "traffic": None, "kernel": "attn_fwd_kernel<bf16>" if self.dt == BF16 else "flash_f32_kernel",
@@ -189,6 +195,57 @@ def measure(dev, w, steps, warmup):
     if qn:
         res["prepass_ms_per_step"] = qsecs / steps * 1e3
     return res
+
+
+def _probes(dev):
+    return dev.module_load(open(_lib.PROBES_PATH, "rb").read())
+
+
+def sustained_mfma(dev):
+    """Dense bf16 MFMA rate and shader clock of a loop of nothing but matrix instructions, on
+    constant and on random operands (probe_mfma_rate in csrc/probes.hip): what the power limit
+    leaves of the published peak."""
+    mod = _probes(dev)
+    out, ticks = dev.alloc(256 * 512 * 4), dev.alloc(256 * 16)
+    res = {}
+    for name, data in (("constant", np.full(8192 * 8, 0x3F80, np.uint16)),
+                       ("random", synth.to_bf16_bits(synth.normal(99, (8192 * 8,))))):
+        src = dev.from_numpy(data)
+        iters = 100000
+        dev.launch(mod, "probe_mfma_rate", (256, 1, 1), (512, 1, 1), [src, out, ticks], [iters])
+        t = dev.launch(mod, "probe_mfma_rate", (256, 1, 1), (512, 1, 1), [src, out, ticks], [iters])
+        c = ticks.copyout(np.int64, (256, 2))
+        res[name] = {"tflops": 256 * 8 * iters * 8 * 32768 / t / 1e12,
+                     "shader_clock_mhz": float((c[:, 0] / c[:, 1]).mean() * 100.0)}
+        src.free()
+    out.free()
+    ticks.free()
+    return res
+
+
+def shader_clock_during(dev, w, steps):
+    """Median shader clock (MHz) while `steps` steps of the workload run: a one-wave sampler
+    (probe_clock_sampler) on a second stream beside them.  Not part of the timed region."""
+    side = Device(dev.ordinal)
+    try:
+        mod = _probes(side)
+        samples = 64
+        ticks = side.alloc(samples * 16)
+        ticks.zero()
+        side.sync()
+        w.step()
+        dev.sync()
+        side.launch(mod, "probe_clock_sampler", (1, 1, 1), (64, 1, 1), [ticks], [samples, 40], wait=False)
+        for _ in range(steps):
+            w.step()
+        dev.sync()
+        side.sync()
+        c = ticks.copyout(np.int64, (samples, 2)).astype(np.float64)
+        ticks.free()
+        mhz = c[:, 0] / np.maximum(c[:, 1], 1.0) * 100.0
+        return float(np.median(mhz[: max(4, samples // 2)]))
+    finally:
+        side.close()
 
 
 def cpu_baseline(w, budget_heads):
@@ -254,6 +311,7 @@ def main():
                     help="one step of the workload plus one plain 1 GiB copy kernel and nothing else: "
                          "the run to put under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-clock", action="store_true", help="skip the shader-clock and sustained-MFMA probes")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -275,6 +333,8 @@ def main():
                           "copy_bytes_read": n16 * 16, "copy_bytes_written": n16 * 16}))
         return
     res = measure(dev, w, args.steps, args.warmup)
+    if w.S >= 1024 and not args.no_clock:
+        res["roofline"]["shader_clock_mhz_under_load"] = shader_clock_during(dev, w, max(4, args.steps // 2))
     log(json.dumps(res))
     cpu = None
     if not args.no_cpu:
@@ -292,11 +352,14 @@ def main():
                 continue
             sw = build_workload(dev, name)
             r = measure(dev, sw, max(args.steps, 20) if sw.S < 1024 else args.steps, args.warmup)
+            if sw.S >= 1024 and not args.no_clock:
+                r["roofline"]["shader_clock_mhz_under_load"] = shader_clock_during(dev, sw, max(4, args.steps // 2))
             if name in REFERENCE_RTX3060_MS:
                 r["reference_kernel_ms_rtx3060"] = REFERENCE_RTX3060_MS[name]
             sw.free()
             log(json.dumps(r))
             secondary.append(r)
+    power = None if args.no_clock else sustained_mfma(dev)
     dev.close()
 
     line = {
@@ -313,6 +376,13 @@ def main():
     }
     if "prepass_ms_per_step" in res:
         line["prepass_ms_per_step"] = res["prepass_ms_per_step"]
+    if power is not None:
+        # the published peaks assume 2.4 GHz; under a matrix load on random data the chip clocks down
+        line["power_limit_probe"] = {"kernel": "probe_mfma_rate (bf16 32x32x16 MFMAs only, 2 waves per SIMD)",
+                                     "constant_operands": power["constant"], "random_operands": power["random"]}
+        line["roofline"]["frac_of_sustained_bf16_mfma_rate"] = (
+            (res["ops_per_step"] / 2 / (PEAK_INT8 / PEAK_BF16) + res["ops_per_step"] / 2) if w.dtype == "int8"
+            else res["ops_per_step"]) / (line["roofline"]["launch_ms"] * 1e-3) / 1e12 / power["random"]["tflops"]
     if secondary:
         line["secondary"] = secondary
     print(json.dumps(line), flush=True)

@@ -167,6 +167,47 @@ def test_fallback_is_reported_not_faked(hdev):
 
 
 @gpu
+def test_fused_attention_wrappers(hdev):
+    """fused_attention / fused_attention_kind (src/models/flash_attention.rs:292-320): no mask, not
+    causal, no GQA; a Tensor when a fused kernel runs, None when the kernels decline."""
+    b, h, n, d = 2, 3, 130, 64
+    q, k, v = _fill((b, h, n, d), 3), _fill((b, h, n, d), 11), _fill((b, h, n, d), 19)
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v))
+    sess = Session()
+    before = host.selections(K_FLASH_F32)
+    out = host.fused_attention(tq, tk, tv, sess)
+    assert out is not None and host.selections(K_FLASH_F32) == before + 1
+    assert float(np.abs(out.to_list() - oracle.flash_f32(q, k, v)).max()) < 2e-5      # tests/flash_cuda.rs:74
+    before = host.selections(K_SAGE)
+    out = host.fused_attention(tq, tk, tv, sess, kind=AttentionKind.Sage)
+    assert out is not None and host.selections(K_SAGE) == before + 1
+    assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v)).max()) < 2e-2
+    out = host.fused_attention(tq, tk, tv, sess, kind=AttentionKind.Flash)
+    assert float(np.abs(out.to_list() - oracle.flash_f32(q, k, v)).max()) < 2e-5
+    # head_dim 32 has no fused kernel: None, not an error (flash_attention.rs:470-472)
+    q32 = _fill((1, 2, 16, 32), 3)
+    t32 = Tensor.from_slice(hdev, q32, q32.shape)
+    assert host.fused_attention(t32, t32, t32, sess) is None
+    # fewer K/V heads without enable_gqa: the wrappers pass enable_gqa = false, so they decline
+    tk2 = Tensor.from_slice(hdev, k[:, :1], (b, 1, n, d))
+    assert host.fused_attention(tq, tk2, tk2, sess) is None
+
+
+@gpu
+def test_attention_debug_line_and_kernel_info(hdev, capfd, monkeypatch):
+    """AUTORUST_ATTN_DEBUG prints one line per kernel on its first dispatch
+    (src/runtime/cuda_flash_bf16.rs:446-456)."""
+    monkeypatch.setenv("AUTORUST_ATTN_DEBUG", "1")
+    q = _fill((1, 2, 64, 64), 3)
+    t = Tensor.from_slice(hdev, q, q.shape, BFLOAT16)
+    sess = Session()
+    t.flash_attention_with(t, t, None, 0.0, False, sess)
+    t.flash_attention_with(t, t, None, 0.0, False, sess)
+    err = capfd.readouterr().err
+    assert err.count("[attention] flash: bf16 MFMA") <= 1      # at most once per process
+
+
+@gpu
 def test_capture_and_replay(hdev):
     """Session::capture_host + Jit replay (session.rs:138-146, jit.rs:186-195): the captured launch
     re-runs on the same buffers and reproduces the result; the allocator serves repeats from its
@@ -178,10 +219,20 @@ def test_capture_and_replay(hdev):
     sess.begin_capture()
     out = tq.attention_with(tk, tv, None, 0.0, True, sess)
     o2 = tq.sage_attention_with(tk, tv, None, 0.0, True, sess)
-    assert sess.end_capture() == 2
+    nsteps = sess.end_capture()
+    # one launch for flash; for Sage the pre-pass launches (quantise Q, K mean in two steps, quantise
+    # K), the attention kernel and the f32 -> bf16 cast of its output, each a HostCall of its own
+    names = [sess.step(i)[0] for i in range(nsteps)]
+    assert names == ["ar_flash_bf16", "ar_sage_quant_blocks_bf16", "ar_sage_kmean_partial_bf16", "ar_sage_kmean_final",
+                     "ar_sage_quant_blocks_bf16", "ar_flash_sage", "ar_cast_bf16"]
     name, grid, vals = sess.step(0)
-    assert name == "ar_flash_bf16" and grid == [(n + 63) // 64, b * h, 1] and vals == [n, d, 1, 0, h, h]
-    assert sess.step(1)[0] == "ar_flash_sage"
+    # grid [query tiles of 128, b*h, 1], vals [n, head_dim, causal, has_mask, hq, hkv] (cuda_flash_bf16.rs:550-599)
+    assert grid == [(n + 127) // 128, b * h, 1] and vals == [n, d, 1, 0, h, h]
+    src, local, nbufs, nvals, sig = sess.step_detail(0)
+    assert src.endswith("attn_kernels.hsaco") and local == [256, 1, 1] and (nbufs, nvals) == (5, 6)
+    BF, F, I32 = 1, 0, 4
+    assert sig == [(0, BF), (1, BF), (2, BF), (3, BF), (4, F)] + [(5 + i, I32) for i in range(6)]   # cuda_flash_bf16.rs:563-578
+    assert sess.step(5)[2] == [n, d, 1, 0, h, h] and sess.step_detail(5)[2:4] == (7, 8)
     first = out.to_list().copy()
     first2 = o2.to_list().copy()
     allocs = hdev.raw_allocs
