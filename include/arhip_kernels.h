@@ -1,0 +1,73 @@
+/*
+ * Entry points of the loadable gfx950 code object autorust_amd/attn_kernels.hsaco
+ * (built from autorust_amd/csrc/attn_entry.hip).
+ *
+ * This is the second face of the boundary: hosts that launch kernels by name, the way the
+ * reference's `HostCall{src, name, signature, bufs, global, local, vals}` ->
+ * `Compiled::run_host_kernel` -> `Prog::call` does (src/engine/session.rs:210-256,
+ * src/runtime/device.rs:383-402), load the code object with arhip_module_load (or
+ * hipModuleLoadData) and launch these with arhip_launch (or hipModuleLaunchKernel).
+ * Arguments are device pointers followed by scalars, in the reference's order
+ * (src/runtime/cuda_flash_bf16.rs:226-231, 550-599):
+ *
+ *     (Q, K, V, O, M,   int N, int head_dim, int causal, int has_mask, int hq, int hkv)
+ *     vals = [n, head_dim, causal, has_mask, hq, hkv]
+ *
+ * Tensors are dense [B, H, N, D]; M (f32 [N, N], additive) is read only when has_mask != 0
+ * (pass O again otherwise, as the reference does: src/runtime/cuda_flash.rs:233-240); B follows
+ * from the grid (grid.y = B * hq <= 65535); scale = 1/sqrt(head_dim); head_dim is 64 or 128.
+ * The grid is in workgroups: [ceil(N / ARHIP_KQ_*), B * hq, 1].
+ */
+#ifndef ARHIP_KERNELS_H
+#define ARHIP_KERNELS_H
+
+/* queries per workgroup and workgroup size of the two tilings */
+#define ARHIP_KQ_GENERAL 128 /* block [256,1,1] */
+#define ARHIP_KQ_LONG 256    /* block [512,1,1] */
+
+/* fp32 exact mode: replaces `ar_flash_f32`, src/runtime/cuda_flash.rs:53-141.
+ * (const float *Q, *K, *V, float *O, const float *M, 6 ints); general tiling. */
+#define ARHIP_KERNEL_FLASH_F32 "ar_flash_f32"
+
+/* bf16: replaces `ar_flash_bf16`, src/runtime/cuda_flash_bf16.rs:226-427.
+ * (const bf16 *Q, *K, *V, bf16 *O, const float *M, 6 ints); general tiling, any mask. */
+#define ARHIP_KERNEL_FLASH_BF16 "ar_flash_bf16"
+/* the software-pipelined variant for long sequences: same arguments, has_mask must be 0,
+ * (N + 320) * head_dim * 2 < 2^31; long tiling. */
+#define ARHIP_KERNEL_FLASH_BF16_LONG "ar_flash_bf16_long"
+
+/* Sage int8: replaces `ar_flash_sage`, src/runtime/cuda_flash_sage.rs:168-414, on pre-quantised
+ * operands (the quantiser is the pre-pass below):
+ * (const int8 *Q8, *K8, const bf16 *V, float *O, const float *M, const float *SQ, const float *SK,
+ *  6 ints, int bq, int bk); SQ [B,hq,ceil(N/bq)], SK [B,hkv,ceil(N/bk)]; any bq, bk >= 1 (1 = the
+ * reference's per-row scales); O is f32 like the reference's; general tiling. */
+#define ARHIP_KERNEL_FLASH_SAGE "ar_flash_sage"
+/* pipelined variant: has_mask 0, bk = 64 * 2^n; one more int `out_f32` (O is f32 when set,
+ * bf16 otherwise); long tiling. */
+#define ARHIP_KERNEL_FLASH_SAGE_LONG "ar_flash_sage_long"
+
+/* Sage pre-pass (src/runtime/cuda_flash_sage.rs:124-137, 201-223 hoisted out of the attention
+ * kernel; K smoothing is an extension).  x is [B*H, N, D]; block [256,1,1] unless noted.
+ *   ar_sage_kmean_partial_{f32,bf16}(x, float *part, int N, int D, int nchunk)
+ *        grid [ceil(nchunk / (256 / (D/8))), B*H, 1], nchunk = ceil(N/64); part [B*H, nchunk, D]
+ *   ar_sage_kmean_final(const float *part, float *mean, int N, int D, int nchunk)
+ *        grid [B*H, 1, 1], block [D, 1, 1]; mean [B*H, D]
+ *   ar_sage_quant_blocks_{f32,bf16}(x, int8 *x8, float *scales, const float *mean,
+ *                                   int N, int D, int blk, int nblk, int smooth)
+ *        grid [nblk, B*H, 1]; scales [B*H, nblk]
+ *   ar_sage_quant_rows_{f32,bf16}(x, int8 *x8, float *scales, const float *mean,
+ *                                 int N, int D, long rows_total, int smooth)
+ *        grid [ceil(rows_total / (256 / (D/8))), 1, 1]; rows_total = B*H*N (a 64-bit scalar)
+ *   ar_cast_bf16(const float *x, bf16 *y, long n)
+ *        grid [min(ceil(n/256), 16384), 1, 1]
+ */
+#define ARHIP_KERNEL_SAGE_KMEAN_PARTIAL_F32 "ar_sage_kmean_partial_f32"
+#define ARHIP_KERNEL_SAGE_KMEAN_PARTIAL_BF16 "ar_sage_kmean_partial_bf16"
+#define ARHIP_KERNEL_SAGE_KMEAN_FINAL "ar_sage_kmean_final"
+#define ARHIP_KERNEL_SAGE_QUANT_BLOCKS_F32 "ar_sage_quant_blocks_f32"
+#define ARHIP_KERNEL_SAGE_QUANT_BLOCKS_BF16 "ar_sage_quant_blocks_bf16"
+#define ARHIP_KERNEL_SAGE_QUANT_ROWS_F32 "ar_sage_quant_rows_f32"
+#define ARHIP_KERNEL_SAGE_QUANT_ROWS_BF16 "ar_sage_quant_rows_bf16"
+#define ARHIP_KERNEL_CAST_BF16 "ar_cast_bf16"
+
+#endif /* ARHIP_KERNELS_H */

@@ -1,0 +1,235 @@
+//! Fused attention on the `HIP` device: the `host_call` builders that stand where
+//! `cuda_flash::host_call`, `cuda_flash_bf16::host_call` and `cuda_flash_sage::host_call` stand
+//! for CUDA (`src/runtime/cuda_flash.rs:283-304`, `cuda_flash_bf16.rs:580-599`,
+//! `cuda_flash_sage.rs:487-535`).  Shipped as source; see `ops_hip.rs` for how it was checked.
+//!
+//! The kernels live in a prebuilt gfx950 code object (`attn_kernels.hsaco`, built from
+//! `csrc/attn_entry.hip`).  A `HostCall`'s `src` is that file's path, its `name` one of the entry
+//! points below, and `exec` launches it through `Compiled::run_host_kernel` unchanged.
+//!
+//! | entry                | block | grid                    | arguments after the buffers                  |
+//! |----------------------|-------|-------------------------|----------------------------------------------|
+//! | `ar_flash_f32`       | 256   | `[ceil(n/128), b*h, 1]` | `n, head_dim, causal, has_mask, hq, hkv`     |
+//! | `ar_flash_bf16`      | 256   | `[ceil(n/128), b*h, 1]` | same                                         |
+//! | `ar_flash_bf16_long` | 512   | `[ceil(n/256), b*h, 1]` | same (`has_mask` must be 0)                  |
+//! | `ar_flash_sage`      | 256   | `[ceil(n/128), b*h, 1]` | same `+ bq, bk`; buffers `+ SQ, SK`; O is f32|
+//! | `ar_flash_sage_long` | 512   | `[ceil(n/256), b*h, 1]` | same `+ bq, bk, out_f32`                     |
+//!
+//! Unlike the CUDA Sage kernel, which quantises inside the attention kernel (K once per query
+//! block, `cuda_flash_sage.rs:248-278`), the quantiser is a pre-pass of its own here, with K
+//! smoothing and per-block scales (128 query tokens / 64 key tokens by default).  A Sage call is
+//! therefore a short sequence of `HostCall`s; their scratch buffers ride in `bufs`, so a JIT
+//! replay finds them again.
+
+use crate::dtype::{self, DTypeId};
+use crate::engine::session::HostCall;
+use crate::runtime::buffer::Buffer;
+use std::sync::atomic::{AtomicU64, Ordering};
+
+/// Path of the code object: `$AUTORUST_HIP_KERNELS`, else next to the executable.
+pub fn src() -> String {
+    if let Some(p) = crate::helpers::env::get_os("AUTORUST_HIP_KERNELS") {
+        return p.to_string_lossy().into_owned();
+    }
+    let exe = std::env::current_exe().ok();
+    let dir = exe.as_deref().and_then(|p| p.parent()).unwrap_or(std::path::Path::new("."));
+    dir.join("attn_kernels.hsaco").to_string_lossy().into_owned()
+}
+
+/// Per-call switches, as `cuda_flash_bf16::Options` (`cuda_flash_bf16.rs:463-476`).
+#[derive(Clone, Copy, Debug)]
+pub struct Options {
+    pub causal: bool,
+    pub has_mask: bool,
+    pub h_kv: i64,
+}
+
+/// Sage quantiser settings (extensions of this device; block 1 / no smoothing reproduces the
+/// CUDA kernel's per-row rule, `cuda_flash_sage.rs:209-222`).
+#[derive(Clone, Copy, Debug)]
+pub struct SageOptions {
+    pub block_q: i64,
+    pub block_k: i64,
+    pub smooth_k: bool,
+}
+
+impl Default for SageOptions {
+    fn default() -> Self {
+        SageOptions { block_q: 128, block_k: 64, smooth_k: true }
+    }
+}
+
+/// `supports` / `supported` gates (`cuda_flash.rs:145-147`, `cuda_flash_bf16.rs:431-441`,
+/// `cuda_flash_sage.rs:69-74`): head_dim 64 or 128, any n > 0, and a grid that fits.
+pub fn supported(b: i64, h: i64, n: i64, d: i64) -> bool {
+    n > 0 && n <= 1 << 24 && (d == 64 || d == 128) && b > 0 && h > 0 && b * h <= 65535
+}
+
+static SELECTED: [AtomicU64; 3] = [AtomicU64::new(0), AtomicU64::new(0), AtomicU64::new(0)];
+
+/// Which kernel family a call went to: 0 fp32 exact, 1 bf16, 2 Sage int8.
+pub fn note_selected(kind: usize) {
+    SELECTED[kind].fetch_add(1, Ordering::Relaxed);
+    static ONCE: [std::sync::Once; 3] = [std::sync::Once::new(), std::sync::Once::new(), std::sync::Once::new()];
+    ONCE[kind].call_once(|| {
+        if crate::helpers::env::get_os("AUTORUST_ATTN_DEBUG").is_some() {
+            eprintln!(
+                "{}",
+                [
+                    "[attention] flash: fp32 exact, fp32 MFMA (gfx950)",
+                    "[attention] flash: bf16 MFMA, software-pipelined for long sequences (gfx950)",
+                    "[attention] sage: int8 MFMA for q.k^T, bf16 MFMA for p.v, K smoothing + block scales (gfx950)",
+                ][kind]
+            );
+        }
+    });
+}
+
+/// Calls dispatched to a kernel family since process start (`cuda_flash_bf16.rs:458-461`).
+pub fn selections(kind: usize) -> u64 {
+    SELECTED[kind].load(Ordering::Relaxed)
+}
+
+fn signature(buf_types: &[DTypeId], nvals: usize, wide: &[usize]) -> Vec<(i64, DTypeId)> {
+    let mut s: Vec<(i64, DTypeId)> = buf_types.iter().enumerate().map(|(i, t)| (i as i64, *t)).collect();
+    for i in 0..nvals {
+        let t = if wide.contains(&i) { dtype::INT64 } else { dtype::INT32 };
+        s.push(((buf_types.len() + i) as i64, t));
+    }
+    s
+}
+
+#[allow(clippy::too_many_arguments)]
+fn call(name: &str, bufs: Vec<Buffer>, buf_types: &[DTypeId], global: [i64; 3], local: [i64; 3], vals: Vec<i64>, wide: &[usize]) -> HostCall {
+    HostCall {
+        device: "HIP".into(),
+        src: src(),
+        name: name.to_string(),
+        signature: signature(buf_types, vals.len(), wide),
+        bufs,
+        global,
+        local: Some(local),
+        vals,
+    }
+}
+
+fn vals(n: i64, d: i64, h: i64, opts: Options) -> Vec<i64> {
+    // `cuda_flash_bf16.rs:550-561`, with the head size as a real parameter
+    vec![n, d, opts.causal as i64, opts.has_mask as i64, h, opts.h_kv]
+}
+
+/// The pipelined kernels want enough workgroups of 256 queries to fill the chip twice and
+/// address K/V with 32-bit byte offsets.
+fn long_variant(dev: &str, b: i64, h: i64, n: i64, d: i64) -> bool {
+    let cus = crate::runtime::ops_hip::compute_units(dev);
+    b * h * ((n + 255) / 256) >= 2 * cus && (n + 320) * d * 2 < 1 << 31
+}
+
+/// fp32 exact mode: `bufs = [q, k, v, o, mask-or-o]`, all f32 `[b, h, n, d]`.
+pub fn host_call_f32(bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
+    let f = dtype::FLOAT32;
+    call("ar_flash_f32", bufs, &[f, f, f, f, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+}
+
+/// bf16: `bufs = [q, k, v, o, mask-or-o]`, q/k/v/o bf16, mask f32 `[n, n]`.
+pub fn host_call_bf16(dev: &str, bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
+    let (bf, f) = (dtype::BFLOAT16, dtype::FLOAT32);
+    if !opts.has_mask && long_variant(dev, b, h, n, d) {
+        call("ar_flash_bf16_long", bufs, &[bf, bf, bf, bf, f], [(n + 255) / 256, b * h, 1], [512, 1, 1], vals(n, d, h, opts), &[])
+    } else {
+        call("ar_flash_bf16", bufs, &[bf, bf, bf, bf, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+    }
+}
+
+/// Scratch tensors of one Sage call; the dispatcher allocates them (uninitialised is enough)
+/// and passes their realised buffers.
+pub struct SageScratch {
+    pub q8: Buffer,   // int8 [b, h, n, d]
+    pub k8: Buffer,   // int8 [b, hkv, n, d]
+    pub sq: Buffer,   // f32 [b, h, ceil(n / block_q)]
+    pub sk: Buffer,   // f32 [b, hkv, ceil(n / block_k)]
+    pub mean: Buffer, // f32 [b, hkv, d]
+    pub part: Buffer, // f32 [b, hkv, ceil(n / 64), d]  (partial sums of the K mean)
+    pub vb: Option<Buffer>,  // bf16 copy of v when the tensors are f32
+    pub o32: Option<Buffer>, // f32 result when the tensors are bf16 and the general kernel runs
+}
+
+/// Sage int8: the launches of one call, in order.  `q, k, v, o` are f32 or bf16 (`bf16_in`),
+/// `mask` is the f32 `[n, n]` additive mask or `o` again.
+#[allow(clippy::too_many_arguments)]
+pub fn host_calls_sage(
+    dev: &str,
+    q: Buffer,
+    k: Buffer,
+    v: Buffer,
+    o: Buffer,
+    mask: Buffer,
+    s: SageScratch,
+    bf16_in: bool,
+    b: i64,
+    h: i64,
+    n: i64,
+    d: i64,
+    opts: Options,
+    sage: SageOptions,
+) -> Vec<HostCall> {
+    let (f, bf, i8t) = (dtype::FLOAT32, dtype::BFLOAT16, dtype::INT8);
+    let x = if bf16_in { bf } else { f };
+    let sfx = if bf16_in { "bf16" } else { "f32" };
+    let hk = opts.h_kv;
+    let (bq, bk) = (sage.block_q, sage.block_k);
+    let (nqb, nkb, nchunk) = ((n + bq - 1) / bq, (n + bk - 1) / bk, (n + 63) / 64);
+    let mut calls = Vec::new();
+    let mut quant = |src: &Buffer, dst: &Buffer, scales: &Buffer, heads: i64, blk: i64, nblk: i64, smooth: bool| {
+        let bufs = vec![src.clone(), dst.clone(), scales.clone(), s.mean.clone()];
+        if blk == 1 {
+            let rows = b * heads * n;
+            let rpb = 256 / (d / 8);
+            calls.push(call(&format!("ar_sage_quant_rows_{sfx}"), bufs, &[x, i8t, f, f], [(rows + rpb - 1) / rpb, 1, 1], [256, 1, 1],
+                            vec![n, d, rows, smooth as i64], &[2]));
+        } else {
+            calls.push(call(&format!("ar_sage_quant_blocks_{sfx}"), bufs, &[x, i8t, f, f], [nblk, b * heads, 1], [256, 1, 1],
+                            vec![n, d, blk, nblk, smooth as i64], &[]));
+        }
+    };
+    quant(&q, &s.q8, &s.sq, h, bq, nqb, false);
+    if sage.smooth_k {
+        let cpb = 256 / (d / 8);
+        calls.push(call(&format!("ar_sage_kmean_partial_{sfx}"), vec![k.clone(), s.part.clone()], &[x, f],
+                        [(nchunk + cpb - 1) / cpb, b * hk, 1], [256, 1, 1], vec![n, d, nchunk], &[]));
+        calls.push(call("ar_sage_kmean_final", vec![s.part.clone(), s.mean.clone()], &[f, f], [b * hk, 1, 1], [d, 1, 1],
+                        vec![n, d, nchunk], &[]));
+    }
+    quant(&k, &s.k8, &s.sk, hk, bk, nkb, sage.smooth_k);
+    let vb = match &s.vb {
+        Some(vb) => {
+            let nv = b * hk * n * d;
+            calls.push(call("ar_cast_bf16", vec![v.clone(), vb.clone()], &[f, bf], [((nv + 255) / 256).min(16384), 1, 1], [256, 1, 1],
+                            vec![nv], &[0]));
+            vb.clone()
+        }
+        None => v.clone(),
+    };
+    let mut sv = vals(n, d, h, opts);
+    sv.push(bq);
+    sv.push(bk);
+    let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
+    if !opts.has_mask && tile_uniform && long_variant(dev, b, h, n, d) {
+        sv.push(!bf16_in as i64); // out_f32
+        calls.push(call("ar_flash_sage_long", vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f],
+                        [(n + 255) / 256, b * h, 1], [512, 1, 1], sv, &[]));
+    } else if !bf16_in {
+        calls.push(call("ar_flash_sage", vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f],
+                        [(n + 127) / 128, b * h, 1], [256, 1, 1], sv, &[]));
+    } else {
+        // the general kernel stores f32 (the CUDA kernel's convention); bf16 tensors get their
+        // bf16 result through one more cast
+        let o32 = s.o32.expect("o32 scratch for bf16 tensors");
+        let m2 = if opts.has_mask { mask } else { o32.clone() };
+        calls.push(call("ar_flash_sage", vec![s.q8, s.k8, vb, o32.clone(), m2, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f],
+                        [(n + 127) / 128, b * h, 1], [256, 1, 1], sv, &[]));
+        let no = b * h * n * d;
+        calls.push(call("ar_cast_bf16", vec![o32, o], &[f, bf], [((no + 255) / 256).min(16384), 1, 1], [256, 1, 1], vec![no], &[0]));
+    }
+    calls
+}

@@ -75,3 +75,13 @@ def test_workspace_size():
     assert lib.arhip_sage_quant_workspace(4, 32, 8192, 128) == 4 * 32 * 128 * 128 * 4
     assert lib.arhip_sage_quant_workspace(1, 1, 65, 64) == 2 * 64 * 4
     assert lib.arhip_sage_quant_workspace(0, 1, 65, 64) == 0
+
+
+def test_code_object_is_built_and_names_every_entry_point():
+    """The named kernels (include/arhip_kernels.h) are all in the code object (no launch here)."""
+    text = open(os.path.join(ROOT, "include", "arhip_kernels.h")).read()
+    names = re.findall(r'#define ARHIP_KERNEL_\w+ "(\w+)"', text)
+    assert len(names) == 13
+    image = open(_lib.KERNELS_PATH, "rb").read()
+    for n in names:
+        assert n.encode() + b"\0" in image or n.encode() in image, n
