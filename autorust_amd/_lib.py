@@ -64,6 +64,8 @@ SIGNATURES = {
     "arhip_sage_quant_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "arhip_sage_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),
+    "arhip_sage_quant_strided": (c_int, [c_void_p, c_void_p, ctypes.POINTER(c_int64), c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),
     "arhip_sage_quant_static_limit": (c_size_t, []),
     "arhip_sage_quant_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),
@@ -71,6 +73,10 @@ SIGNATURES = {
     "arhip_sage_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_float,
                                c_void_p, ctypes.POINTER(ctypes.c_int32), c_int, _pd]),
+    "arhip_sage_fwd_strided": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), c_void_p, c_void_p,
+                                       c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_float,
+                                       c_void_p, ctypes.POINTER(ctypes.c_int32), c_int, _pd]),
     "arhip_selections": (ctypes.c_uint64, [c_int]),
 }
 

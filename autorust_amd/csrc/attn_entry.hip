@@ -51,6 +51,7 @@ __device__ __forceinline__ AttnParams dense_params(const void *q, const void *k,
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     dense(p.qs, hq, N, D);
     dense(p.ks, hkv, N, D);
+    dense(p.vs, hkv, N, D);
     dense(p.os, hq, N, D);
     p.bq = p.bk = 1;
     p.nq = (int)gridDim.x;
@@ -201,11 +202,11 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_
 // smooth != 0 subtracts mean[bh][d] first (K smoothing).
 extern "C" __global__ void __launch_bounds__(256) ar_sage_kmean_partial_f32(const float *x, float *part, int N, int D, int nchunk)
 {
-    k_mean_partial_body<float>(x, part, N, D, nchunk, blockIdx);
+    k_mean_partial_body<float>(x, part, N, D, nchunk, XLayout::dense(1, N, D), blockIdx);
 }
 extern "C" __global__ void __launch_bounds__(256) ar_sage_kmean_partial_bf16(const uint16_t *x, float *part, int N, int D, int nchunk)
 {
-    k_mean_partial_body<uint16_t>(x, part, N, D, nchunk, blockIdx);
+    k_mean_partial_body<uint16_t>(x, part, N, D, nchunk, XLayout::dense(1, N, D), blockIdx);
 }
 extern "C" __global__ void ar_sage_kmean_final(const float *part, float *mean, int N, int D, int nchunk)
 {
@@ -215,29 +216,29 @@ extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_blocks_f32(const
                                                                             const float *mean, int N, int D, int blk, int nblk,
                                                                             int smooth)
 {
-    if (smooth) quant_blocks_body<float, true>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
-    else quant_blocks_body<float, false>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
+    if (smooth) quant_blocks_body<float, true>(x, x8, scales, mean, N, D, blk, nblk, XLayout::dense(1, N, D), blockIdx);
+    else quant_blocks_body<float, false>(x, x8, scales, mean, N, D, blk, nblk, XLayout::dense(1, N, D), blockIdx);
 }
 extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_blocks_bf16(const uint16_t *x, int8_t *x8, float *scales,
                                                                              const float *mean, int N, int D, int blk, int nblk,
                                                                              int smooth)
 {
-    if (smooth) quant_blocks_body<uint16_t, true>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
-    else quant_blocks_body<uint16_t, false>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
+    if (smooth) quant_blocks_body<uint16_t, true>(x, x8, scales, mean, N, D, blk, nblk, XLayout::dense(1, N, D), blockIdx);
+    else quant_blocks_body<uint16_t, false>(x, x8, scales, mean, N, D, blk, nblk, XLayout::dense(1, N, D), blockIdx);
 }
 extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_f32(const float *x, int8_t *x8, float *scales,
                                                                           const float *mean, int N, int D, long rows_total,
                                                                           int smooth)
 {
-    if (smooth) quant_rows_body<float, true>(x, x8, scales, mean, N, D, rows_total, blockIdx);
-    else quant_rows_body<float, false>(x, x8, scales, mean, N, D, rows_total, blockIdx);
+    if (smooth) quant_rows_body<float, true>(x, x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);
+    else quant_rows_body<float, false>(x, x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);
 }
 extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_bf16(const uint16_t *x, int8_t *x8, float *scales,
                                                                            const float *mean, int N, int D, long rows_total,
                                                                            int smooth)
 {
-    if (smooth) quant_rows_body<uint16_t, true>(x, x8, scales, mean, N, D, rows_total, blockIdx);
-    else quant_rows_body<uint16_t, false>(x, x8, scales, mean, N, D, rows_total, blockIdx);
+    if (smooth) quant_rows_body<uint16_t, true>(x, x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);
+    else quant_rows_body<uint16_t, false>(x, x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);
 }
 extern "C" __global__ void __launch_bounds__(256) ar_cast_bf16(const float *x, uint16_t *y, long n)
 {

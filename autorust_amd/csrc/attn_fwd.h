@@ -74,9 +74,10 @@ struct AttnParams {
     int32_t *dbg;            // MODE_I8 debug: [32][64] raw logits
     int dbg_bh, dbg_qt, dbg_kt;
     int Hq, Hkv, N;
-    // element strides of q / k,v / o: [batch, head, token]; the channel stride is 1.
+    // element strides of q / k / o (and v, below): [batch, head, token]; the channel stride is 1.
     // Dense [B,H,N,D] is {H*N*D, N*D, D}; token-major [B,N,H,D] is {N*H*D, D, H*D}.
     long qs[3], ks[3], os[3];
+    long vs[3];    // V's own strides (the int8 path reads a dense K8 next to a V that may be strided)
     int bq, bk;
     int bk_tile_shift;  // log2(bk / 64) when the K scales are tile-uniform
     int nq;        // query tiles per head
@@ -92,7 +93,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     return __builtin_bit_cast(uint32_t, p);
 }
 
-// v_max3_f32 (the generic fmaxf spends an extra instruction per operand on NaN quieting)
+// v_max3_f32 (the generic fmaxf spends an extra instruction per operand on NaN quieting).
+// Never hand it the raw result registers of a matrix instruction: the compiler pads the wait
+// between an MFMA and the first vector read of its result only for instructions it generated,
+// not for inline assembly, and an early read returns a partial sum.  Operands must have passed
+// through an ordinary vector instruction (a scale, a convert) first.
 __device__ __forceinline__ float max3(float a, float b, float c)
 {
     float r;
@@ -218,7 +223,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     const size_t kv_off = (size_t)b * p.ks[0] + (size_t)kvh * p.ks[1];
     const size_t k_rs = (size_t)p.ks[2];  // elements between consecutive tokens of K / V
     const unsigned char *kbase = (const unsigned char *)p.k + kv_off * QK_BYTES;
-    const uint16_t *vbase = p.v + kv_off;
+    const uint16_t *vbase = p.v + (size_t)b * p.vs[0] + (size_t)kvh * p.vs[1];
+    const size_t v_rs = (size_t)p.vs[2];
 
     // ---- Q operand, resident in registers for the whole kernel.  Rows past N
     // read row N-1: their results are never stored. ----
@@ -260,9 +266,9 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
                 const int row = c / V_CPR, col = c % V_CPR;
                 const int gr = k0 + row;
                 if (full) {
-                    vst[slot][j] = *(const uint4 *)(vbase + (size_t)gr * k_rs + col * 8);
+                    vst[slot][j] = *(const uint4 *)(vbase + (size_t)gr * v_rs + col * 8);
                 } else {
-                    uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * k_rs + col * 8);
+                    uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * v_rs + col * 8);
                     if (gr >= kend) val = make_uint4(0, 0, 0, 0);
                     vst[slot][j] = val;
                 }
@@ -412,6 +418,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
                 for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[r], c, -m_run));
                 rs = row_sum();
                 if (__any(!(rs <= 16.0f * LAZY_LIMIT))) {
+                    // (s has been read by the vector instructions above, so max3 may take it as it is)
                     float mx = max3((float)s[0], (float)s[1], (float)s[2]);
 #pragma unroll
                     for (int r = 3; r < 15; r += 2) mx = max3(mx, (float)s[r], (float)s[r + 1]);

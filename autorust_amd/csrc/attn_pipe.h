@@ -125,7 +125,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     // ---- buffer resources over this head's K and V: offsets past kend rows read as zero ----
     const size_t kv_off = (size_t)b * p.ks[0] + (size_t)kvh * p.ks[1];
     const uint32_t k_rowb = (uint32_t)p.ks[2] * QK_BYTES;  // bytes between consecutive keys
-    const uint32_t v_rowb = (uint32_t)p.ks[2] * 2;
+    const uint32_t v_rowb = (uint32_t)p.vs[2] * 2;
     // raw buffer descriptor: base address, stride 0, size in bytes, 32-bit untyped data
     auto make_rsrc = [](const void *base, uint32_t bytes) __attribute__((always_inline)) -> i32x4 {
         const uint64_t a = (uint64_t)(uintptr_t)base;
@@ -137,7 +137,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         return r;
     };
     const i32x4 k_rsrc = make_rsrc((const unsigned char *)p.k + kv_off * QK_BYTES, (uint32_t)kend * k_rowb);
-    const i32x4 v_rsrc = make_rsrc(p.v + kv_off, (uint32_t)kend * v_rowb);
+    const i32x4 v_rsrc = make_rsrc(p.v + (size_t)b * p.vs[0] + (size_t)kvh * p.vs[1], (uint32_t)kend * v_rowb);
 
     // transfer x of a tile (x = wave + 8 j): rows 16 g .. 16 g + 15 of piece pc of K (x < 4 KP) or V;
     // lane l fetches row 16 g + l / 4, chunk (l % 4) ^ ((l / 16) % 4) of that piece
@@ -341,10 +341,16 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
             else
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kt), __builtin_bit_cast(bf16x8, qreg[q]), s, 0, 0, 0);
         }
-        float mx = max3((float)s[0], (float)s[1], (float)s[2]);
+        // max3 is inline assembly, which the compiler leaves out when it pads the distance between a
+        // matrix instruction and the first vector read of its result: the scaled copies below are
+        // ordinary vector instructions, so the result has landed by the time max3 runs
+        float x[16];
 #pragma unroll
-        for (int r = 3; r < 15; r += 2) mx = max3(mx, (float)s[r], (float)s[r + 1]);
-        mx = xhalf_max(fmaxf(mx, (float)s[15])) * c;
+        for (int r = 0; r < 16; ++r) x[r] = (float)s[r] * c;
+        float mx = max3(x[0], x[1], x[2]);
+#pragma unroll
+        for (int r = 3; r < 15; r += 2) mx = max3(mx, x[r], x[r + 1]);
+        mx = xhalf_max(fmaxf(mx, x[15]));
         move_reference(mx);
         exp_pack(s, c, pb, rs);
     };

@@ -9,6 +9,8 @@
 #include "attn_pipe.h"
 #include "flash_f32.h"
 
+#include <algorithm>
+
 
 using namespace arhip;
 
@@ -140,8 +142,9 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
         const int64_t *all[3] = {q_strides, kv_strides, o_strides};
         for (int t = 0; t < 3; ++t)
             for (int i = 0; i < 3; ++i)
-                ARHIP_REQUIRE(all[t][i] >= 0 && all[t][i] % 8 == 0 && (i != 2 || all[t][i] >= D),
-                              "arhip_flash_fwd_strided: stride %lld (multiples of 8 elements, token stride >= D)",
+                ARHIP_REQUIRE(all[t][i] >= 0 && all[t][i] % 8 == 0 && (i != 2 || all[t][i] >= D) && (t != 2 || all[t][i] > 0),
+                              "arhip_flash_fwd_strided: stride %lld (multiples of 8 elements, token stride >= D, output "
+                              "strides > 0 so that output rows cannot alias)",
                               (long long)all[t][i]);
     }
     ARHIP_HIP(hipSetDevice(dev->ordinal));
@@ -186,6 +189,7 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
     for (int i = 0; i < 3; ++i) {
         p.qs[i] = (long)q_strides[i];
         p.ks[i] = (long)kv_strides[i];
+        p.vs[i] = (long)kv_strides[i];
         p.os[i] = (long)o_strides[i];
     }
     p.bq = p.bk = 1;
@@ -229,12 +233,33 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
                               int32_t *dbg_logits, const int32_t dbg_sel[3],
                               int wait, double *secs)
 {
+    return arhip_sage_fwd_strided(dev, q8, k8, sq, sk, v, o, nullptr, nullptr, mask, kv_len, B, Hq, Hkv, N, D, bq, bk, causal,
+                                  out_dtype, scale, dbg_logits, dbg_sel, wait, secs);
+}
+
+extern "C" int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const int8_t *k8,
+                                      const float *sq, const float *sk, const uint16_t *v, void *o,
+                                      const int64_t v_strides[3], const int64_t o_strides[3],
+                                      const float *mask, const int32_t *kv_len,
+                                      int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                                      int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
+                                      int32_t *dbg_logits, const int32_t dbg_sel[3],
+                                      int wait, double *secs)
+{
     if (int rc = check_common("arhip_sage_fwd", dev, q8, k8, v, o, mask, B, Hq, Hkv, N, D)) return rc;
     ARHIP_REQUIRE(sq && sk, "arhip_sage_fwd: null scale pointer");
     ARHIP_REQUIRE(bq >= 1 && bk >= 1, "arhip_sage_fwd: block sizes bq=%lld bk=%lld", (long long)bq, (long long)bk);
     ARHIP_REQUIRE(out_dtype == ARHIP_F32 || out_dtype == ARHIP_BF16, "arhip_sage_fwd: out_dtype %d", out_dtype);
     ARHIP_REQUIRE(dbg_logits == nullptr || dbg_sel != nullptr, "arhip_sage_fwd: dbg_logits without dbg_sel");
     ARHIP_REQUIRE(dbg_logits == nullptr || mask == nullptr, "arhip_sage_fwd: the logits export does not take a mask");
+    for (int t = 0; t < 2; ++t) {
+        const int64_t *st = t == 0 ? v_strides : o_strides;
+        if (!st) continue;
+        for (int i = 0; i < 3; ++i)
+            ARHIP_REQUIRE(st[i] >= 0 && st[i] % 8 == 0 && (i != 2 || st[i] >= D) && (t == 0 || st[i] > 0),
+                          "arhip_sage_fwd_strided: stride %lld (multiples of 8 elements, token stride >= D, output strides > 0)",
+                          (long long)st[i]);
+    }
     ARHIP_HIP(hipSetDevice(dev->ordinal));
 
     AttnParams p = {};
@@ -244,7 +269,12 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
     dense_strides(p.qs, Hq, N, D);
     dense_strides(p.ks, Hkv, N, D);
+    dense_strides(p.vs, Hkv, N, D);
     dense_strides(p.os, Hq, N, D);
+    for (int i = 0; i < 3; ++i) {
+        if (v_strides) p.vs[i] = (long)v_strides[i];
+        if (o_strides) p.os[i] = (long)o_strides[i];
+    }
     p.bq = (int)bq; p.bk = (int)bk;
     p.scale = scale;
     const bool dbg = dbg_logits != nullptr;
@@ -257,7 +287,7 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
     p.bk_tile_shift = shift;
     int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg);
     if (nw == 1) nw = 4;
-    if (nw == 8 && !pipe_addressable(N, D, 2)) nw = 4;
+    if (nw == 8 && !pipe_addressable(N, std::max<int64_t>(D, v_strides ? v_strides[2] : D), 2)) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;

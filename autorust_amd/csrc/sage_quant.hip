@@ -39,7 +39,7 @@ int arhip_static_scratch_setup(int ordinal)
     return ARHIP_OK;
 }
 
-static int sage_quant_impl(arhip_device *dev, const void *x, int8_t *x8, float *scales, float *mean,
+static int sage_quant_impl(arhip_device *dev, const void *x, const int64_t x_strides[3], int8_t *x8, float *scales, float *mean,
                            void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
                            int64_t block, int dtype, int smooth, int wait, double *secs, int prof_kernel)
 {
@@ -52,6 +52,15 @@ static int sage_quant_impl(arhip_device *dev, const void *x, int8_t *x8, float *
     ARHIP_REQUIRE(arhip_aligned16(x) && (reinterpret_cast<uintptr_t>(x8) & 7u) == 0,
                   "arhip_sage_quant: x must be 16-byte and x8 8-byte aligned");
     ARHIP_REQUIRE(!smooth || (mean && workspace), "arhip_sage_quant: smoothing needs mean and workspace buffers");
+    XLayout lay = XLayout::dense((int)H, (int)N, (int)D);
+    if (x_strides) {
+        // rows stay 16-byte aligned and do not overlap: multiples of 8 elements, token stride >= D
+        for (int i = 0; i < 3; ++i)
+            ARHIP_REQUIRE(x_strides[i] >= 0 && x_strides[i] % 8 == 0 && (i != 2 || x_strides[i] >= D),
+                          "arhip_sage_quant_strided: stride %lld (multiples of 8 elements, token stride >= D)",
+                          (long long)x_strides[i]);
+        lay = XLayout{(long)x_strides[0], (long)x_strides[1], (long)x_strides[2], (int)H};
+    }
     ARHIP_HIP(hipSetDevice(dev->ordinal));
     const int nblk = (int)((N + block - 1) / block);
     const int nchunk = (int)((N + MEAN_CHUNK - 1) / MEAN_CHUNK);
@@ -64,10 +73,10 @@ static int sage_quant_impl(arhip_device *dev, const void *x, int8_t *x8, float *
         const dim3 pgrid((unsigned)((nchunk + cpb - 1) / cpb), (unsigned)(B * H));
         if (dtype == ARHIP_F32)
             hipLaunchKernelGGL(k_mean_partial_kernel<float>, pgrid, dim3(256), 0, dev->stream,
-                               (const float *)x, (float *)workspace, (int)N, (int)D, nchunk);
+                               (const float *)x, (float *)workspace, (int)N, (int)D, nchunk, lay);
         else
             hipLaunchKernelGGL(k_mean_partial_kernel<uint16_t>, pgrid, dim3(256), 0, dev->stream,
-                               (const uint16_t *)x, (float *)workspace, (int)N, (int)D, nchunk);
+                               (const uint16_t *)x, (float *)workspace, (int)N, (int)D, nchunk, lay);
         hipLaunchKernelGGL(k_mean_final_kernel, dim3((unsigned)(B * H)), dim3((unsigned)D), 0, dev->stream,
                            (const float *)workspace, mean, (int)N, (int)D, nchunk);
     }
@@ -78,32 +87,32 @@ static int sage_quant_impl(arhip_device *dev, const void *x, int8_t *x8, float *
         if (smooth) {
             if (dtype == ARHIP_F32)
                 hipLaunchKernelGGL((quant_rows_kernel<float, true>), rgrid, dim3(256), 0, dev->stream,
-                                   (const float *)x, x8, scales, mean, (int)N, (int)D, rows);
+                                   (const float *)x, x8, scales, mean, (int)N, (int)D, rows, lay);
             else
                 hipLaunchKernelGGL((quant_rows_kernel<uint16_t, true>), rgrid, dim3(256), 0, dev->stream,
-                                   (const uint16_t *)x, x8, scales, mean, (int)N, (int)D, rows);
+                                   (const uint16_t *)x, x8, scales, mean, (int)N, (int)D, rows, lay);
         } else {
             if (dtype == ARHIP_F32)
                 hipLaunchKernelGGL((quant_rows_kernel<float, false>), rgrid, dim3(256), 0, dev->stream,
-                                   (const float *)x, x8, scales, nullptr, (int)N, (int)D, rows);
+                                   (const float *)x, x8, scales, nullptr, (int)N, (int)D, rows, lay);
             else
                 hipLaunchKernelGGL((quant_rows_kernel<uint16_t, false>), rgrid, dim3(256), 0, dev->stream,
-                                   (const uint16_t *)x, x8, scales, nullptr, (int)N, (int)D, rows);
+                                   (const uint16_t *)x, x8, scales, nullptr, (int)N, (int)D, rows, lay);
         }
     } else if (smooth) {
         if (dtype == ARHIP_F32)
             hipLaunchKernelGGL((quant_blocks_kernel<float, true>), qgrid, dim3(256), 0, dev->stream,
-                               (const float *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk);
+                               (const float *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk, lay);
         else
             hipLaunchKernelGGL((quant_blocks_kernel<uint16_t, true>), qgrid, dim3(256), 0, dev->stream,
-                               (const uint16_t *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk);
+                               (const uint16_t *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk, lay);
     } else {
         if (dtype == ARHIP_F32)
             hipLaunchKernelGGL((quant_blocks_kernel<float, false>), qgrid, dim3(256), 0, dev->stream,
-                               (const float *)x, x8, scales, nullptr, (int)N, (int)D, (int)block, nblk);
+                               (const float *)x, x8, scales, nullptr, (int)N, (int)D, (int)block, nblk, lay);
         else
             hipLaunchKernelGGL((quant_blocks_kernel<uint16_t, false>), qgrid, dim3(256), 0, dev->stream,
-                               (const uint16_t *)x, x8, scales, nullptr, (int)N, (int)D, (int)block, nblk);
+                               (const uint16_t *)x, x8, scales, nullptr, (int)N, (int)D, (int)block, nblk, lay);
     }
     arhip_note_selected(ARHIP_K_SAGE_QUANT);
     return t.end();
@@ -113,7 +122,16 @@ extern "C" int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, fl
                                 void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
                                 int64_t block, int dtype, int smooth, int wait, double *secs)
 {
-    return sage_quant_impl(dev, x, x8, scales, mean, workspace, B, H, N, D, block, dtype, smooth, wait, secs,
+    return sage_quant_impl(dev, x, nullptr, x8, scales, mean, workspace, B, H, N, D, block, dtype, smooth, wait, secs,
+                           ARHIP_K_SAGE_QUANT);
+}
+
+extern "C" int arhip_sage_quant_strided(arhip_device *dev, const void *x, const int64_t x_strides[3], int8_t *x8,
+                                        float *scales, float *mean, void *workspace, int64_t B, int64_t H, int64_t N,
+                                        int64_t D, int64_t block, int dtype, int smooth, int wait, double *secs)
+{
+    ARHIP_REQUIRE(x_strides != nullptr, "arhip_sage_quant_strided: null strides");
+    return sage_quant_impl(dev, x, x_strides, x8, scales, mean, workspace, B, H, N, D, block, dtype, smooth, wait, secs,
                            ARHIP_K_SAGE_QUANT);
 }
 
@@ -141,7 +159,7 @@ extern "C" int arhip_sage_quant_static(arhip_device *dev, const void *x, int8_t 
                       "arhip_sage_quant_static: the scratch address of device %d was not resolved at open", dev->ordinal);
         ws = g_scratch_ptr[dev->ordinal];
     }
-    return sage_quant_impl(dev, x, x8, scales, mean, ws, B, H, N, D, block, dtype, smooth, wait, secs, -1);
+    return sage_quant_impl(dev, x, nullptr, x8, scales, mean, ws, B, H, N, D, block, dtype, smooth, wait, secs, -1);
 }
 
 extern "C" int arhip_cast_bf16(arhip_device *dev, const float *x, uint16_t *y, int64_t n, int wait, double *secs)

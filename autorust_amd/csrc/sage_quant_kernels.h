@@ -21,6 +21,16 @@ namespace arhip {
 
 constexpr int MEAN_CHUNK = 64;  // tokens per partial sum
 
+// Where the input tensor's rows are: element strides of batch / head / token (the channel stride
+// is 1).  Dense [B, H, N, D] is {H*N*D, N*D, D}; the token-major layout a projection produces,
+// [B, N, H, D], is {N*H*D, D, H*D}.  Outputs of the pre-pass are always dense.
+struct XLayout {
+    long sb, sh, st;
+    int H;
+    __host__ __device__ static XLayout dense(int H, int N, int D) { return {(long)H * N * D, (long)N * D, (long)D, H}; }
+    __device__ __forceinline__ size_t head(int bh) const { return (size_t)(bh / H) * sb + (size_t)(bh % H) * sh; }
+};
+
 
 __device__ __forceinline__ void ld8(const float *x, size_t e, float v[8])
 {
@@ -40,7 +50,7 @@ __device__ __forceinline__ void ld8(const uint16_t *x, size_t e, float v[8])
 // One thread owns 8 adjacent channels of one 64-token chunk: D/8 threads read a whole row
 // (coalesced), 256/(D/8) chunks per workgroup.
 template <typename T>
-__device__ __forceinline__ void k_mean_partial_body(const T *x, float *part, int N, int D, int nchunk, const dim3 bid)
+__device__ __forceinline__ void k_mean_partial_body(const T *x, float *part, int N, int D, int nchunk, const XLayout lay, const dim3 bid)
 {
     const int gpr = D / 8;                       // 8-channel groups per row
     const int cpb = 256 / gpr;                   // chunks per workgroup
@@ -49,11 +59,11 @@ __device__ __forceinline__ void k_mean_partial_body(const T *x, float *part, int
     if (c >= nchunk) return;
     const int j0 = c * MEAN_CHUNK;
     const int j1 = min(N, j0 + MEAN_CHUNK);
-    const size_t base = (size_t)bh * N * D + g * 8;
+    const size_t base = lay.head(bh) + g * 8;
     float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int j = j0; j < j1; ++j) {
         float v[8];
-        ld8(x, base + (size_t)j * D, v);
+        ld8(x, base + (size_t)j * lay.st, v);
 #pragma unroll
         for (int i = 0; i < 8; ++i) s[i] += v[i];
     }
@@ -63,9 +73,9 @@ __device__ __forceinline__ void k_mean_partial_body(const T *x, float *part, int
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256) k_mean_partial_kernel(const T *x, float *part, int N, int D, int nchunk)
+__global__ void __launch_bounds__(256) k_mean_partial_kernel(const T *x, float *part, int N, int D, int nchunk, const XLayout lay)
 {
-    k_mean_partial_body<T>(x, part, N, D, nchunk, blockIdx);
+    k_mean_partial_body<T>(x, part, N, D, nchunk, lay, blockIdx);
 }
 
 // mean[bh][d] = (part[0] + part[1] + ...) / N in chunk order (loads batched, adds in order)
@@ -96,14 +106,17 @@ __global__ void k_mean_final_kernel(const float *part, float *mean, int N, int D
 // ones are read twice.
 template <typename T, bool SMOOTH>
 __device__ __forceinline__ void quant_blocks_body(const T *x, int8_t *x8, float *scales, const float *mean,
-                                                           int N, int D, int blk, int nblk, const dim3 bid)
+                                                  int N, int D, int blk, int nblk, const XLayout lay, const dim3 bid)
 {
     constexpr int KEEP = 8;  // 8-element groups a thread can hold
     __shared__ float red[4];  // one instance per kernel that inlines this body
     const int bi = bid.x, bh = bid.y, tid = threadIdx.x;
     const int r0 = bi * blk;
     const int r1 = min(N, r0 + blk);
-    const size_t base = ((size_t)bh * N + r0) * D;
+    const size_t base = ((size_t)bh * N + r0) * D;  // of the dense output
+    const size_t xbase = lay.head(bh) + (size_t)r0 * lay.st;
+    // element e of the block (row e / D, channel e % D) in the input
+    auto xin = [&](int e) __attribute__((always_inline)) { return xbase + (size_t)(e / D) * lay.st + (e % D); };
     const int nelem = (r1 - r0) * D;  // multiple of 8
     const float *mu = SMOOTH ? mean + (size_t)bh * D : nullptr;
     const bool keep = nelem <= 256 * 8 * KEEP;
@@ -115,7 +128,7 @@ __device__ __forceinline__ void quant_blocks_body(const T *x, int8_t *x8, float 
         for (int it = 0; it < KEEP; ++it) {
             const int e = (it * 256 + tid) * 8;
             if (e < nelem) {
-                ld8(x, base + e, held[it]);
+                ld8(x, xin(e), held[it]);
                 const int d = e % D;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
@@ -127,7 +140,7 @@ __device__ __forceinline__ void quant_blocks_body(const T *x, int8_t *x8, float 
     } else {
         for (int e = tid * 8; e < nelem; e += 256 * 8) {
             float v[8];
-            ld8(x, base + e, v);
+            ld8(x, xin(e), v);
             const int d = e % D;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -166,7 +179,7 @@ __device__ __forceinline__ void quant_blocks_body(const T *x, int8_t *x8, float 
     } else {
         for (int e = tid * 8; e < nelem; e += 256 * 8) {
             float v[8];
-            ld8(x, base + e, v);
+            ld8(x, xin(e), v);
             const int d = e % D;
             if (SMOOTH) {
 #pragma unroll
@@ -179,9 +192,9 @@ __device__ __forceinline__ void quant_blocks_body(const T *x, int8_t *x8, float 
 
 template <typename T, bool SMOOTH>
 __global__ void __launch_bounds__(256) quant_blocks_kernel(const T *x, int8_t *x8, float *scales, const float *mean,
-                                                           int N, int D, int blk, int nblk)
+                                                           int N, int D, int blk, int nblk, const XLayout lay)
 {
-    quant_blocks_body<T, SMOOTH>(x, x8, scales, mean, N, D, blk, nblk, blockIdx);
+    quant_blocks_body<T, SMOOTH>(x, x8, scales, mean, N, D, blk, nblk, lay, blockIdx);
 }
 
 // The reference's own granularity, one scale per token row (block == 1): D/8 lanes share a row,
@@ -189,7 +202,7 @@ __global__ void __launch_bounds__(256) quant_blocks_kernel(const T *x, int8_t *x
 // inside the lane group.  Same arithmetic, same order of operations per element.
 template <typename T, bool SMOOTH>
 __device__ __forceinline__ void quant_rows_body(const T *x, int8_t *x8, float *scales, const float *mean,
-                                                         int N, int D, long rows_total, const dim3 bid)
+                                                int N, int D, long rows_total, const XLayout lay, const dim3 bid)
 {
     const int gpr = D / 8;                                   // lanes per row (8 or 16)
     const long row = (long)bid.x * (256 / gpr) + threadIdx.x / gpr;   // global row over [B*H*N]
@@ -197,7 +210,7 @@ __device__ __forceinline__ void quant_rows_body(const T *x, int8_t *x8, float *s
     const bool live = row < rows_total;
     float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (live) {
-        ld8(x, (size_t)row * D + g * 8, v);
+        ld8(x, lay.head((int)(row / N)) + (size_t)(row % N) * lay.st + g * 8, v);
         if (SMOOTH) {
             const float *mu = mean + (size_t)(row / N) * D + g * 8;
 #pragma unroll
@@ -225,9 +238,9 @@ __device__ __forceinline__ void quant_rows_body(const T *x, int8_t *x8, float *s
 
 template <typename T, bool SMOOTH>
 __global__ void __launch_bounds__(256) quant_rows_kernel(const T *x, int8_t *x8, float *scales, const float *mean,
-                                                         int N, int D, long rows_total)
+                                                         int N, int D, long rows_total, const XLayout lay)
 {
-    quant_rows_body<T, SMOOTH>(x, x8, scales, mean, N, D, rows_total, blockIdx);
+    quant_rows_body<T, SMOOTH>(x, x8, scales, mean, N, D, rows_total, lay, blockIdx);
 }
 
 __device__ __forceinline__ void cast_bf16_body(const float *x, uint16_t *y, size_t n, const dim3 bid)

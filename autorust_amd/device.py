@@ -184,11 +184,19 @@ class Device:
     def sage_quant_workspace(self, B, H, N, D):
         return self.lib.arhip_sage_quant_workspace(B, H, N, D)
 
-    def sage_quant(self, x, x8, scales, B, H, N, D, block, dtype, mean=None, workspace=None, smooth=False, wait=True):
+    def sage_quant(self, x, x8, scales, B, H, N, D, block, dtype, mean=None, workspace=None, smooth=False, wait=True,
+                   x_strides=None):
+        """x_strides: element strides {batch, head, token} of x (None = dense [B,H,N,D])."""
         s = ctypes.c_double()
-        check(self.lib.arhip_sage_quant(self.handle, self._ptr(x), self._ptr(x8), self._ptr(scales), self._ptr(mean),
-                                        self._ptr(workspace), B, H, N, D, block, dtype, int(smooth), int(wait),
-                                        ctypes.byref(s)))
+        if x_strides is None:
+            check(self.lib.arhip_sage_quant(self.handle, self._ptr(x), self._ptr(x8), self._ptr(scales), self._ptr(mean),
+                                            self._ptr(workspace), B, H, N, D, block, dtype, int(smooth), int(wait),
+                                            ctypes.byref(s)))
+        else:
+            xs = (ctypes.c_int64 * 3)(*[int(t) for t in x_strides])
+            check(self.lib.arhip_sage_quant_strided(self.handle, self._ptr(x), xs, self._ptr(x8), self._ptr(scales),
+                                                    self._ptr(mean), self._ptr(workspace), B, H, N, D, block, dtype,
+                                                    int(smooth), int(wait), ctypes.byref(s)))
         return s.value if wait else None
 
     def sage_quant_static(self, x, x8, scales, B, H, N, D, block, dtype, mean=None, smooth=False, wait=True):
@@ -205,16 +213,18 @@ class Device:
         return s.value if wait else None
 
     def sage_fwd(self, q8, k8, sq, sk, v, o, B, Hq, Hkv, N, D, bq, bk, out_dtype=F32, mask=None, kv_len=None,
-                 causal=False, scale=None, dbg_logits=None, dbg_sel=None, wait=True):
+                 causal=False, scale=None, dbg_logits=None, dbg_sel=None, wait=True, v_strides=None, o_strides=None):
         scale = float(1.0 / np.sqrt(np.float32(D))) if scale is None else float(scale)
         sel = None
         if dbg_sel is not None:
             sel = (ctypes.c_int32 * 3)(*dbg_sel)
         s = ctypes.c_double()
-        check(self.lib.arhip_sage_fwd(self.handle, self._ptr(q8), self._ptr(k8), self._ptr(sq), self._ptr(sk),
-                                      self._ptr(v), self._ptr(o), self._ptr(mask), self._ptr(kv_len),
-                                      B, Hq, Hkv, N, D, bq, bk, int(causal), out_dtype, scale,
-                                      self._ptr(dbg_logits), sel, int(wait), ctypes.byref(s)))
+        arr = lambda t: None if t is None else (ctypes.c_int64 * 3)(*[int(x) for x in t])
+        check(self.lib.arhip_sage_fwd_strided(self.handle, self._ptr(q8), self._ptr(k8), self._ptr(sq), self._ptr(sk),
+                                              self._ptr(v), self._ptr(o), arr(v_strides), arr(o_strides),
+                                              self._ptr(mask), self._ptr(kv_len),
+                                              B, Hq, Hkv, N, D, bq, bk, int(causal), out_dtype, scale,
+                                              self._ptr(dbg_logits), sel, int(wait), ctypes.byref(s)))
         return s.value if wait else None
 
 

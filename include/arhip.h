@@ -179,6 +179,14 @@ int arhip_sage_quant(arhip_device *dev, const void *x, int8_t *x8, float *scales
                      void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
                      int64_t block, int dtype, int smooth, int wait, double *secs);
 
+/* arhip_sage_quant_strided: arhip_sage_quant on a strided input (element strides {batch, head,
+ *   token}, channel stride 1; every stride a multiple of 8, token stride >= D): the projection
+ *   output [B,N,H,D] is quantised in place of the copy to [B,H,N,D] the reference makes
+ *   (src/models/transformer.rs:286-299).  x8, scales and mean are dense as for arhip_sage_quant. */
+int arhip_sage_quant_strided(arhip_device *dev, const void *x, const int64_t x_strides[3], int8_t *x8,
+                             float *scales, float *mean, void *workspace, int64_t B, int64_t H, int64_t N,
+                             int64_t D, int64_t block, int dtype, int smooth, int wait, double *secs);
+
 /* arhip_sage_quant_static: arhip_sage_quant without a workspace argument and without any
  *   allocation inside the call.  It has no counterpart in the reference; it is for callers that
  *   cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
@@ -213,6 +221,18 @@ int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t *k8,
                    int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
                    int32_t *dbg_logits, const int32_t dbg_sel[3],
                    int wait, double *secs);
+
+/* arhip_sage_fwd_strided: arhip_sage_fwd with element strides {batch, head, token} for v and o
+ *   (NULL = dense): v as the projection produced it ([B,N,Hkv,D]), o written as [B,N,Hq*D].
+ *   q8, k8 and the scales are this library's own pre-pass outputs and stay dense. */
+int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const int8_t *k8,
+                           const float *sq, const float *sk, const uint16_t *v, void *o,
+                           const int64_t v_strides[3], const int64_t o_strides[3],
+                           const float *mask, const int32_t *kv_len,
+                           int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                           int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
+                           int32_t *dbg_logits, const int32_t dbg_sel[3],
+                           int wait, double *secs);
 
 /* dispatch counters: `selections()` (src/runtime/cuda_flash_bf16.rs:443-461,
  *   cuda_flash_sage.rs:417-436) */

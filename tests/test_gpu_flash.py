@@ -12,7 +12,7 @@ import pytest
 import oracle
 from autorust_amd import _lib, synth
 from autorust_amd.device import BF16, F32, selections
-from gpu_util import fill_qkv, ref_mask, run_flash
+from gpu_util import bf16_ulps, fill_qkv, ref_mask, run_flash
 
 pytestmark = pytest.mark.gpu
 
@@ -125,6 +125,21 @@ def test_bf16_is_deterministic(dev):
     assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("kind", ["bf16", "int8"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_long_sequence_kernels_are_deterministic(dev, kind, causal):
+    """Same assertion at a shape the software-pipelined kernels take (two waves per SIMD, so a
+    result read one instruction too early shows up as a run-to-run difference)."""
+    shape = (1, 32, 4096, 128)
+    q, k, v = synth.normal(931, shape), synth.normal(932, shape), synth.normal(933, shape)
+    if kind == "bf16":
+        runs = [run_flash(dev, q, k, v, BF16, causal=causal) for _ in range(3)]
+    else:
+        from gpu_util import run_sage
+        runs = [run_sage(dev, q, k, v, 128, 64, out_dtype=BF16, causal=causal)["out"] for _ in range(3)]
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+
+
 @pytest.mark.parametrize("dtype", [BF16, F32])
 @pytest.mark.parametrize("D,N", [(64, 197), (128, 300), (128, 1100)])
 def test_token_major_layout_is_the_same_function(dev, dtype, D, N):
@@ -145,6 +160,11 @@ def test_token_major_layout_is_the_same_function(dev, dtype, D, N):
         raw = to.copyout(np.uint16 if dtype == BF16 else np.float32, (B, N, Hq, D))
     got = (synth.from_bf16_bits(raw) if dtype == BF16 else raw).transpose(0, 2, 1, 3)
     assert np.array_equal(got, dense)
+    # and it is the right function, not merely the same one: against the oracle on the same inputs
+    if dtype == BF16:
+        assert bf16_ulps(got, oracle.attn_bf16(q, k, v, causal=True)) <= 3
+    else:
+        assert np.abs(got - oracle.flash_f32(q, k, v, causal=True)).max() < 2e-5
     # strides that would misalign rows are rejected
     with pytest.raises(_lib.ArhipError):
         d = dev.alloc(64)
@@ -179,3 +199,28 @@ def test_log_sum_exp_output(dev, dtype, tol, D, N):
     want = oracle.lse_f64(qq, kk, kv_len=kv_len, causal=True)
     err = float(np.abs(lse - want).max())
     assert err <= tol
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_token_major_layout_long_sequences(dev, causal):
+    """The same through the software-pipelined kernel (enough workgroups of 256 queries to be
+    chosen): [B, N, H, D] in, [B, N, H*D] out, with per-batch key lengths, against the oracle on
+    sampled rows and bit for bit against the dense call."""
+    from gpu_util import Bufs
+    B, Hq, Hkv, N, D = 2, 16, 8, 4096 + 40, 128
+    q, k, v = synth.normal(931, (B, Hq, N, D)), synth.normal(932, (B, Hkv, N, D)), synth.normal(933, (B, Hkv, N, D))
+    kv_len = np.array([N, N - 1000], np.int32)
+    dense = run_flash(dev, q, k, v, BF16, kv_len=kv_len, causal=causal)
+    with Bufs(dev) as bufs:
+        tq, tk, tv = (bufs.put(synth.to_bf16_bits(np.ascontiguousarray(t.transpose(0, 2, 1, 3)))) for t in (q, k, v))
+        to = bufs.new(q.size * 2)
+        dl = bufs.put(kv_len)
+        dev.flash_fwd_strided(tq, tk, tv, to, (N * Hq * D, D, Hq * D), (N * Hkv * D, D, Hkv * D), (N * Hq * D, D, Hq * D),
+                              B, Hq, Hkv, N, D, BF16, kv_len=dl, causal=causal)
+        got = synth.from_bf16_bits(to.copyout(np.uint16, (B, N, Hq, D))).transpose(0, 2, 1, 3)
+    assert np.array_equal(got, dense)
+    rows = np.array([0, 1, 63, 64, 255, 256, 257, 2047, 3095, 3096, 4095, 4096, N - 1], np.int32)
+    want = oracle.attn_bf16(q, k, v, kv_len=kv_len, causal=causal, rows=rows)
+    assert bf16_ulps(got[:, :, rows], want) <= 3
+    truth = oracle.sdpa_f64(q, k, v, kv_len=kv_len, causal=causal, rows=rows)
+    assert np.abs(got[:, :, rows] - truth).max() <= 2e-2

@@ -133,3 +133,51 @@ def test_per_row_scales_with_smoothing(dev, D):
     want = oracle.sage(q8, k8, sq, sk, v, 1, 1)
     err = float(np.abs(r["out"] - want).max())
     assert err < 4e-3
+
+
+@pytest.mark.parametrize("N,Hq,Hkv", [(300, 4, 2), (4096 + 24, 16, 16)])
+def test_token_major_layout(dev, N, Hq, Hkv):
+    """Strided Sage entry points: Q, K, V as the projections produce them, [B, N, H, D], quantised
+    without the copy to [B, H, N, D], and the output written as [B, N, H*D]
+    (src/models/transformer.rs:286-299).  Quantised tensors, scales and mean bit-exact against the
+    oracle; output identical to the dense calls and within the emulation's bound."""
+    from gpu_util import Bufs, bf16_ulps
+    B, D, bq, bk = 2, 128, 128, 64
+    q = synth.normal(941, (B, Hq, N, D))
+    k = synth.normal(942, (B, Hkv, N, D)) + np.float32(3.0) * synth.normal(944, (1, Hkv, 1, D))
+    v = synth.normal(943, (B, Hkv, N, D))
+    nqb, nkb = (N + bq - 1) // bq, (N + bk - 1) // bk
+    tm = lambda t: synth.to_bf16_bits(np.ascontiguousarray(t.transpose(0, 2, 1, 3)))
+    outs = []
+    with Bufs(dev) as bufs:
+        for strided in (False, True):
+            if strided:
+                dq, dk, dv = bufs.put(tm(q)), bufs.put(tm(k)), bufs.put(tm(v))
+                qs, ks = (N * Hq * D, D, Hq * D), (N * Hkv * D, D, Hkv * D)
+            else:
+                dq, dk, dv = (bufs.put(synth.to_bf16_bits(t)) for t in (q, k, v))
+                qs = ks = None
+            q8, k8 = bufs.new(q.size), bufs.new(k.size)
+            sq, sk, mean = bufs.new(B * Hq * nqb * 4), bufs.new(B * Hkv * nkb * 4), bufs.new(B * Hkv * D * 4)
+            ws = bufs.new(dev.sage_quant_workspace(B, Hkv, N, D), zero=False)
+            dev.sage_quant(dq, q8, sq, B, Hq, N, D, bq, BF16, x_strides=qs)
+            dev.sage_quant(dk, k8, sk, B, Hkv, N, D, bk, BF16, mean=mean, workspace=ws, smooth=True, x_strides=ks)
+            do = bufs.new(q.size * 2)
+            dev.sage_fwd(q8, k8, sq, sk, dv, do, B, Hq, Hkv, N, D, bq, bk, out_dtype=BF16, causal=True,
+                         v_strides=ks, o_strides=qs)
+            o = synth.from_bf16_bits(do.copyout(np.uint16, (B, N, Hq, D) if strided else q.shape))
+            outs.append((q8.copyout(np.int8, q.shape), k8.copyout(np.int8, k.shape), sq.copyout(np.float32, (B, Hq, nqb)),
+                         sk.copyout(np.float32, (B, Hkv, nkb)), mean.copyout(np.float32, (B, Hkv, D)),
+                         o.transpose(0, 2, 1, 3) if strided else o))
+    qb, kb = oracle.bf16_round(q), oracle.bf16_round(k)
+    mu = oracle.k_mean(kb)
+    w_q8, w_sq = oracle.quant_blocks(qb, bq)
+    w_k8, w_sk = oracle.quant_blocks(kb, bk, sub=mu)
+    for g_q8, g_k8, g_sq, g_sk, g_mean, _ in outs:
+        assert np.array_equal(g_mean, mu)
+        assert np.array_equal(g_q8, w_q8) and np.array_equal(g_sq, w_sq)
+        assert np.array_equal(g_k8, w_k8) and np.array_equal(g_sk, w_sk)
+    assert np.array_equal(outs[0][5], outs[1][5])
+    rows = np.array(sorted({0, 1, 127, 128, 255, 256, N // 2, N - 2, N - 1}), np.int32)
+    want = oracle.sage(w_q8, w_k8, w_sq, w_sk, v, bq, bk, causal=True, rows=rows, round_out=True)
+    assert bf16_ulps(outs[1][5][:, :, rows], want) <= 3
