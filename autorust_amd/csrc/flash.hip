@@ -86,10 +86,14 @@ static bool pipe_addressable(int64_t N, int64_t kv_token_stride, int64_t elem_by
 static int pick_waves(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bool special)
 {
     // masks, per-key scales and the debug export are built for 4 waves (and 1 at D = 64) only
+    // The 8-wave kernel is the software-pipelined one: it hides the memory latency of a tile
+    // behind the tiles before, which from ~8 tiles per workgroup on outweighs leaving compute units
+    // without a workgroup (B8 H6 N789 D64: 23 us against 56 us with 1200 one-wave workgroups).
+    const int64_t cus = dev->cus, wg256 = heads * ((N + 255) / 256), wg128 = heads * ((N + 127) / 128);
     int nw;
-    if (D == 64 && heads * ((N + 127) / 128) < 2 * (int64_t)dev->cus) nw = 1;
-    else if (special) nw = 4;
-    else nw = (heads * ((N + 255) / 256) >= 2 * (int64_t)dev->cus) ? 8 : 4;
+    if (!special && (wg256 >= 2 * cus || (N >= 512 && 2 * wg256 >= cus))) nw = 8;
+    else if (D == 64 && wg128 < 2 * cus && (special || N < 512)) nw = 1;
+    else nw = 4;
     // ARHIP_ATTN_WAVES (read once when the device is opened) is a tuning aid; results do not depend on it
     const int w = dev->attn_waves;
     if ((w == 1 || w == 4 || w == 8) && !special && (w != 1 || D == 64)) nw = w;
@@ -161,21 +165,23 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
             fp.ks[i] = (long)kv_strides[i];
             fp.os[i] = (long)o_strides[i];
         }
-        // 4 waves (128 queries) per workgroup when that still fills the chip, else 1 wave
-        const int nw = (B * Hq * ((N + 127) / 128) >= 2 * (int64_t)dev->cus) ? 4 : 1;
-        fp.nq = (int)((N + nw * 32 - 1) / (nw * 32));
+        // 4 waves per workgroup: 128 queries when that still fills the chip, else the same 32
+        // queries with the key tiles dealt out between the waves
+        const bool splitk = B * Hq * ((N + 127) / 128) < 2 * (int64_t)dev->cus;
+        const int bq = splitk ? 32 : 128;
+        fp.nq = (int)((N + bq - 1) / bq);
         fp.scale = scale;
         if (int rc = t.begin()) return rc;
-        const dim3 grid((unsigned)(fp.nq * B * Hq)), block((unsigned)(nw * 64));
-#define F32_LAUNCH(DD, NWW)                                                                           \
+        const dim3 grid((unsigned)(fp.nq * B * Hq)), block(256);
+#define F32_LAUNCH(DD, SK)                                                                            \
     do {                                                                                              \
-        if (causal) hipLaunchKernelGGL((flash_f32_kernel<DD, NWW, true>), grid, block, 0, dev->stream, fp);  \
-        else hipLaunchKernelGGL((flash_f32_kernel<DD, NWW, false>), grid, block, 0, dev->stream, fp); \
+        if (causal) hipLaunchKernelGGL((flash_f32_kernel<DD, 4, true, SK>), grid, block, 0, dev->stream, fp);  \
+        else hipLaunchKernelGGL((flash_f32_kernel<DD, 4, false, SK>), grid, block, 0, dev->stream, fp); \
     } while (0)
         if (D == 64) {
-            if (nw == 4) F32_LAUNCH(64, 4); else F32_LAUNCH(64, 1);
+            if (splitk) F32_LAUNCH(64, true); else F32_LAUNCH(64, false);
         } else {
-            if (nw == 4) F32_LAUNCH(128, 4); else F32_LAUNCH(128, 1);
+            if (splitk) F32_LAUNCH(128, true); else F32_LAUNCH(128, false);
         }
 #undef F32_LAUNCH
         arhip_note_selected(ARHIP_K_FLASH_F32);

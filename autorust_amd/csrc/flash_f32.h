@@ -36,20 +36,26 @@ struct FlashF32Params {
     float scale;
 };
 
-// LDS floats flash_f32_body needs: one padded K tile and one V tile
-template <int D>
+// LDS floats flash_f32_body needs: one padded K tile and one V tile (one pair per wave with SPLITK)
+template <int D, int NW = 1, bool SPLITK = false>
 constexpr int flash_f32_lds_floats()
 {
-    return F32_BK * (D + 4) + F32_BK * D;
+    return (SPLITK ? NW : 1) * (F32_BK * (D + 4) + F32_BK * D);
 }
 
-// The kernel body.  lds: flash_f32_lds_floats<D>() floats of workgroup memory, 16-byte aligned;
-// wg_linear: this workgroup's index in [0, nq * B * Hq).
-template <int D, int NW, bool CAUSAL>
+// The kernel body.  lds: flash_f32_lds_floats<D, NW, SPLITK>() floats of workgroup memory, 16-byte
+// aligned; wg_linear: this workgroup's index in [0, nq * B * Hq).
+//
+// SPLITK (few, short heads: the launch would otherwise leave most SIMDs idle behind one wave's
+// chain of matrix instructions): the NW waves of a workgroup share the same 32 queries and deal
+// the key tiles out between them (wave w takes tiles w, w + NW, ...), each staging its own tiles
+// in its own LDS slab with no workgroup barrier; at the end the partial (m, l, O) of the waves are
+// merged through LDS: m = max m_w, l = sum l_w e^(m_w - m), O = sum O_w e^(m_w - m).
+template <int D, int NW, bool CAUSAL, bool SPLITK = false>
 __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *lds, int wg_linear)
 {
-    constexpr int T = NW * 64;
-    constexpr int BQ = NW * 32;
+    constexpr int T = SPLITK ? 64 : NW * 64;      // threads staging one tile
+    constexpr int BQ = SPLITK ? 32 : NW * 32;
     constexpr int HALF = D / 2;          // channels per lane half
     constexpr int KROW = D + 4;          // padded K row (floats): conflict-free 128-bit row reads
     constexpr int DB = D / 32;
@@ -57,10 +63,11 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     constexpr int PER_THREAD = (CHUNKS + T - 1) / T;
     static_assert(CHUNKS % T == 0, "tile staging must divide evenly");
 
-    float *ks = lds;                  // [F32_BK][KROW]
-    float *vs = lds + F32_BK * KROW;  // [F32_BK][D]
-
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int SLAB = F32_BK * KROW + F32_BK * D;
+    float *ks = lds + (SPLITK ? wave * SLAB : 0);  // [F32_BK][KROW]
+    float *vs = ks + F32_BK * KROW;                // [F32_BK][D]
+    const int stid = SPLITK ? lane : tid;          // index among the threads staging a tile
     const int i32 = lane & 31, h = lane >> 5;
     const int bh = wg_linear / p.nq;
     int qt = wg_linear - bh * p.nq;
@@ -68,7 +75,7 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     const int b = bh / p.Hq, head = bh - b * p.Hq;
     const int N = p.N;
     const int qblk = qt * BQ;
-    const int wq0 = qblk + wave * 32;
+    const int wq0 = qblk + (SPLITK ? 0 : wave * 32);
     const int q_row = wq0 + i32;
 
     int kvl = N;
@@ -105,23 +112,37 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
         for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
     float m_run = -1e30f, l_run = 0.f;
 
-    for (int it = 0; it < ntiles; ++it) {
-        const int k0 = it * F32_BK;
-        __syncthreads();  // the previous tile has been consumed
+    // The global loads of a tile are issued one tile ahead of its use, into registers, so that
+    // their latency is spent under the matrix instructions of the tile before.
+    float4 kx[PER_THREAD], vx[PER_THREAD];
+    auto fetch = [&](int tile) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < PER_THREAD; ++j) {
-            const int c = tid + j * T;
+            const int c = stid + j * T;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-            const int gr = k0 + row;
-            float4 kx = make_float4(0.f, 0.f, 0.f, 0.f), vx = kx;
+            const int gr = tile * F32_BK + row;
+            kx[j] = vx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (gr < kend) {
-                kx = *(const float4 *)(kp + (size_t)gr * k_rs + col);
-                vx = *(const float4 *)(vp + (size_t)gr * k_rs + col);
+                kx[j] = *(const float4 *)(kp + (size_t)gr * k_rs + col);
+                vx[j] = *(const float4 *)(vp + (size_t)gr * k_rs + col);
             }
-            *(float4 *)&ks[row * KROW + col] = kx;
-            *(float4 *)&vs[row * D + col] = vx;
         }
-        __syncthreads();
+    };
+    constexpr int STEP = SPLITK ? NW : 1;
+    const int first = SPLITK ? wave : 0;
+    if (first < ntiles) fetch(first);
+    for (int it = first; it < ntiles; it += STEP) {
+        const int k0 = it * F32_BK;
+        if (!SPLITK) __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int c = stid + j * T;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            *(float4 *)&ks[row * KROW + col] = kx[j];
+            *(float4 *)&vs[row * D + col] = vx[j];
+        }
+        if (it + STEP < ntiles) fetch(it + STEP);
+        if (!SPLITK) __syncthreads();
         if (it >= my_tiles) continue;  // under the causal mask this wave is done (it still helps staging)
 
         // ---- S^T = K . Q^T ----
@@ -179,6 +200,54 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if constexpr (SPLITK) {
+        // ---- merge the waves' partial results ----
+        // slab of wave w, reused: O_w as [32 queries][D + 4], then m_w[32], l_w[32]
+        constexpr int OROW = D + 4;
+        static_assert(32 * OROW + 64 <= SLAB, "merge buffers fit the staging slab");
+        float *ow = lds + wave * SLAB;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                *(float4 *)&ow[i32 * OROW + db * 32 + 8 * g + 4 * h] =
+                    make_float4(oacc[db][4 * g], oacc[db][4 * g + 1], oacc[db][4 * g + 2], oacc[db][4 * g + 3]);
+        if (h == 0) {
+            ow[32 * OROW + i32] = m_run;
+            ow[32 * OROW + 32 + i32] = l_tot;
+        }
+        __syncthreads();
+        // thread t: query t % 32, channels [cg * CPT, cg * CPT + CPT)
+        constexpr int CPT = D / (NW * 2);
+        static_assert(CPT % 4 == 0, "whole float4s per thread");
+        const int q = tid & 31, cg = tid >> 5;
+        const int row = qblk + q;
+        float m = -1e30f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) m = fmaxf(m, lds[w * SLAB + 32 * OROW + q]);
+        float l = 0.f, acc[CPT];
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) acc[c] = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float f = expf(lds[w * SLAB + 32 * OROW + q] - m);
+            l += lds[w * SLAB + 32 * OROW + 32 + q] * f;
+#pragma unroll
+            for (int c = 0; c < CPT; c += 4) {
+                const float4 x = *(const float4 *)&lds[w * SLAB + q * OROW + cg * CPT + c];
+                acc[c] += x.x * f; acc[c + 1] += x.y * f; acc[c + 2] += x.z * f; acc[c + 3] += x.w * f;
+            }
+        }
+        const float inv = (l > 0.f) ? 1.f / l : 0.f;
+        if (row < N) {
+            if (p.lse != nullptr && cg == 0) p.lse[(size_t)bh * N + row] = (l > 0.f) ? m + logf(l) : -1e30f;
+            float *op = p.o + (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)row * p.os[2] + cg * CPT;
+#pragma unroll
+            for (int c = 0; c < CPT; c += 4)
+                *(float4 *)(op + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
+        }
+        return;
+    }
     const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
     if (p.lse != nullptr && h == 0 && q_row < N)
         p.lse[(size_t)bh * N + q_row] = (l_tot > 0.f) ? m_run + logf(l_tot) : -1e30f;
@@ -195,11 +264,11 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     }
 }
 
-template <int D, int NW, bool CAUSAL>
+template <int D, int NW, bool CAUSAL, bool SPLITK = false>
 __global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params p)
 {
-    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<D>()];
-    flash_f32_body<D, NW, CAUSAL>(p, lds, (int)blockIdx.x);
+    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<D, NW, SPLITK>()];
+    flash_f32_body<D, NW, CAUSAL, SPLITK>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

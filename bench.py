@@ -108,7 +108,7 @@ class SageWorkload:
         ach = self.ops / secs / 1e12
         return {"bound": "mfma", "achieved": ach, "peak": PEAK_INT8, "unit": "TOP/s", "frac": ach / PEAK_INT8,
                 "traffic": MEASURED_TRAFFIC.get(self.name), "traffic_source": "rocprofv3 --pmc profile (profiles/), not this run",
-                "kernel": "attn_pipe_kernel<int8>", "launch_ms": secs * 1e3,
+                "kernel": "attn_fwd_kernel<int8>" if self.bk == 1 else "attn_pipe_kernel<int8>", "launch_ms": secs * 1e3,
                 "ops_per_launch": self.ops, "peak_note": "dense int8 MFMA; half of the ops are bf16 (P.V)",
                 "frac_of_mixed_int8_bf16_bound": t_min / secs}
 
@@ -194,6 +194,19 @@ def measure(dev, w, steps, warmup):
            "roofline": w.roofline(ksecs / max(kn, 1))}
     if qn:
         res["prepass_ms_per_step"] = qsecs / steps * 1e3
+    if w.S < 1024:
+        # launch-bound shapes: the same steps recorded once into a HIP graph and replayed as one
+        # submission (the reference's captured replay, src/engine/jit.rs:186-195), so that the
+        # per-launch host overhead drops out of the step time
+        dev.graph_begin()
+        for _ in range(steps):
+            w.step()
+        g = dev.graph_end()
+        dev.graph_launch(g)
+        reps = 5
+        secs = min(dev.graph_launch(g) for _ in range(reps))
+        dev.graph_destroy(g)
+        res["ms_per_step_graph_replay"] = secs / steps * 1e3
     return res
 
 
@@ -383,6 +396,8 @@ def main():
         line["roofline"]["frac_of_sustained_bf16_mfma_rate"] = (
             (res["ops_per_step"] / 2 / (PEAK_INT8 / PEAK_BF16) + res["ops_per_step"] / 2) if w.dtype == "int8"
             else res["ops_per_step"]) / (line["roofline"]["launch_ms"] * 1e-3) / 1e12 / power["random"]["tflops"]
+    if "ms_per_step_graph_replay" in res:
+        line["ms_per_step_graph_replay"] = res["ms_per_step_graph_replay"]
     if secondary:
         line["secondary"] = secondary
     print(json.dumps(line), flush=True)
