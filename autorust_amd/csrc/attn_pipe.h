@@ -120,7 +120,10 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     int kend = kvl;
     if (CAUSAL) kend = min(kend, min(N, qblk + BQ));
     const int ntiles = (kend + BK - 1) / BK;
-    const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / BK + 1) : ntiles;
+    // key `key` is masked for this lane's query iff key > min(q_row, kend - 1) (causal) or
+    // key > kend - 1.  Element r of a block whose first key is kb0 is key kb0 + 4 h + 8 (r / 4) + r % 4,
+    // so with rel = lim4h - kb0 the test is 8 (r / 4) + r % 4 > rel.
+    const int lim4h = (CAUSAL ? min(q_row, kend - 1) : kend - 1) - 4 * h;
 
     // ---- buffer resources over this head's K and V: offsets past kend rows read as zero ----
     const size_t kv_off = (size_t)b * p.ks[0] + (size_t)kvh * p.ks[1];
@@ -329,7 +332,9 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     // not finite (the first block, or a jump of the maximum), moves the reference and redoes the
     // block.  Rare, so the raw logits are not kept for it: they are recomputed from the K block,
     // which is still in LDS (block blk of stage st).
-    auto fix_reference = [&](const unsigned char *st, int blk, float c, uint4 (&pb)[2], float &rs) __attribute__((always_inline)) {
+    auto fix_reference = [&](auto masked, const unsigned char *st, int blk, float c, int rel, uint4 (&pb)[2], float &rs)
+                             __attribute__((always_inline)) {
+        constexpr bool M = decltype(masked)::value;
         acc_t s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0;
@@ -346,38 +351,36 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         // ordinary vector instructions, so the result has landed by the time max3 runs
         float x[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) x[r] = (float)s[r] * c;
-        float mx = max3(x[0], x[1], x[2]);
-#pragma unroll
-        for (int r = 3; r < 15; r += 2) mx = max3(mx, x[r], x[r + 1]);
-        mx = xhalf_max(fmaxf(mx, x[15]));
-        move_reference(mx);
-        exp_pack(s, c, pb, rs);
-    };
-    // a block with masked keys (causal diagonal, key-length edge), no look-ahead
-    auto masked_block = [&](const unsigned char *st, int blk, int k0, float c) __attribute__((always_inline)) {
-        load_kf(st, blk);
-        load_vf(st, blk);
-        const acc_t s = mfma_qk();
-        float x[16];
-#pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int key = k0 + blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-            float xv = (float)s[r] * c;
-            if (key >= kend || (CAUSAL && key > q_row)) xv = NEG_SENTINEL;
-            x[r] = xv;
+            x[r] = (float)s[r] * c;
+            if (M && 8 * (r >> 2) + (r & 3) > rel) x[r] = NEG_SENTINEL;
         }
         float mx = max3(x[0], x[1], x[2]);
 #pragma unroll
         for (int r = 3; r < 15; r += 2) mx = max3(mx, x[r], x[r + 1]);
         mx = xhalf_max(fmaxf(mx, x[15]));
-        if (__any(mx > m_run + LAZY_TAU)) move_reference(mx);
+        move_reference(mx);
+        if constexpr (M) {
+            // masked keys contribute exactly 0 whatever the reference is
+            float half[2];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_run);
-        l_run += row_sum(x);
-        uint4 pb[2];
-        pack(x, pb);
-        mfma_pv(pb);
+            for (int ks = 0; ks < 2; ++ks) {
+                float e[8];
+#pragma unroll
+                for (int r = 0; r < 8; ++r) {
+                    const int rr = ks * 8 + r;
+                    e[r] = (8 * (rr >> 2) + (rr & 3) > rel) ? 0.f : __builtin_amdgcn_exp2f(x[rr] - m_run);
+                }
+                half[ks] = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+                pb[ks].x = pack_bf16x2(e[0], e[1]);
+                pb[ks].y = pack_bf16x2(e[2], e[3]);
+                pb[ks].z = pack_bf16x2(e[4], e[5]);
+                pb[ks].w = pack_bf16x2(e[6], e[7]);
+            }
+            rs = half[0] + half[1];
+        } else {
+            exp_pack(s, c, pb, rs);
+        }
     };
 
     uint4 pb[2];     // P of the block about to be multiplied with V
@@ -389,7 +392,8 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     constexpr int SM_HALF = SM_CVT + 8 + 8 + 7 + 4;
     constexpr int SM_OPS = 2 * SM_HALF;
     float sm_t[8], sm_x[8], sm_a[6], sm_half[2];
-    auto sm_op = [&](auto ic, const acc_t &s, float c, uint4 (&pn)[2]) __attribute__((always_inline)) {
+    auto sm_op = [&](auto masked, auto ic, const acc_t &s, float c, int rel, uint4 (&pn)[2]) __attribute__((always_inline)) {
+        constexpr bool M = decltype(masked)::value;
         constexpr int i = decltype(ic)::value;
         constexpr int ks = i / SM_HALF, k = i % SM_HALF;
         if constexpr (k < SM_CVT) {
@@ -397,6 +401,8 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         } else if constexpr (k < SM_CVT + 8) {
             constexpr int r = k - SM_CVT;
             sm_t[r] = __builtin_fmaf((MODE == MODE_I8) ? sm_t[r] : (float)s[ks * 8 + r], c, -m_run);
+            // a masked key: exp2 of the sentinel is exactly 0
+            if (M && 8 * ((ks * 8 + r) >> 2) + (r & 3) > rel) sm_t[r] = NEG_SENTINEL;
         } else if constexpr (k < SM_CVT + 16) {
             constexpr int r = k - SM_CVT - 8;
             sm_x[r] = __builtin_amdgcn_exp2f(sm_t[r]);
@@ -430,8 +436,11 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     constexpr int R2_SLOTS = DB * 2 - 2;  // S is not ready under the first two O^T MFMAs
     constexpr int SM_SPLIT = (MODE == MODE_I8) ? (SM_OPS * R2_SLOTS) / (R2_SLOTS + KSTEPS) : SM_HALF;
     uint4 pn[2];  // P of the block whose softmax is in progress
-    auto pipe_block = [&](acc_t &s_old, acc_t &s_new, const unsigned char *sc, int cb, const unsigned char *sv, int vb,
-                          const unsigned char *sk, int kb, float c_cur, float c_next) __attribute__((always_inline)) {
+    // mc / mn: block j / block j+1 has masked keys (causal diagonal, key-length edge); rel_cur /
+    // rel_next are their mask offsets (see lim4h).
+    auto pipe_block = [&](auto mc, auto mn, acc_t &s_old, acc_t &s_new, const unsigned char *sc, int cb,
+                          const unsigned char *sv, int vb, const unsigned char *sk, int kb, float c_cur, float c_next,
+                          int rel_cur, int rel_next) __attribute__((always_inline)) {
         // ---- R1 ----
 #pragma unroll
         for (int r = 0; r < 16; ++r) s_new[r] = 0;
@@ -444,12 +453,12 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
                 s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s_new, 0, 0, 0);
             ARHIP_FENCE();
             constexpr int lo = SM_SPLIT + st * (SM_OPS - SM_SPLIT) / KSTEPS, hi = SM_SPLIT + (st + 1) * (SM_OPS - SM_SPLIT) / KSTEPS;
-            static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(ic, s_old, c_cur, pn); });
+            static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mc, ic, s_old, c_cur, rel_cur, pn); });
             kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
             ARHIP_FENCE();
         });
         rs = sm_half[0] + sm_half[1];
-        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(sc, cb, c_cur, pn, rs);
+        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(mc, sc, cb, c_cur, rel_cur, pn, rs);
         l_run += rs;
         pb[0] = pn[0];
         pb[1] = pn[1];
@@ -464,7 +473,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
             ARHIP_FENCE();
             if constexpr (g >= 2) {
                 constexpr int lo = (g - 2) * SM_SPLIT / R2_SLOTS, hi = (g - 1) * SM_SPLIT / R2_SLOTS;
-                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(ic, s_new, c_next, pn); });
+                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mn, ic, s_new, c_next, rel_next, pn); });
             }
             if constexpr (ks == 1) {
 #pragma unroll
@@ -478,11 +487,11 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     };
 
     // ---- prologue: tiles 0..2 on their way, tiles 0 and 1 visible ----
-    // The pipelined loop covers the tiles in which no key is masked for ANY wave of the workgroup
-    // (all full tiles; under the causal mask those before the workgroup's first query), so that
-    // every wave runs the same code between barriers.  The remaining tiles (at most 4 on the causal
-    // diagonal, or the last partial one) go block by block with the masks applied.
-    const int npipe = CAUSAL ? min(kend / BK, qblk / BK) : kend / BK;
+    // Tiles [0, nfull) have no masked key for ANY wave of the workgroup (all full tiles; under the
+    // causal mask those before the workgroup's first query); the remaining ones (at most 4 on the
+    // causal diagonal, or the last partial one) run the same pipeline with the mask applied inside
+    // the softmax.  Every wave runs every tile, so all waves execute the same code between barriers.
+    const int nfull = CAUSAL ? min(kend / BK, qblk / BK) : kend / BK;
     issue_tile(0, 0);
     issue_tile(1, 1);
     issue_tile(2, 2);
@@ -504,38 +513,49 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     acc_t s_a, s_b;  // logits of the even / odd block of a tile
 #pragma unroll
     for (int r = 0; r < 16; ++r) s_a[r] = s_b[r] = 0;
-    if (npipe > 0) {
+    constexpr std::false_type PLAIN{};
+    constexpr std::true_type MASKED{};
+    if (ntiles > 0) {
         load_kf(lds, 0);
         s_a = mfma_qk();
         load_kf(lds, 1);
         load_vf(lds, 0);
         const float c0 = tile_c(0, 0);
-        static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(ic, s_a, c0, pn); });
+        if (nfull > 0)
+            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(PLAIN, ic, s_a, c0, 0, pn); });
+        else
+            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(MASKED, ic, s_a, c0, lim4h, pn); });
     }
 
-#pragma clang loop unroll(disable)
-    for (int it = 0; it < npipe; ++it) {
+    // one tile: its two blocks; m0 / m1 / m2 say whether the first block, the second block and the
+    // first block of the next tile have masked keys
+    auto tile_iter = [&](auto m0, auto m1, auto m2, int it) __attribute__((always_inline)) {
         const unsigned char *st_cur = lds + (it & 3) * STAGE;
         const unsigned char *st_nxt = lds + ((it + 1) & 3) * STAGE;
         // tile it + 3 goes to the stage tile it - 1 vacated at the last barrier
         issue_tile(it + 3, (it + 3) & 3);
         advance_sk_group(it);
         const float c_cur = tile_c(it, it), c_nxt = tile_c(it + 1, it);
-        pipe_block(s_a, s_b, st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, c_cur);
-        pipe_block(s_b, s_a, st_cur, 1, st_nxt, 0, st_nxt, 1, c_cur, c_nxt);
+        const int rel0 = lim4h - it * BK;
+        pipe_block(m0, m1, s_a, s_b, st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, c_cur, rel0, rel0 - 32);
+        pipe_block(m1, m2, s_b, s_a, st_cur, 1, st_nxt, 0, st_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64);
         wait_vmem_le<XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
         __syncthreads();
-    }
+    };
+    // the last unmasked tile hands a masked block to the look-ahead: it is peeled off
+    const int nplain = (nfull < ntiles) ? max(nfull - 1, 0) : nfull;
 #pragma clang loop unroll(disable)
-    for (int it = npipe; it < ntiles; ++it) {
-        const unsigned char *st_cur = lds + (it & 3) * STAGE;
+    for (int it = 0; it < nplain; ++it) tile_iter(PLAIN, PLAIN, PLAIN, it);
+    if (nplain < nfull) tile_iter(PLAIN, PLAIN, MASKED, nplain);
+    // under the causal mask a wave is done once the tiles start past its last query; it keeps
+    // feeding the transfers and the barriers the other waves rely on
+    const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / BK + 1) : ntiles;
+    // (two loops rather than a branch inside one: the accumulators would be copied at the join)
+#pragma clang loop unroll(disable)
+    for (int it = nfull; it < my_tiles; ++it) tile_iter(MASKED, MASKED, MASKED, it);
+#pragma clang loop unroll(disable)
+    for (int it = max(nfull, my_tiles); it < ntiles; ++it) {
         issue_tile(it + 3, (it + 3) & 3);
-        advance_sk_group(it);
-        if (it < my_tiles) {
-            const float c_cur = tile_c(it, it);
-            masked_block(st_cur, 0, it * BK, c_cur);
-            masked_block(st_cur, 1, it * BK, c_cur);
-        }
         wait_vmem_le<XPW_MIN>();
         __syncthreads();
     }
