@@ -15,7 +15,7 @@ KERNELS_PATH = os.path.join(_HERE, "attn_kernels.hsaco")
 OK, EINVAL, EUNSUPPORTED, EHIP, ENODEVICE = 0, -1, -2, -3, -4
 F32, BF16 = 0, 1
 ATTN_SDPA, ATTN_FLASH, ATTN_SAGE = 0, 1, 2
-K_FLASH_F32, K_FLASH_BF16, K_SAGE, K_SAGE_QUANT = 0, 1, 2, 3
+K_FLASH_F32, K_FLASH_BF16, K_SAGE, K_SAGE_QUANT, K_FLASH_BWD = 0, 1, 2, 3, 4
 
 c_void_p, c_int, c_int64, c_size_t = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
 c_float, c_double, c_char_p = ctypes.c_float, ctypes.c_double, ctypes.c_char_p
@@ -61,6 +61,7 @@ SIGNATURES = {
                                     ctypes.POINTER(c_int64), ctypes.POINTER(c_int64), ctypes.POINTER(c_int64),
                                     c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int, c_int, c_float, c_int, _pd]),
+    "arhip_flash_bwd": (c_int, [c_void_p] * 13 + [c_int64] * 5 + [c_int, c_float, c_int, _pd]),
     "arhip_sage_quant_workspace": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "arhip_sage_quant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),

@@ -19,7 +19,7 @@ HOST_LIB = os.path.join(HERE, "libautorust_host.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 SOURCES = ["device.hip", "flash.hip", "sage_quant.hip"]
-HEADERS = ["arhip_internal.h", "attn_fwd.h", "attn_pipe.h", "flash_f32.h", "sage_quant_kernels.h", os.path.join("..", "..", "include", "arhip.h")]
+HEADERS = ["arhip_internal.h", "attn_fwd.h", "attn_pipe.h", "flash_f32.h", "flash_bwd_f32.h", "sage_quant_kernels.h", os.path.join("..", "..", "include", "arhip.h")]
 
 # -packed-fp32-ops off: packed fp32 VALU instructions are not used by this build.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -20,11 +20,18 @@
 // The Sage entries take pre-quantised operands (the quantiser is the pre-pass below, not part of
 // the attention kernel as in the reference):
 //     (Q8, K8, V, O, M, SQ, SK,  N, head_dim, causal, has_mask, hq, hkv, bq, bk [, out_f32])
+// Training (src/runtime/cuda_flash_train.rs:57-309), f32, dense, the reference's argument order with
+// head_dim inserted after N:
+//   ar_fl_fwd      [256,1,1]  [ceil(n/128), B*hq, 1]   (Q, K, V, O, LSE, M,  N, head_dim, causal, has_mask, hq, hkv)
+//   ar_fl_prep     [256,1,1]  [ceil(n/4), B*hq, 1]     (O, dO, D,  N, head_dim)
+//   ar_fl_bwd_dq   [256,1,1]  [ceil(n/128), B*hq, 1]   (Q, K, V, dO, LSE, D, M, dQ,  N, head_dim, causal, has_mask, hq, hkv)
+//   ar_fl_bwd_dkv  [256,1,1]  [ceil(n/128), B*hkv, 1]  (Q, K, V, dO, LSE, D, M, dK, dV,  N, head_dim, causal, has_mask, hq, hkv)
 // head_dim must be 64 or 128; any other value makes the kernel return without writing.
 // The *_long entries address K and V with 32-bit byte offsets: (N + 320) * head_dim * 2 < 2^31.
 #include "attn_fwd.h"
 #include "attn_pipe.h"
 #include "flash_f32.h"
+#include "flash_bwd_f32.h"
 // last: it switches floating-point contraction off for the rest of the file
 #include "sage_quant_kernels.h"
 
@@ -84,6 +91,88 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_f32(const float *Q, c
     } else if (head_dim == 128) {
         if (causal) flash_f32_body<128, 4, true>(p, lds, wg);
         else flash_f32_body<128, 4, false>(p, lds, wg);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_fl_fwd(const float *Q, const float *K, const float *V, float *O,
+                                                             float *LSE, const float *M, int N, int head_dim, int causal,
+                                                             int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<128>()];
+    FlashF32Params p = {};
+    p.q = Q; p.k = K; p.v = V; p.o = O; p.lse = LSE;
+    p.mask = has_mask ? M : nullptr;
+    p.Hq = hq; p.Hkv = hkv; p.N = N;
+    p.nq = (int)gridDim.x;
+    dense(p.qs, hq, N, head_dim);
+    dense(p.ks, hkv, N, head_dim);
+    dense(p.os, hq, N, head_dim);
+    p.scale = 1.0f / __builtin_sqrtf((float)head_dim);
+    const int wg = linear_wg();
+    if (head_dim == 64) {
+        if (causal) flash_f32_body<64, 4, true>(p, lds, wg);
+        else flash_f32_body<64, 4, false>(p, lds, wg);
+    } else if (head_dim == 128) {
+        if (causal) flash_f32_body<128, 4, true>(p, lds, wg);
+        else flash_f32_body<128, 4, false>(p, lds, wg);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_fl_prep(const float *O, const float *dO, float *D, int N, int head_dim)
+{
+    const long row0 = (long)blockIdx.y * N + (long)blockIdx.x * 4, rows = ((long)blockIdx.y + 1) * N;
+    if (head_dim == 64) bwd_prep_body<64>(O, dO, D, rows, row0);
+    else if (head_dim == 128) bwd_prep_body<128>(O, dO, D, rows, row0);
+}
+
+namespace {
+__device__ __forceinline__ FlashBwdParams bwd_params(const float *Q, const float *K, const float *V, const float *dO,
+                                                     const float *LSE, const float *D, const float *M, int N,
+                                                     int head_dim, int has_mask, int hq, int hkv)
+{
+    FlashBwdParams p = {};
+    p.q = Q; p.k = K; p.v = V; p.dout = dO; p.lse = LSE; p.delta = D;
+    p.mask = has_mask ? M : nullptr;
+    p.Hq = hq; p.Hkv = hkv; p.N = N;
+    p.nt = (int)gridDim.x;
+    p.scale = 1.0f / __builtin_sqrtf((float)head_dim);
+    return p;
+}
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(256) ar_fl_bwd_dq(const float *Q, const float *K, const float *V,
+                                                                const float *dO, const float *LSE, const float *D,
+                                                                const float *M, float *dQ, int N, int head_dim, int causal,
+                                                                int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<128>()];
+    FlashBwdParams p = bwd_params(Q, K, V, dO, LSE, D, M, N, head_dim, has_mask, hq, hkv);
+    p.dq = dQ;
+    const int wg = linear_wg();
+    if (head_dim == 64) {
+        if (causal) bwd_dq_body<64, 4, true>(p, lds, wg);
+        else bwd_dq_body<64, 4, false>(p, lds, wg);
+    } else if (head_dim == 128) {
+        if (causal) bwd_dq_body<128, 4, true>(p, lds, wg);
+        else bwd_dq_body<128, 4, false>(p, lds, wg);
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_fl_bwd_dkv(const float *Q, const float *K, const float *V,
+                                                                 const float *dO, const float *LSE, const float *D,
+                                                                 const float *M, float *dK, float *dV, int N, int head_dim,
+                                                                 int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<128>()];
+    FlashBwdParams p = bwd_params(Q, K, V, dO, LSE, D, M, N, head_dim, has_mask, hq, hkv);
+    p.dk = dK; p.dv = dV;
+    const int wg = linear_wg();
+    if (head_dim == 64) {
+        if (causal) bwd_dkv_body<64, 4, true>(p, lds, wg);
+        else bwd_dkv_body<64, 4, false>(p, lds, wg);
+    } else if (head_dim == 128) {
+        if (causal) bwd_dkv_body<128, 4, true>(p, lds, wg);
+        else bwd_dkv_body<128, 4, false>(p, lds, wg);
     }
 }
 

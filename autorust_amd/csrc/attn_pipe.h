@@ -158,8 +158,11 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     // The transfers are written as inline assembly on purpose: the compiler makes every LDS read
     // wait for all outstanding transfers it knows of (it cannot tell the stages apart), which
     // would put the whole memory latency in front of every tile.  Here the waits are explicit
-    // (wait_vmem_le before the barrier that publishes a tile).  m0 holds the LDS destination;
-    // one wait state is required between writing m0 and the transfer.
+    // (wait_vmem_le before the barrier that publishes a tile).  m0 holds the LDS destination; one
+    // wait state is required between writing m0 and the transfer, and five between a vector
+    // instruction writing a scalar register (v_readfirstlane of the descriptors, a scalar register
+    // reloaded from a spill lane) and a memory instruction reading it: the compiler pads neither
+    // for inline assembly, so the assembly carries the wait states itself (s_mov + s_nop 3).
     auto issue_tile = [&](int tile, int stage) __attribute__((always_inline)) {
         const uint32_t dst = (uint32_t)(uintptr_t)(lds_ptr_t)lds + stage * STAGE;
 #pragma unroll
@@ -171,7 +174,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
                 const bool is_k = x < KP * 4;
                 const uint32_t off = xoff[j] + (uint32_t)tile * BK * (is_k ? k_rowb : v_rowb);
                 const i32x4 rsrc = is_k ? k_rsrc : v_rsrc;
-                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                              :
                              : "s"(dst + x * 1024), "v"(off), "s"(rsrc)
                              : "memory", "m0");
@@ -273,32 +276,6 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s, 0, 0, 0);
         }
         return s;
-    };
-    auto mfma_pv = [&](const uint4 (&pb)[2]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                const uint4 a = make_uint4(vf[db][ks][0].x, vf[db][ks][0].y, vf[db][ks][1].x, vf[db][ks][1].y);
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                                   __builtin_bit_cast(bf16x8, pb[ks]), oacc[db], 0, 0, 0);
-            }
-    };
-    auto row_sum = [&](const float (&x)[16]) __attribute__((always_inline)) {
-        // over the unrounded probabilities (src/runtime/cuda_flash_bf16.rs:365-377)
-        float rs0 = (x[0] + x[1]) + (x[2] + x[3]), rs1 = (x[8] + x[9]) + (x[10] + x[11]);
-        rs0 += (x[4] + x[5]) + (x[6] + x[7]);
-        rs1 += (x[12] + x[13]) + (x[14] + x[15]);
-        return rs0 + rs1;
-    };
-    auto pack = [&](const float (&x)[16], uint4 (&pb)[2]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            pb[ks].x = pack_bf16x2(x[ks * 8 + 0], x[ks * 8 + 1]);
-            pb[ks].y = pack_bf16x2(x[ks * 8 + 2], x[ks * 8 + 3]);
-            pb[ks].z = pack_bf16x2(x[ks * 8 + 4], x[ks * 8 + 5]);
-            pb[ks].w = pack_bf16x2(x[ks * 8 + 6], x[ks * 8 + 7]);
-        }
     };
     auto move_reference = [&](float mx) __attribute__((always_inline)) {
         const float m_new = fmaxf(m_run, mx);

@@ -7,6 +7,7 @@
 #include "arhip_internal.h"
 #include "attn_fwd.h"
 #include "attn_pipe.h"
+#include "flash_bwd_f32.h"
 #include "flash_f32.h"
 
 #include <algorithm>
@@ -327,5 +328,47 @@ extern "C" int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const
 #undef SAGE_D
 #undef SAGE_V
     arhip_note_selected(ARHIP_K_SAGE);
+    return t.end();
+}
+
+extern "C" int arhip_flash_bwd(arhip_device *dev, const float *q, const float *k, const float *v, const float *o,
+                               const float *lse, const float *dout, float *dq, float *dk, float *dv, float *delta,
+                               const float *mask, const int32_t *kv_len,
+                               int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                               int causal, float scale, int wait, double *secs)
+{
+    if (int rc = check_common("arhip_flash_bwd", dev, q, k, v, o, mask, B, Hq, Hkv, N, D)) return rc;
+    ARHIP_REQUIRE(lse && dout && dq && dk && dv && delta, "arhip_flash_bwd: null tensor pointer");
+    ARHIP_REQUIRE(arhip_aligned16(dout) && arhip_aligned16(dq) && arhip_aligned16(dk) && arhip_aligned16(dv),
+                  "arhip_flash_bwd: dout/dq/dk/dv must be 16-byte aligned");
+    ARHIP_REQUIRE(((reinterpret_cast<uintptr_t>(lse) | reinterpret_cast<uintptr_t>(delta)) & 3u) == 0,
+                  "arhip_flash_bwd: lse/delta must be 4-byte aligned");
+    ARHIP_HIP(hipSetDevice(dev->ordinal));
+    arhip_call_timer t{dev, wait, secs};
+    t.kernel = ARHIP_K_FLASH_BWD;
+    FlashBwdParams p = {};
+    p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta; p.mask = mask; p.kv_len = kv_len;
+    p.dq = dq; p.dk = dk; p.dv = dv;
+    p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
+    p.scale = scale;
+    if (int rc = t.begin()) return rc;
+    const long rows = (long)(B * Hq * N);
+    const int nt = (int)((N + 127) / 128);
+    const dim3 block(256), grid_prep((unsigned)((rows + 3) / 4)), grid_q((unsigned)(nt * B * Hq)), grid_kv((unsigned)(nt * B * Hkv));
+    p.nt = nt;
+#define BWD_LAUNCH(DD)                                                                                  \
+    do {                                                                                                \
+        hipLaunchKernelGGL((bwd_prep_kernel<DD>), grid_prep, block, 0, dev->stream, o, dout, delta, rows); \
+        if (causal) {                                                                                   \
+            hipLaunchKernelGGL((bwd_dq_kernel<DD, 4, true>), grid_q, block, 0, dev->stream, p);         \
+            hipLaunchKernelGGL((bwd_dkv_kernel<DD, 4, true>), grid_kv, block, 0, dev->stream, p);       \
+        } else {                                                                                        \
+            hipLaunchKernelGGL((bwd_dq_kernel<DD, 4, false>), grid_q, block, 0, dev->stream, p);        \
+            hipLaunchKernelGGL((bwd_dkv_kernel<DD, 4, false>), grid_kv, block, 0, dev->stream, p);      \
+        }                                                                                               \
+    } while (0)
+    if (D == 64) BWD_LAUNCH(64); else BWD_LAUNCH(128);
+#undef BWD_LAUNCH
+    arhip_note_selected(ARHIP_K_FLASH_BWD);
     return t.end();
 }

@@ -1,0 +1,379 @@
+// fp32 FlashAttention backward: the softmax-backward row scalar, dQ, and dK/dV.
+//
+// Semantics of the reference's training kernels (src/runtime/cuda_flash_train.rs:145-309):
+//   prep   D[bh, i]  = sum_d O[i, d] dO[i, d]
+//   dQ     s = (q_i . k_j) scale (+ mask[i, j]);  p = lse_i > -5e29 ? exp(s - lse_i) : 0;
+//          dp = dO_i . v_j;  ds = p (dp - D_i) scale;  dQ_i = sum_j ds k_j
+//   dK/dV  dK_j = sum_{g, i} ds q_i;  dV_j = sum_{g, i} p dO_i   (g over the GQA group of the K/V head,
+//          in a fixed order: no atomics, bit-reproducible)
+// Keys past the diagonal (causal) or past kv_len contribute p = 0.  head_dim and scale are parameters
+// here (the reference hard-codes 64 and 0.125).
+//
+// All contractions run on v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate) with the decomposition of
+// the forward kernel (flash_f32.h): one row of the "resident" operand per lane.
+//   dQ kernel   a wave owns 32 queries (lane = query): S^T = K Q^T and dP^T = V dO^T leave, per lane,
+//               16 keys of one query, so lse_i and D_i are per-lane scalars and dS^T is already the B
+//               operand of dQ^T += K^T dS^T.  K and V tiles of 32 keys are staged in LDS.
+//   dK/dV kernel  a wave owns 32 keys (lane = key): S = Q K^T and dP = dO V^T leave, per lane, 16
+//               queries of one key; P and dS are the B operands of dV^T += dO^T P and dK^T += Q^T dS.
+//               Q and dO tiles of 32 queries (with their lse and D) are staged in LDS.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "flash_f32.h"
+
+namespace arhip {
+
+struct FlashBwdParams {
+    const float *q, *k, *v, *dout, *lse, *delta, *mask;
+    const int32_t *kv_len;  // [B] or null
+    float *dq, *dk, *dv;
+    int Hq, Hkv, N;
+    int nt;  // tiles per head: query tiles (dQ kernel) or key tiles (dK/dV kernel)
+    float scale;
+};
+
+constexpr float BWD_LSE_FLOOR = -5e29f;  // lse at or below: the row saw no key (cuda_flash_train.rs:206)
+
+// D[bh, i] = O[i] . dO[i]; one wave per row group: lane l of a wave sums channels l, l + 64, ...
+// in increasing order, then the 64 partial sums are added by a fixed butterfly.
+template <int D>
+__device__ __forceinline__ void bwd_prep_body(const float *o, const float *dout, float *delta, long rows, long row0)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long row = row0 + wave;
+    if (row >= rows) return;
+    float s = 0.f;
+#pragma unroll
+    for (int c = lane; c < D; c += 64) s += o[row * D + c] * dout[row * D + c];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off);
+    if (lane == 0) delta[row] = s;
+}
+
+template <int D>
+constexpr int bwd_lds_floats()
+{
+    return 2 * F32_BK * (D + 4) + 64;
+}
+
+// dQ.  lds: bwd_lds_floats<D>() floats.  Workgroup wg_linear in [0, nt * B * Hq): 32 NW queries of one head.
+template <int D, int NW, bool CAUSAL>
+__device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds, int wg_linear)
+{
+    constexpr int T = NW * 64;
+    constexpr int BQ = NW * 32;
+    constexpr int HALF = D / 2;
+    constexpr int ROW = D + 4;  // padded row: conflict-free 128-bit row reads
+    constexpr int DB = D / 32;
+    constexpr int CHUNKS = F32_BK * D / 4;
+    constexpr int PER_THREAD = CHUNKS / T;
+    static_assert(CHUNKS % T == 0, "tile staging must divide evenly");
+
+    float *ks = lds;
+    float *vs = lds + F32_BK * ROW;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i32 = lane & 31, h = lane >> 5;
+    const int bh = wg_linear / p.nt;
+    int qt = wg_linear - bh * p.nt;
+    if (CAUSAL) qt = p.nt - 1 - qt;
+    const int b = bh / p.Hq, head = bh - b * p.Hq;
+    const int N = p.N;
+    const int qblk = qt * BQ;
+    const int q_row = qblk + wave * 32 + i32;
+    const int rr = min(q_row, N - 1);
+    int kvl = N;
+    if (p.kv_len) {
+        kvl = p.kv_len[b];
+        kvl = kvl < 0 ? 0 : (kvl > N ? N : kvl);
+    }
+    int kend = kvl;
+    if (CAUSAL) kend = min(kend, min(N, qblk + BQ));
+    const int ntiles = (kend + F32_BK - 1) / F32_BK;
+    const int my_tiles = CAUSAL ? min(ntiles, (qblk + wave * 32 + 31) / F32_BK + 1) : ntiles;
+    const int kvh = head / (p.Hq / p.Hkv);
+    const float *kp = p.k + ((size_t)b * p.Hkv + kvh) * (size_t)N * D;
+    const float *vp = p.v + ((size_t)b * p.Hkv + kvh) * (size_t)N * D;
+    const size_t qoff = ((size_t)bh * N + rr) * D + h * HALF;
+
+    float qr[HALF], dor[HALF];
+#pragma unroll
+    for (int s = 0; s < HALF; s += 4) {
+        const float4 x = *(const float4 *)(p.q + qoff + s);
+        const float4 y = *(const float4 *)(p.dout + qoff + s);
+        qr[s] = x.x; qr[s + 1] = x.y; qr[s + 2] = x.z; qr[s + 3] = x.w;
+        dor[s] = y.x; dor[s + 1] = y.y; dor[s + 2] = y.z; dor[s + 3] = y.w;
+    }
+    const float lse = p.lse[(size_t)bh * N + rr];
+    const float di = p.delta[(size_t)bh * N + rr];
+    const bool row_live = lse > BWD_LSE_FLOOR;
+
+    f32x16_t acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+
+    float4 kx[PER_THREAD], vx[PER_THREAD];
+    auto fetch = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int c = tid + j * T;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            const int gr = tile * F32_BK + row;
+            kx[j] = vx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (gr < kend) {
+                kx[j] = *(const float4 *)(kp + (size_t)gr * D + col);
+                vx[j] = *(const float4 *)(vp + (size_t)gr * D + col);
+            }
+        }
+    };
+    if (ntiles > 0) fetch(0);
+    for (int it = 0; it < ntiles; ++it) {
+        const int k0 = it * F32_BK;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int c = tid + j * T;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            *(float4 *)&ks[row * ROW + col] = kx[j];
+            *(float4 *)&vs[row * ROW + col] = vx[j];
+        }
+        if (it + 1 < ntiles) fetch(it + 1);
+        __syncthreads();
+        if (it >= my_tiles) continue;
+
+        // S^T = K Q^T and dP^T = V dO^T: lane = query, register r = key 8 (r / 4) + 4 h + r % 4
+        f32x16_t s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+        const float *krow = &ks[i32 * ROW + h * HALF];
+        const float *vrow = &vs[i32 * ROW + h * HALF];
+#pragma unroll
+        for (int st = 0; st < HALF; st += 4) {
+            const float4 a = *(const float4 *)(krow + st);
+            const float4 c = *(const float4 *)(vrow + st);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, qr[st + 0], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.x, dor[st + 0], dp, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, qr[st + 1], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.y, dor[st + 1], dp, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, qr[st + 2], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.z, dor[st + 2], dp, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, qr[st + 3], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.w, dor[st + 3], dp, 0, 0, 0);
+        }
+        float ds[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = k0 + 8 * (r >> 2) + 4 * h + (r & 3);
+            float xv = s[r] * p.scale;
+            if (p.mask != nullptr && key < N) xv += p.mask[(size_t)rr * N + key];
+            const bool dead = key >= kend || (CAUSAL && key > q_row) || !row_live;
+            const float pr = dead ? 0.f : expf(xv - lse);
+            ds[r] = pr * (dp[r] - di) * p.scale;
+        }
+        // dQ^T += K^T dS^T: step (g, t) multiplies key 8 g + 4 h + t
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float *kcol = &ks[(8 * (r >> 2) + 4 * h + (r & 3)) * ROW + i32];
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(kcol[db * 32], ds[r], acc[db], 0, 0, 0);
+        }
+    }
+    if (q_row < N) {
+        float *op = p.dq + ((size_t)bh * N + q_row) * D;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                *(float4 *)(op + db * 32 + 8 * g + 4 * h) =
+                    make_float4(acc[db][4 * g], acc[db][4 * g + 1], acc[db][4 * g + 2], acc[db][4 * g + 3]);
+    }
+}
+
+// dK and dV.  Workgroup wg_linear in [0, nt * B * Hkv): 32 NW keys of one K/V head.
+template <int D, int NW, bool CAUSAL>
+__device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds, int wg_linear)
+{
+    constexpr int T = NW * 64;
+    constexpr int BKW = NW * 32;  // keys per workgroup
+    constexpr int HALF = D / 2;
+    constexpr int ROW = D + 4;
+    constexpr int DB = D / 32;
+    constexpr int CHUNKS = F32_BK * D / 4;
+    constexpr int PER_THREAD = CHUNKS / T;
+    static_assert(CHUNKS % T == 0, "tile staging must divide evenly");
+
+    float *qs = lds;
+    float *dos = lds + F32_BK * ROW;
+    float *stat = lds + 2 * F32_BK * ROW;  // lse[32], D[32] of the staged queries
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i32 = lane & 31, h = lane >> 5;
+    const int kv_bh = wg_linear / p.nt;
+    const int kt = wg_linear - kv_bh * p.nt;
+    const int b = kv_bh / p.Hkv, kvh = kv_bh - b * p.Hkv;
+    const int group = p.Hq / p.Hkv;
+    const int N = p.N;
+    const int kblk = kt * BKW;
+    const int wk0 = kblk + wave * 32;
+    const int key = wk0 + i32;
+    const int jj = min(key, N - 1);
+    int kvl = N;
+    if (p.kv_len) {
+        kvl = p.kv_len[b];
+        kvl = kvl < 0 ? 0 : (kvl > N ? N : kvl);
+    }
+    const bool key_live = key < kvl;
+
+    float kr[HALF], vr[HALF];
+    {
+        const size_t off = ((size_t)kv_bh * N + jj) * D + h * HALF;
+#pragma unroll
+        for (int s = 0; s < HALF; s += 4) {
+            const float4 x = *(const float4 *)(p.k + off + s);
+            const float4 y = *(const float4 *)(p.v + off + s);
+            kr[s] = x.x; kr[s + 1] = x.y; kr[s + 2] = x.z; kr[s + 3] = x.w;
+            vr[s] = y.x; vr[s + 1] = y.y; vr[s + 2] = y.z; vr[s + 3] = y.w;
+        }
+    }
+    f32x16_t dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dk[db][r] = dv[db][r] = 0.f;
+
+    // queries before the workgroup's first key see none of its keys under the causal mask
+    const int qt0 = CAUSAL ? kblk / F32_BK : 0;
+    const int qtiles = (N + F32_BK - 1) / F32_BK;
+    const int steps = group * (qtiles - qt0);  // (head of the group, query tile) pairs, head-major
+
+    float4 qx[PER_THREAD], dx[PER_THREAD];
+    float st_l = 0.f, st_d = 0.f;
+    auto fetch = [&](int step) __attribute__((always_inline)) {
+        const int g = step / (qtiles - qt0);
+        const int q0 = (qt0 + step - g * (qtiles - qt0)) * F32_BK;
+        const size_t bh = (size_t)b * p.Hq + (size_t)kvh * group + g;
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int c = tid + j * T;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            const int gr = q0 + row;
+            qx[j] = dx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (gr < N) {
+                qx[j] = *(const float4 *)(p.q + (bh * N + gr) * D + col);
+                dx[j] = *(const float4 *)(p.dout + (bh * N + gr) * D + col);
+            }
+        }
+        if (tid < F32_BK) {
+            const int gr = q0 + tid;
+            st_l = gr < N ? p.lse[bh * N + gr] : -1e30f;
+            st_d = gr < N ? p.delta[bh * N + gr] : 0.f;
+        }
+    };
+    if (steps > 0) fetch(0);
+    for (int step = 0; step < steps; ++step) {
+        const int g = step / (qtiles - qt0);
+        const int q0 = (qt0 + step - g * (qtiles - qt0)) * F32_BK;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int c = tid + j * T;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            *(float4 *)&qs[row * ROW + col] = qx[j];
+            *(float4 *)&dos[row * ROW + col] = dx[j];
+        }
+        if (tid < F32_BK) {
+            stat[tid] = st_l;
+            stat[32 + tid] = st_d;
+        }
+        if (step + 1 < steps) fetch(step + 1);
+        __syncthreads();
+        if (CAUSAL && q0 + F32_BK - 1 < wk0) continue;  // every query of the tile precedes this wave's keys
+
+        // S = Q K^T and dP = dO V^T: lane = key, register r = query 8 (r / 4) + 4 h + r % 4 of the tile
+        f32x16_t s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+        const float *qrow = &qs[i32 * ROW + h * HALF];
+        const float *drow = &dos[i32 * ROW + h * HALF];
+#pragma unroll
+        for (int st = 0; st < HALF; st += 4) {
+            const float4 a = *(const float4 *)(qrow + st);
+            const float4 c = *(const float4 *)(drow + st);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, kr[st + 0], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.x, vr[st + 0], dp, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, kr[st + 1], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.y, vr[st + 1], dp, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, kr[st + 2], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.z, vr[st + 2], dp, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, kr[st + 3], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.w, vr[st + 3], dp, 0, 0, 0);
+        }
+        float pr[16], ds[16];
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            const float4 l4 = *(const float4 *)&stat[8 * gq + 4 * h];
+            const float4 d4 = *(const float4 *)&stat[32 + 8 * gq + 4 * h];
+            const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dvv[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int r = 4 * gq + t;
+                const int qi = q0 + 8 * gq + 4 * h + t;
+                float xv = s[r] * p.scale;
+                if (p.mask != nullptr && qi < N) xv += p.mask[(size_t)qi * N + jj];
+                const bool dead = qi >= N || !key_live || (CAUSAL && key > qi) || !(lv[t] > BWD_LSE_FLOOR);
+                pr[r] = dead ? 0.f : expf(xv - lv[t]);
+                ds[r] = pr[r] * (dp[r] - dvv[t]) * p.scale;
+            }
+        }
+        // dV^T += dO^T P and dK^T += Q^T dS: step (g, t) multiplies query 8 g + 4 h + t of the tile
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int qi = 8 * (r >> 2) + 4 * h + (r & 3);
+            const float *dcol = &dos[qi * ROW + i32];
+            const float *qcol = &qs[qi * ROW + i32];
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                dv[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(dcol[db * 32], pr[r], dv[db], 0, 0, 0);
+                dk[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(qcol[db * 32], ds[r], dk[db], 0, 0, 0);
+            }
+        }
+    }
+    if (key < N) {
+        float *okp = p.dk + ((size_t)kv_bh * N + key) * D;
+        float *ovp = p.dv + ((size_t)kv_bh * N + key) * D;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = db * 32 + 8 * g + 4 * h;
+                *(float4 *)(okp + d) = make_float4(dk[db][4 * g], dk[db][4 * g + 1], dk[db][4 * g + 2], dk[db][4 * g + 3]);
+                *(float4 *)(ovp + d) = make_float4(dv[db][4 * g], dv[db][4 * g + 1], dv[db][4 * g + 2], dv[db][4 * g + 3]);
+            }
+    }
+}
+
+template <int D>
+__global__ void __launch_bounds__(256) bwd_prep_kernel(const float *o, const float *dout, float *delta, long rows)
+{
+    bwd_prep_body<D>(o, dout, delta, rows, (long)blockIdx.x * 4);
+}
+
+template <int D, int NW, bool CAUSAL>
+__global__ void __launch_bounds__(NW * 64) bwd_dq_kernel(const FlashBwdParams p)
+{
+    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<D>()];
+    bwd_dq_body<D, NW, CAUSAL>(p, lds, (int)blockIdx.x);
+}
+
+template <int D, int NW, bool CAUSAL>
+__global__ void __launch_bounds__(NW * 64) bwd_dkv_kernel(const FlashBwdParams p)
+{
+    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<D>()];
+    bwd_dkv_body<D, NW, CAUSAL>(p, lds, (int)blockIdx.x);
+}
+
+}  // namespace arhip

@@ -493,6 +493,65 @@ std::optional<Tensor> fused_attention_ex(const Tensor &q, const Tensor &k, const
     return out;
 }
 
+// ---- training --------------------------------------------------------------------------
+
+// `train_shape` (flash_attention.rs:760-787): 4-D, same n and d for q/k/v, hk divides h
+static bool train_shape(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *mask)
+{
+    const auto &qs = q.shape(), &ks = k.shape(), &vs = v.shape();
+    if (qs.size() != 4 || ks.size() != 4 || vs.size() != 4) return false;
+    if (ks != vs || ks[0] != qs[0] || ks[2] != qs[2] || ks[3] != qs[3]) return false;
+    if (ks[1] <= 0 || qs[1] % ks[1] != 0) return false;
+    if (qs[2] <= 0 || (qs[3] != 64 && qs[3] != 128)) return false;   // cuda_flash_train.rs:312-314 (d == 64 there)
+    if (q.dtype() != DType::Float32 || k.dtype() != DType::Float32 || v.dtype() != DType::Float32) return false;
+    if (mask && (mask->dtype() != DType::Float32 || mask->shape() != std::vector<int64_t>{qs[2], qs[2]})) return false;
+    return qs[0] * qs[1] <= 65535;
+}
+
+std::optional<TrainOut> fused_attention_train(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
+                                              bool is_causal, Session &sess)
+{
+    if (!train_shape(q, k, v, attn_mask)) return std::nullopt;
+    const int64_t b = q.shape()[0], h = q.shape()[1], n = q.shape()[2], d = q.shape()[3], hk = k.shape()[1];
+    const auto dev = q.device();
+    const DType F = DType::Float32;
+    Tensor out = Tensor::empty(dev, {b, h, n, d}, F), lse = Tensor::empty(dev, {b * h, n}, F);
+    const Tensor mslot = attn_mask ? *attn_mask : out;
+    const HostCall call = make_call(dev, "ar_fl_fwd", {q, k, v, out, lse, mslot}, {F, F, F, F, F, F}, {(n + 127) / 128, b * h, 1},
+                                    {256, 1, 1}, {n, d, (int64_t)is_causal, (int64_t)(attn_mask != nullptr), h, hk});
+    sess.capture_host(call);
+    call.exec();
+    return TrainOut{out, lse};
+}
+
+std::optional<Grads> fused_attention_backward(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor &out,
+                                              const Tensor &lse, const Tensor &dout, const Tensor *attn_mask,
+                                              bool is_causal, Session &sess)
+{
+    if (!train_shape(q, k, v, attn_mask)) return std::nullopt;
+    if (dout.dtype() != DType::Float32 || dout.shape() != q.shape() || out.shape() != q.shape()) return std::nullopt;  // :892-901
+    const int64_t b = q.shape()[0], h = q.shape()[1], n = q.shape()[2], d = q.shape()[3], hk = k.shape()[1];
+    if (lse.dtype() != DType::Float32 || lse.numel() != b * h * n) return std::nullopt;
+    const auto dev = q.device();
+    const DType F = DType::Float32;
+    Tensor delta = Tensor::empty(dev, {b * h, n}, F);
+    Grads g{Tensor::empty(dev, {b, h, n, d}, F), Tensor::empty(dev, {b, hk, n, d}, F), Tensor::empty(dev, {b, hk, n, d}, F)};
+    const Tensor mslot = attn_mask ? *attn_mask : g.dq;   // the reference's dummy (cuda_flash_train.rs:442-449)
+    const std::vector<int64_t> vals = {n, d, (int64_t)is_causal, (int64_t)(attn_mask != nullptr), h, hk};
+    const std::vector<HostCall> calls = {
+        make_call(dev, "ar_fl_prep", {out, dout, delta}, {F, F, F}, {(n + 3) / 4, b * h, 1}, {256, 1, 1}, {n, d}),
+        make_call(dev, "ar_fl_bwd_dq", {q, k, v, dout, lse, delta, mslot, g.dq}, {F, F, F, F, F, F, F, F},
+                  {(n + 127) / 128, b * h, 1}, {256, 1, 1}, vals),
+        make_call(dev, "ar_fl_bwd_dkv", {q, k, v, dout, lse, delta, mslot, g.dk, g.dv}, {F, F, F, F, F, F, F, F, F},
+                  {(n + 127) / 128, b * hk, 1}, {256, 1, 1}, vals),
+    };
+    for (const HostCall &call : calls) {
+        sess.capture_host(call);
+        call.exec();
+    }
+    return g;
+}
+
 // ---- Tensor API -----------------------------------------------------------------------
 
 Tensor Tensor::attention_kind(const Tensor &key, const Tensor &value, const Tensor *mask, double dropout_p, bool is_causal,

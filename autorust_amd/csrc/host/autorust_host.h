@@ -184,4 +184,16 @@ std::optional<Tensor> fused_attention_ex(const Tensor &q, const Tensor &k, const
                                          const Settings &st);                                // :348-702
 uint64_t selections(Kernel k);   // cuda_flash_bf16.rs:458-461
 
+// ---- training: forward with the saved log-sum-exp, and the backward ------------------------
+// `fused_attention_train` / `fused_attention_backward` (src/models/flash_attention.rs:789-977):
+// f32 only, 4-D, mask f32 [n, n] or none; anything else => std::nullopt (the caller keeps its
+// graph path).  train returns (out [b,h,n,d], lse [b*h, n]); backward returns (dq, dk, dv).
+struct TrainOut { Tensor out, lse; };
+struct Grads { Tensor dq, dk, dv; };
+std::optional<TrainOut> fused_attention_train(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
+                                              bool is_causal, Session &sess);
+std::optional<Grads> fused_attention_backward(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor &out,
+                                              const Tensor &lse, const Tensor &dout, const Tensor *attn_mask,
+                                              bool is_causal, Session &sess);
+
 }  // namespace autorust

@@ -180,6 +180,36 @@ void *arh_fused_attention(void *q, void *k, void *v, int kind, void *sess, const
     }, nullptr);
 }
 
+// fused_attention_train / fused_attention_backward (src/models/flash_attention.rs:789-977).
+// Return 1 and fill the outputs, 0 when the kernels decline (the reference's None), -1 on error.
+int arh_fused_attention_train(void *q, void *k, void *v, void *mask, int is_causal, void *sess, void **out, void **lse)
+{
+    g_err.clear();
+    return guard([&]() -> int {
+        auto r = fused_attention_train(*(Tensor *)q, *(Tensor *)k, *(Tensor *)v, (const Tensor *)mask, is_causal != 0,
+                                       ((SessionBox *)sess)->sess);
+        if (!r) return 0;
+        *out = new Tensor(r->out);
+        *lse = new Tensor(r->lse);
+        return 1;
+    }, -1);
+}
+
+int arh_fused_attention_backward(void *q, void *k, void *v, void *out, void *lse, void *dout, void *mask, int is_causal,
+                                 void *sess, void **dq, void **dk, void **dv)
+{
+    g_err.clear();
+    return guard([&]() -> int {
+        auto r = fused_attention_backward(*(Tensor *)q, *(Tensor *)k, *(Tensor *)v, *(Tensor *)out, *(Tensor *)lse,
+                                          *(Tensor *)dout, (const Tensor *)mask, is_causal != 0, ((SessionBox *)sess)->sess);
+        if (!r) return 0;
+        *dq = new Tensor(r->dq);
+        *dk = new Tensor(r->dk);
+        *dv = new Tensor(r->dv);
+        return 1;
+    }, -1);
+}
+
 int arh_plan_fused(const int64_t *q, int qn, const int64_t *k, int kn, const int64_t *v, int vn, int qd, int kd, int vd,
                    const int64_t *mask, int mn, int mask_dtype, int enable_gqa, int quantized, const arh_settings *st,
                    int *sage_declined)

@@ -168,6 +168,17 @@ class Device:
                                                int(wait), ctypes.byref(s)))
         return s.value if wait else None
 
+    def flash_bwd(self, q, k, v, o, lse, dout, dq, dk, dv, delta, B, Hq, Hkv, N, D, mask=None, kv_len=None,
+                  causal=False, scale=None, wait=True):
+        """f32 dense [B,H,N,D]; o and lse from flash_fwd_lse of the same call; delta: B*Hq*N floats of scratch."""
+        scale = float(1.0 / np.sqrt(np.float32(D))) if scale is None else float(scale)
+        s = ctypes.c_double()
+        check(self.lib.arhip_flash_bwd(self.handle, self._ptr(q), self._ptr(k), self._ptr(v), self._ptr(o),
+                                       self._ptr(lse), self._ptr(dout), self._ptr(dq), self._ptr(dk), self._ptr(dv),
+                                       self._ptr(delta), self._ptr(mask), self._ptr(kv_len), B, Hq, Hkv, N, D,
+                                       int(causal), scale, int(wait), ctypes.byref(s)))
+        return s.value if wait else None
+
     def flash_fwd_lse(self, q, k, v, o, lse, B, Hq, Hkv, N, D, dtype, mask=None, kv_len=None, causal=False,
                       scale=None, wait=True):
         """Dense [B,H,N,D] tensors; also writes lse [B,Hq,N] (f32)."""

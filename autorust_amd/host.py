@@ -81,6 +81,9 @@ def host():
                                               i64p, ci]
         h.arh_fused_attention.restype = vp
         h.arh_fused_attention.argtypes = [vp, vp, vp, ci, vp, ctypes.POINTER(Settings)]
+        pvp = ctypes.POINTER(vp)
+        h.arh_fused_attention_train.argtypes = [vp, vp, vp, vp, ci, vp, pvp, pvp]
+        h.arh_fused_attention_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, vp, pvp, pvp, pvp]
         h.arh_attention.restype = vp
         h.arh_attention.argtypes = [vp, vp, vp, vp, ctypes.c_double, ci, ci, vp, ctypes.POINTER(Settings)]
         h.arh_plan_fused.argtypes = [i64p, ci, i64p, ci, i64p, ci, ci, ci, ci, i64p, ci, ci, ci, ci,
@@ -225,6 +228,32 @@ def fused_attention(q, k, v, sess, kind=None, settings=None):
             raise HostError(msg.decode("utf-8", "replace"))
         return None
     return Tensor(h)
+
+
+def _declined_or_raise(rc):
+    if rc < 0:
+        raise HostError(host().arh_last_error().decode("utf-8", "replace"))
+    return rc == 0
+
+
+def fused_attention_train(q, k, v, sess, mask=None, is_causal=False):
+    """`fused_attention_train` (src/models/flash_attention.rs:789-870): (out, lse) or None."""
+    out, lse = ctypes.c_void_p(), ctypes.c_void_p()
+    rc = host().arh_fused_attention_train(q.h, k.h, v.h, mask.h if mask is not None else None, int(is_causal), sess.h,
+                                          ctypes.byref(out), ctypes.byref(lse))
+    if _declined_or_raise(rc):
+        return None
+    return Tensor(out.value), Tensor(lse.value)
+
+
+def fused_attention_backward(q, k, v, out, lse, dout, sess, mask=None, is_causal=False):
+    """`fused_attention_backward` (src/models/flash_attention.rs:872-977): (dq, dk, dv) or None."""
+    dq, dk, dv = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    rc = host().arh_fused_attention_backward(q.h, k.h, v.h, out.h, lse.h, dout.h, mask.h if mask is not None else None,
+                                             int(is_causal), sess.h, ctypes.byref(dq), ctypes.byref(dk), ctypes.byref(dv))
+    if _declined_or_raise(rc):
+        return None
+    return Tensor(dq.value), Tensor(dk.value), Tensor(dv.value)
 
 
 def plan_fused(q, k, v, qd=FLOAT32, kd=None, vd=None, mask=None, mask_dtype=FLOAT32, enable_gqa=False, quantized=False,

@@ -51,7 +51,7 @@ enum { ARHIP_F32 = 0, ARHIP_BF16 = 1 };
 enum { ARHIP_ATTN_SDPA = 0, ARHIP_ATTN_FLASH = 1, ARHIP_ATTN_SAGE = 2 };
 
 /* kernels counted by arhip_selections() */
-enum { ARHIP_K_FLASH_F32 = 0, ARHIP_K_FLASH_BF16 = 1, ARHIP_K_SAGE = 2, ARHIP_K_SAGE_QUANT = 3, ARHIP_K_COUNT = 4 };
+enum { ARHIP_K_FLASH_F32 = 0, ARHIP_K_FLASH_BF16 = 1, ARHIP_K_SAGE = 2, ARHIP_K_SAGE_QUANT = 3, ARHIP_K_FLASH_BWD = 4, ARHIP_K_COUNT = 5 };
 
 const char *arhip_last_error(void);
 
@@ -161,6 +161,20 @@ int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void *k, const v
                         const float *mask, const int32_t *kv_len,
                         int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
                         int causal, int dtype, float scale, int wait, double *secs);
+
+/* arhip_flash_bwd: `fused_attention_backward` (src/models/flash_attention.rs:789-977) = the three
+ *   training kernels of src/runtime/cuda_flash_train.rs:145-309 in one call: ar_fl_prep
+ *   (delta[b,h,i] = O_i . dO_i), ar_fl_bwd_dq and ar_fl_bwd_dkv.  f32 only, dense [B,H,N,D] tensors
+ *   (the reference: "f32 only; other dtypes keep the graph path"); o and lse are what
+ *   arhip_flash_fwd_lse(dtype = ARHIP_F32) produced for the same q, k, v, mask, kv_len, causal and
+ *   scale.  dq [B,Hq,N,D], dk and dv [B,Hkv,N,D] are written in full (no zero-fill needed: the
+ *   sum over a GQA group happens inside the kernel, in a fixed order, without atomics).  delta is a
+ *   caller-provided scratch of B*Hq*N floats.  D is 64 or 128 (the reference: 64). */
+int arhip_flash_bwd(arhip_device *dev, const float *q, const float *k, const float *v, const float *o,
+                    const float *lse, const float *dout, float *dq, float *dk, float *dv, float *delta,
+                    const float *mask, const int32_t *kv_len,
+                    int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                    int causal, float scale, int wait, double *secs);
 
 /* arhip_sage_quant: the quantiser of the Sage kernel hoisted into a pre-pass
  *   (the reference quantises inside the attention kernel, K once per query

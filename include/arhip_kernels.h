@@ -29,6 +29,19 @@
  * (const float *Q, *K, *V, float *O, const float *M, 6 ints); general tiling. */
 #define ARHIP_KERNEL_FLASH_F32 "ar_flash_f32"
 
+/* Training kernels, f32: replace `ar_fl_fwd`, `ar_fl_prep`, `ar_fl_bwd_dq`, `ar_fl_bwd_dkv`,
+ * src/runtime/cuda_flash_train.rs:57-309, with the reference's argument order and head_dim
+ * inserted after N; block [256,1,1].
+ *   ar_fl_fwd     (Q, K, V, float *O, float *LSE, M, 6 ints)           grid [ceil(N/128), B*hq, 1]
+ *   ar_fl_prep    (O, dO, float *D, int N, int head_dim)               grid [ceil(N/4), B*hq, 1]
+ *   ar_fl_bwd_dq  (Q, K, V, dO, LSE, D, M, float *dQ, 6 ints)          grid [ceil(N/128), B*hq, 1]
+ *   ar_fl_bwd_dkv (Q, K, V, dO, LSE, D, M, float *dK, float *dV, 6 ints)  grid [ceil(N/128), B*hkv, 1]
+ * LSE and D are [B, hq, N]; dK and dV are summed over the GQA group inside the kernel. */
+#define ARHIP_KERNEL_FL_FWD "ar_fl_fwd"
+#define ARHIP_KERNEL_FL_PREP "ar_fl_prep"
+#define ARHIP_KERNEL_FL_BWD_DQ "ar_fl_bwd_dq"
+#define ARHIP_KERNEL_FL_BWD_DKV "ar_fl_bwd_dkv"
+
 /* bf16: replaces `ar_flash_bf16`, src/runtime/cuda_flash_bf16.rs:226-427.
  * (const bf16 *Q, *K, *V, bf16 *O, const float *M, 6 ints); general tiling, any mask. */
 #define ARHIP_KERNEL_FLASH_BF16 "ar_flash_bf16"

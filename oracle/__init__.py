@@ -145,6 +145,49 @@ def lse_f64(q, k, mask=None, causal=False, kv_len=None, rows=None, scale=None):
     return out
 
 
+def attention_backward_f64(q, k, v, dout, mask=None, causal=False, kv_len=None, scale=None):
+    """Training forward + backward in binary64, by the reference's formulas
+    (src/runtime/cuda_flash_train.rs:145-309): lse = log sum exp(s), o = softmax(s) v,
+    D_i = o_i . dO_i, p = exp(s - lse), dp = dO v^T, ds = p (dp - D) scale, dQ = ds K,
+    dK = sum over the GQA group of ds^T Q, dV = sum over the group of p^T dO; masked keys
+    (causal: j > i, key length: j >= kv_len[b]) have p = 0.  Returns (o, lse, dq, dk, dv) as
+    float32 arrays.  Pinned against torch.autograd in tests/test_oracle.py."""
+    q, k, v, dout = (np.asarray(t, np.float64) for t in (q, k, v, dout))
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    group = Hq // Hkv
+    scale = 1.0 / np.sqrt(D) if scale is None else float(scale)
+    o = np.zeros((B, Hq, N, D)); lse = np.full((B, Hq, N), -1e30)
+    dq = np.zeros((B, Hq, N, D)); dk = np.zeros((B, Hkv, N, D)); dv = np.zeros((B, Hkv, N, D))
+    i, j = np.arange(N)[:, None], np.arange(N)[None, :]
+    for b in range(B):
+        dead = np.zeros((N, N), bool)
+        if causal:
+            dead |= j > i
+        if kv_len is not None:
+            dead |= j >= int(kv_len[b])
+        for h in range(Hq):
+            kh = h // group
+            s = (q[b, h] @ k[b, kh].T) * scale
+            if mask is not None:
+                s = s + np.broadcast_to(np.asarray(mask, np.float64), (B, Hq, N, N))[b, h]
+            s = np.where(dead, -np.inf, s)
+            m = s.max(axis=1, keepdims=True)
+            live = np.isfinite(m[:, 0])
+            e = np.where(live[:, None], np.exp(s - np.where(live[:, None], m, 0.0)), 0.0)
+            l = e.sum(axis=1, keepdims=True)
+            pr = np.where(live[:, None], e / np.where(l > 0, l, 1.0), 0.0)
+            lse[b, h] = np.where(live, (m + np.log(np.where(l > 0, l, 1.0)))[:, 0], -1e30)
+            o[b, h] = pr @ v[b, kh]
+            delta = (o[b, h] * dout[b, h]).sum(axis=1, keepdims=True)
+            dp = dout[b, h] @ v[b, kh].T
+            ds = pr * (dp - delta) * scale
+            dq[b, h] = ds @ k[b, kh]
+            dk[b, kh] += ds.T @ q[b, h]
+            dv[b, kh] += pr.T @ dout[b, h]
+    return tuple(t.astype(np.float32) for t in (o, lse, dq, dk, dv))
+
+
 def flash_f32(q, k, v, mask=None, causal=False, kv_len=None, rows=None, scale=None, bq=64, bk=32):
     """fp32 exact-mode FA2 kernel restated (src/runtime/cuda_flash.rs:53-141)."""
     scale = np.float32(1.0) / np.sqrt(np.float32(q.shape[-1])) if scale is None else scale

@@ -165,3 +165,32 @@ def test_ar_flash_sage_long_by_name(dev, kernels, causal, out_f32):
     # the int8 error to wash out, so they are left to the comparison with the emulation above
     lo = 256 if causal else 0
     assert np.abs(got - oracle.sdpa_f64(q, k, v, causal=causal))[:, :, lo:].max() <= 2e-2
+
+
+@pytest.mark.parametrize("case", [(2, 4, 2, 37, 64, True, False), (1, 4, 4, 150, 128, False, True)], ids=str)
+def test_training_kernels_by_name(dev, kernels, case):
+    """ar_fl_fwd / ar_fl_prep / ar_fl_bwd_dq / ar_fl_bwd_dkv launched the way the reference's
+    `fused_attention_train` + `fused_attention_backward` launch theirs
+    (src/runtime/cuda_flash_train.rs:336-541), against the float64 oracle at the reference's 2e-3
+    (tests/flash_train_cuda.rs:84-106)."""
+    b, hq, hkv, n, d, causal, has_mask = case
+    q, k, v = fill_qkv(b, hq, hkv, n, d)
+    do = synth.normal(77, q.shape)
+    mask = ref_mask(n).reshape(n, n) if has_mask else None
+    vals = [n, d, int(causal), int(has_mask), hq, hkv]
+    with Bufs(dev) as bufs:
+        dq_, dk_, dv_, ddo = bufs.put(q), bufs.put(k), bufs.put(v), bufs.put(do)
+        o, lse, delta = bufs.new(q.nbytes), bufs.new(b * hq * n * 4), bufs.new(b * hq * n * 4, zero=False)
+        gq, gk, gv = bufs.new(q.nbytes, zero=False), bufs.new(k.nbytes, zero=False), bufs.new(v.nbytes, zero=False)
+        dm = bufs.put(mask) if has_mask else o
+        blk = (256, 1, 1)
+        dev.launch(kernels, "ar_fl_fwd", _grid(n, 128, b, hq), blk, [dq_, dk_, dv_, o, lse, dm], vals)
+        dev.launch(kernels, "ar_fl_prep", ((n + 3) // 4, b * hq, 1), blk, [o, ddo, delta], [n, d])
+        dev.launch(kernels, "ar_fl_bwd_dq", _grid(n, 128, b, hq), blk, [dq_, dk_, dv_, ddo, lse, delta, dm, gq], vals)
+        dev.launch(kernels, "ar_fl_bwd_dkv", _grid(n, 128, b, hkv), blk, [dq_, dk_, dv_, ddo, lse, delta, dm, gk, gv], vals)
+        got = (o.copyout(np.float32, q.shape), lse.copyout(np.float32, (b, hq, n)), gq.copyout(np.float32, q.shape),
+               gk.copyout(np.float32, k.shape), gv.copyout(np.float32, v.shape))
+    want = oracle.attention_backward_f64(q, k, v, do, mask=mask, causal=causal)
+    for name, g, w in zip(("o", "lse", "dq", "dk", "dv"), got, want):
+        assert np.abs(g - w).max() < 2e-3, name
+        assert np.abs(g - w).max() <= 3e-5 * max(1.0, np.abs(w).max()), name

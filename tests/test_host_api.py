@@ -194,6 +194,32 @@ def test_fused_attention_wrappers(hdev):
 
 
 @gpu
+def test_fused_attention_train_and_backward(hdev):
+    """The reference's own differential test of the training path (tests/flash_train_cuda.rs:40-106):
+    fused forward (out, lse) then fused backward (dq, dk, dv) within 2e-3 of the gradients of SDPA
+    under loss = sum(out * dO), through the host API and a captured replay."""
+    def data(n, seed):
+        return (np.sin(np.arange(n, dtype=np.float32) * np.float32(0.0137) + np.float32(seed)) * np.float32(0.6)).astype(np.float32)
+    b, h, hk, n, d, causal = 2, 4, 2, 37, 64, True
+    q, k, v, do = (data(b * hh * n * d, s).reshape(b, hh, n, d) for hh, s in ((h, 0.0), (hk, 1.3), (hk, 2.7), (h, 4.1)))
+    tq, tk, tv, tdo = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v, do))
+    sess = Session()
+    sess.begin_capture()
+    out, lse = host.fused_attention_train(tq, tk, tv, sess, is_causal=causal)
+    dq, dk, dv = host.fused_attention_backward(tq, tk, tv, out, lse, tdo, sess, is_causal=causal)
+    assert sess.end_capture() == 4
+    assert [sess.step(i)[0] for i in range(4)] == ["ar_fl_fwd", "ar_fl_prep", "ar_fl_bwd_dq", "ar_fl_bwd_dkv"]
+    want = oracle.attention_backward_f64(q, k, v, do, causal=causal, scale=0.125)
+    for name, got, w in zip(("out", "lse", "dq", "dk", "dv"), (out, lse, dq, dk, dv), want):
+        assert float(np.abs(got.to_list().reshape(w.shape) - w).max()) < 2e-3, name
+    sess.replay()                                         # same buffers, same results
+    assert float(np.abs(dq.to_list() - want[2]).max()) < 2e-3
+    # bf16 tensors keep the graph path: None (flash_attention.rs:802-807)
+    tb = Tensor.from_slice(hdev, q, q.shape, BFLOAT16)
+    assert host.fused_attention_train(tb, tb, tb, sess) is None
+
+
+@gpu
 def test_attention_debug_line_and_kernel_info(hdev, capfd, monkeypatch):
     """AUTORUST_ATTN_DEBUG prints one line per kernel on its first dispatch
     (src/runtime/cuda_flash_bf16.rs:446-456)."""

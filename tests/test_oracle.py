@@ -358,3 +358,71 @@ def test_log_sum_exp_against_scipy():
     want = sp.logsumexp(s, axis=-1)
     got = oracle.lse_f64(q, k, causal=True, kv_len=np.array([30], np.int32))
     assert np.abs(got - want).max() < 1e-5
+
+
+def _train_data(n, seed):
+    """The generator of the reference's training test (tests/flash_train_cuda.rs:18-22)."""
+    return (np.sin(np.arange(n, dtype=np.float32) * np.float32(0.0137) + np.float32(seed)) * np.float32(0.6)).astype(np.float32)
+
+
+TRAIN_CASES = [  # tests/flash_train_cuda.rs:108-123: b, h, hk, n, causal, with_mask
+    (2, 4, 4, 37, False, False), (1, 2, 2, 197, False, False), (2, 4, 4, 37, True, False),
+    (2, 4, 4, 37, False, True), (2, 4, 2, 37, False, False), (2, 4, 2, 37, True, False), (2, 4, 1, 37, False, True),
+]
+
+
+@pytest.mark.parametrize("case", TRAIN_CASES, ids=str)
+def test_backward_reference_against_torch_autograd(case):
+    """The reference checks its fused backward against the autograd of its graph SDPA
+    (tests/flash_train_cuda.rs:62-70: loss = sum(out * dO)); torch's autograd in float64 is the
+    library stand-in for that here."""
+    import torch
+    b, h, hk, n, causal, with_mask = case
+    d = 64
+    q = _train_data(b * h * n * d, 0.0).reshape(b, h, n, d)
+    k = _train_data(b * hk * n * d, 1.3).reshape(b, hk, n, d)
+    v = _train_data(b * hk * n * d, 2.7).reshape(b, hk, n, d)
+    do = _train_data(b * h * n * d, 4.1).reshape(b, h, n, d)
+    mask = _train_data(n * n, 5.3).reshape(n, n) if with_mask else None
+    o, lse, dq, dk, dv = oracle.attention_backward_f64(q, k, v, do, mask=mask, causal=causal, scale=0.125)
+
+    tq, tk, tv = (torch.tensor(t, dtype=torch.float64, requires_grad=True) for t in (q, k, v))
+    g = h // hk
+    s = (tq @ tk.repeat_interleave(g, dim=1).transpose(-1, -2)) * 0.125
+    if with_mask:
+        s = s + torch.tensor(mask, dtype=torch.float64)
+    if causal:
+        s = s.masked_fill(torch.ones(n, n, dtype=torch.bool).triu(1), float("-inf"))
+    out = torch.softmax(s, dim=-1) @ tv.repeat_interleave(g, dim=1)
+    (out * torch.tensor(do, dtype=torch.float64)).sum().backward()
+    assert np.abs(o - out.detach().numpy()).max() < 1e-6
+    assert np.abs(lse - torch.logsumexp(s, dim=-1).detach().numpy()).max() < 1e-5
+    for got, want in ((dq, tq.grad), (dk, tk.grad), (dv, tv.grad)):
+        want = want.numpy()
+        assert np.abs(got - want).max() <= 1e-6 * max(1.0, np.abs(want).max())
+
+
+def test_backward_reference_closed_forms():
+    """What the mathematics fixes: with one visible key p = 1, so dQ = 0, dK = 0 and dV_0 = sum of
+    the dO rows; a key-length mask equals the truncated problem; gradients are linear in dO."""
+    q, k, v, do = (synth.normal(s, (1, 2, 9, 64)) for s in (41, 42, 43, 44))
+    o, lse, dq, dk, dv = oracle.attention_backward_f64(q, k, v, do, kv_len=np.array([1]))
+    assert np.abs(dq).max() == 0 and np.abs(dk).max() == 0
+    assert np.abs(dv[:, :, 0] - do.sum(axis=2)).max() < 1e-5 and np.abs(dv[:, :, 1:]).max() == 0
+    full = oracle.attention_backward_f64(q, k, v, do, kv_len=np.array([5]), causal=True)
+    # truncated problem, evaluated directly: rows i see keys j <= min(i, 4)
+    qq, kk, vv, dd = (np.asarray(t, np.float64) for t in (q, k, v, do))
+    for h in range(2):
+        s = (qq[0, h] @ kk[0, h, :5].T) / 8.0
+        s = np.where(np.arange(5)[None, :] > np.arange(9)[:, None], -np.inf, s)
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        p /= p.sum(axis=1, keepdims=True)
+        oo = p @ vv[0, h, :5]
+        ds = p * (dd[0, h] @ vv[0, h, :5].T - (oo * dd[0, h]).sum(axis=1, keepdims=True)) / 8.0
+        assert np.abs(full[2][0, h] - ds @ kk[0, h, :5]).max() < 1e-5
+        assert np.abs(full[3][0, h, :5] - ds.T @ qq[0, h]).max() < 1e-5 and np.abs(full[3][0, h, 5:]).max() == 0
+        assert np.abs(full[4][0, h, :5] - p.T @ dd[0, h]).max() < 1e-5 and np.abs(full[4][0, h, 5:]).max() == 0
+    a = oracle.attention_backward_f64(q, k, v, do)
+    b2 = oracle.attention_backward_f64(q, k, v, 3.0 * do)
+    for x, y in zip(a[2:], b2[2:]):
+        assert np.abs(3.0 * x - y).max() < 1e-4
