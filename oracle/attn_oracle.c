@@ -20,7 +20,7 @@
  * (src/tensor/mod.rs:2417-2433) and as `gj < N` in the kernels
  * (src/runtime/cuda_flash.rs:104-113).
  *
- * What pins each function (see tests/test_oracle_*.py):
+ * What pins each function (see tests/test_oracle.py):
  *   ar_head_sdpa_f32/f64  the six reference-held vectors of
  *                         tests/attention_golden.rs (tolerance of
  *                         tests/nn_attention.rs:20), torch's CPU SDPA, fp64.
@@ -34,6 +34,12 @@
  *                         order independent; tiny brute force in Python ints.
  *   ar_logits_i32         exact integer arithmetic; known answer of
  *                         tests/sage_layout_probe.rs:73-84.
+ *   ar_head_sage          re-derived with torch tensor operations (integer matmul,
+ *                         (sq*sk)*scale, additive mask, causal, key lengths,
+ *                         bf16(p) @ bf16(v) / sum p) over causal x mask x kv_len x
+ *                         GQA at block sizes (1,1), (128,64), (32,16); closed forms;
+ *                         single-line mutations of the masks and rounding points
+ *                         each fail a test (tests/test_oracle.py).
  *   ar_k_mean             PARITY UNPINNED by the reference (it has no
  *                         K smoothing, src/runtime/cuda_flash_sage.rs:13-14).
  *                         Pinned by: softmax shift invariance, fp64 mean within
