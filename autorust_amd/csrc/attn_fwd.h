@@ -55,6 +55,7 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 
 constexpr int MODE_BF16 = 0;  // q, k bf16
 constexpr int MODE_I8 = 1;    // q, k int8 with block scales
+constexpr int MODE_FP8 = 2;   // q, k FP8 E4M3 (OCP) with block scales: the reference's AR_FP8 branch, cuda_flash_sage.rs:92-147
 constexpr int BK = 64;        // keys per tile
 constexpr float NEG_SENTINEL = -1e30f;  // src/runtime/cuda_flash_bf16.rs:106 (AR_NEG)
 constexpr float LOG2E = 1.4426950408889634f;
@@ -138,7 +139,7 @@ __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70)
 template <int D, int NW, int MODE, bool PER_KEY, bool SMALL = false>
 constexpr int attn_fwd_lds_bytes()
 {
-    constexpr int QKB = (MODE == MODE_I8) ? 1 : 2;
+    constexpr int QKB = (MODE != MODE_BF16) ? 1 : 2;
     return (SMALL ? 4 : 2) * (BK * (D * QKB + 16) + BK * (D * 2 + 64) + (PER_KEY ? BK * 4 : 0));
 }
 
@@ -154,7 +155,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     constexpr int NSLOT = SMALL ? 4 : 1;  // register sets for tiles in flight
     constexpr int T = NW * 64;
     constexpr int BQ = NW * 32;
-    constexpr int QK_BYTES = (MODE == MODE_I8) ? 1 : 2;        // bytes per q/k element
+    constexpr int QK_BYTES = (MODE != MODE_BF16) ? 1 : 2;        // bytes per q/k element
     constexpr int KROW = D * QK_BYTES + 16;                    // padded K row in LDS
     constexpr int K_TILE = BK * KROW;
     constexpr int VROW = D * 2 + 64;                           // V row in LDS: 4 rows fill the 64 banks
@@ -167,11 +168,12 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     constexpr int V_CPR = D * 2 / 16;                          // 16-byte chunks per V row
     constexpr int V_CHUNKS = BK * V_CPR;
     constexpr int V_PER_THREAD = (V_CHUNKS + T - 1) / T;
-    constexpr int KSTEPS = (MODE == MODE_I8) ? D / 32 : D / 16;  // MFMA k steps over D
+    constexpr int KSTEPS = (MODE != MODE_BF16) ? D / 32 : D / 16;  // MFMA k steps over D
     constexpr int DB = D / 32;                                 // 32-channel output blocks
     static_assert(K_CHUNKS % T == 0 || K_CHUNKS < T, "K staging must divide evenly");
     static_assert(V_CHUNKS % T == 0 || V_CHUNKS < T, "V staging must divide evenly");
-    static_assert(!PER_KEY || MODE == MODE_I8, "per-key scales belong to the int8 path");
+    static_assert(!PER_KEY || MODE != MODE_BF16, "per-key scales belong to the 8-bit paths");
+    static_assert(!DBG || MODE == MODE_I8, "the logits export is int32");
 
     static_assert(NSTAGE * STAGE == attn_fwd_lds_bytes<D, NW, MODE, PER_KEY, SMALL>(), "LDS size bookkeeping");
 
@@ -240,7 +242,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     uint4 kst[NSLOT][K_PER_THREAD];
     uint4 vst[NSLOT][V_PER_THREAD];
     float sst = 0.f;
-    const int nkb = (MODE == MODE_I8) ? (N + p.bk - 1) / p.bk : 0;
+    const int nkb = (MODE != MODE_BF16) ? (N + p.bk - 1) / p.bk : 0;
 
     auto load_tile = [&](int k0, int slot = 0) __attribute__((always_inline)) {
         const bool full = k0 + BK <= kend;  // uniform: the common case has no bounds logic
@@ -309,7 +311,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     float m_run = NEG_SENTINEL;  // running max in the exp2 domain (x * log2e)
     float l_run = 0.f;           // this lane half's part of the running sum
     float sq_lane = 1.f;
-    if (MODE == MODE_I8) {
+    if (MODE != MODE_BF16) {
         const int nqb = (N + p.bq - 1) / p.bq;
         sq_lane = p.sq[(size_t)bh * nqb + min(q_row, N - 1) / p.bq];
     }
@@ -349,10 +351,18 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
         for (int r = 0; r < 16; ++r) s[r] = 0;
 #pragma unroll
         for (int st = 0; st < KSTEPS; ++st) {
-            if constexpr (MODE == MODE_I8)
+            if constexpr (MODE == MODE_I8) {
                 s = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kf[st]), __builtin_bit_cast(i32x4, qreg[st]), s, 0, 0, 0);
-            else
+            } else if constexpr (MODE == MODE_FP8) {
+                // same 16-byte fragments as int8; the FP8 instruction contracts 8 bytes per lane, so a
+                // fragment is two steps (low halves, then high halves: any order Q and K agree on)
+                s = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8((long)(kf[st].x | ((uint64_t)kf[st].y << 32)),
+                                                               (long)(qreg[st].x | ((uint64_t)qreg[st].y << 32)), s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8((long)(kf[st].z | ((uint64_t)kf[st].w << 32)),
+                                                               (long)(qreg[st].z | ((uint64_t)qreg[st].w << 32)), s, 0, 0, 0);
+            } else {
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s, 0, 0, 0);
+            }
         }
         return s;
     };
@@ -375,7 +385,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
         const unsigned char *kl = lds + (it % NSTAGE) * STAGE;
         const unsigned char *vl = kl + K_TILE;
         float f_tile = 1.f;
-        if (MODE == MODE_I8 && !PER_KEY) f_tile = p.sk[(size_t)kv_bh * nkb + (it >> p.bk_tile_shift)];
+        if (MODE != MODE_BF16 && !PER_KEY) f_tile = p.sk[(size_t)kv_bh * nkb + (it >> p.bk_tile_shift)];
         // online softmax of one 32-key block: raw accumulators in, probabilities (bf16, B-operand
         // layout) out; updates the running reference / sum and, rarely, rescales the accumulators
         auto softmax_block = [&](int blk, const acc_t &s, uint4 (&pb)[2]) __attribute__((always_inline)) {
@@ -413,7 +423,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
                 // src/runtime/cuda_flash_sage.rs:315-322.  The row sum bounds the largest probability
                 // (max <= sum <= 16 max), so only a sum that is too large (or not finite: the very first
                 // block, or a jump of the maximum) sends the wave to the exact path below.
-                const float c = (MODE == MODE_I8) ? ((sq_lane * f_tile) * p.scale) * LOG2E : c_scale;
+                const float c = (MODE != MODE_BF16) ? ((sq_lane * f_tile) * p.scale) * LOG2E : c_scale;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[r], c, -m_run));
                 rs = row_sum();
@@ -434,7 +444,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
                     const int kt = blk * 32 + 8 * (r >> 2) + 4 * h + (r & 3);  // key within the tile
                     const int key = k0 + kt;
                     float cc = c_scale;
-                    if (MODE == MODE_I8) {
+                    if (MODE != MODE_BF16) {
                         const float skv = PER_KEY ? *(const float *)(vl + V_TILE + kt * 4) : f_tile;
                         cc = ((sq_lane * skv) * p.scale) * LOG2E;
                     }

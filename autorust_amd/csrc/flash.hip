@@ -244,14 +244,13 @@ extern "C" int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t 
                                   out_dtype, scale, dbg_logits, dbg_sel, wait, secs);
 }
 
-extern "C" int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const int8_t *k8,
-                                      const float *sq, const float *sk, const uint16_t *v, void *o,
-                                      const int64_t v_strides[3], const int64_t o_strides[3],
-                                      const float *mask, const int32_t *kv_len,
-                                      int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
-                                      int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
-                                      int32_t *dbg_logits, const int32_t dbg_sel[3],
-                                      int wait, double *secs)
+static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
+                         const float *sq, const float *sk, const uint16_t *v, void *o,
+                         const int64_t v_strides[3], const int64_t o_strides[3],
+                         const float *mask, const int32_t *kv_len,
+                         int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                         int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
+                         int32_t *dbg_logits, const int32_t dbg_sel[3], int wait, double *secs, bool fp8)
 {
     if (int rc = check_common("arhip_sage_fwd", dev, q8, k8, v, o, mask, B, Hq, Hkv, N, D)) return rc;
     ARHIP_REQUIRE(sq && sk, "arhip_sage_fwd: null scale pointer");
@@ -285,6 +284,7 @@ extern "C" int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const
     p.bq = (int)bq; p.bk = (int)bk;
     p.scale = scale;
     const bool dbg = dbg_logits != nullptr;
+    ARHIP_REQUIRE(!(fp8 && dbg), "arhip_sage_fwd_fp8: the logits export is an int8 facility");
     const bool c = causal != 0, hm = mask != nullptr, f32o = out_dtype == ARHIP_F32;
     // K scales that are uniform over a 64-key tile (bk = 64 * 2^n) take the fast kernel; anything
     // else, including the reference's per-key scales (bk == 1), stages the tile's scales in LDS
@@ -292,7 +292,7 @@ extern "C" int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const
     while (((int64_t)64 << shift) < bk) ++shift;
     const bool per_key = ((int64_t)64 << shift) != bk;
     p.bk_tile_shift = shift;
-    int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg);
+    int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg || fp8);   // FP8 runs on the general kernel
     if (nw == 1) nw = 4;
     if (nw == 8 && !pipe_addressable(N, std::max<int64_t>(D, v_strides ? v_strides[2] : D), 2)) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
@@ -323,12 +323,44 @@ extern "C" int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const
         else if (f32o) launch_pipe<DD, MODE_I8, true>(dev->stream, p, c);                              \
         else launch_pipe<DD, MODE_I8, false>(dev->stream, p, c);                                       \
     } while (0)
-    if (D == 64) SAGE_D(64);
+#define SAGE_F(DD, PK)                                                                                 \
+    do {                                                                                               \
+        if (f32o) launch_attn<DD, 4, MODE_FP8, PK, true, false, true>(dev->stream, p, c, hm);          \
+        else launch_attn<DD, 4, MODE_FP8, PK, false, false, true>(dev->stream, p, c, hm);              \
+    } while (0)
+    if (fp8) {
+        if (D == 64) { if (per_key) SAGE_F(64, true); else SAGE_F(64, false); }
+        else { if (per_key) SAGE_F(128, true); else SAGE_F(128, false); }
+    } else if (D == 64) SAGE_D(64);
     else SAGE_D(128);
+#undef SAGE_F
 #undef SAGE_D
 #undef SAGE_V
     arhip_note_selected(ARHIP_K_SAGE);
     return t.end();
+}
+
+extern "C" int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const int8_t *k8,
+                                      const float *sq, const float *sk, const uint16_t *v, void *o,
+                                      const int64_t v_strides[3], const int64_t o_strides[3],
+                                      const float *mask, const int32_t *kv_len,
+                                      int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                                      int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
+                                      int32_t *dbg_logits, const int32_t dbg_sel[3], int wait, double *secs)
+{
+    return sage_fwd_impl(dev, q8, k8, sq, sk, v, o, v_strides, o_strides, mask, kv_len, B, Hq, Hkv, N, D, bq, bk, causal,
+                         out_dtype, scale, dbg_logits, dbg_sel, wait, secs, false);
+}
+
+extern "C" int arhip_sage_fwd_fp8(arhip_device *dev, const uint8_t *q8, const uint8_t *k8,
+                                  const float *sq, const float *sk, const uint16_t *v, void *o,
+                                  const float *mask, const int32_t *kv_len,
+                                  int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                                  int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
+                                  int wait, double *secs)
+{
+    return sage_fwd_impl(dev, (const int8_t *)q8, (const int8_t *)k8, sq, sk, v, o, nullptr, nullptr, mask, kv_len, B, Hq, Hkv,
+                         N, D, bq, bk, causal, out_dtype, scale, nullptr, nullptr, wait, secs, true);
 }
 
 extern "C" int arhip_flash_bwd(arhip_device *dev, const float *q, const float *k, const float *v, const float *o,

@@ -39,9 +39,24 @@ int arhip_static_scratch_setup(int ordinal)
     return ARHIP_OK;
 }
 
+// block == 1: one scale per row (scales [B,H,N]); otherwise one workgroup per (block, head)
+template <typename T, bool SMOOTH, bool FP8>
+static void launch_quant(arhip_device *dev, const void *x, int8_t *x8, float *scales, const float *mean, int64_t N, int64_t D,
+                         int64_t block, int nblk, long rows, int64_t heads, const XLayout &lay)
+{
+    if (block == 1) {
+        const int rpb = 256 / (int)(D / 8);
+        hipLaunchKernelGGL((quant_rows_kernel<T, SMOOTH, FP8>), dim3((unsigned)((rows + rpb - 1) / rpb)), dim3(256), 0,
+                           dev->stream, (const T *)x, x8, scales, mean, (int)N, (int)D, rows, lay);
+    } else {
+        hipLaunchKernelGGL((quant_blocks_kernel<T, SMOOTH, FP8>), dim3((unsigned)nblk, (unsigned)heads), dim3(256), 0,
+                           dev->stream, (const T *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk, lay);
+    }
+}
+
 static int sage_quant_impl(arhip_device *dev, const void *x, const int64_t x_strides[3], int8_t *x8, float *scales, float *mean,
                            void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
-                           int64_t block, int dtype, int smooth, int wait, double *secs, int prof_kernel)
+                           int64_t block, int dtype, int smooth, int wait, double *secs, int prof_kernel, bool fp8 = false)
 {
     ARHIP_REQUIRE(dev != nullptr, "arhip_sage_quant: null device");
     ARHIP_REQUIRE(x && x8 && scales, "arhip_sage_quant: null pointer");
@@ -64,7 +79,6 @@ static int sage_quant_impl(arhip_device *dev, const void *x, const int64_t x_str
     ARHIP_HIP(hipSetDevice(dev->ordinal));
     const int nblk = (int)((N + block - 1) / block);
     const int nchunk = (int)((N + MEAN_CHUNK - 1) / MEAN_CHUNK);
-    const dim3 qgrid((unsigned)nblk, (unsigned)(B * H));
     arhip_call_timer t{dev, wait, secs};
     t.kernel = prof_kernel;
     if (int rc = t.begin()) return rc;
@@ -80,39 +94,17 @@ static int sage_quant_impl(arhip_device *dev, const void *x, const int64_t x_str
         hipLaunchKernelGGL(k_mean_final_kernel, dim3((unsigned)(B * H)), dim3((unsigned)D), 0, dev->stream,
                            (const float *)workspace, mean, (int)N, (int)D, nchunk);
     }
-    if (block == 1) {  // scales [B,H,N]: one per row
-        const long rows = (long)(B * H * N);
-        const int rpb = 256 / (int)(D / 8);
-        const dim3 rgrid((unsigned)((rows + rpb - 1) / rpb));
-        if (smooth) {
-            if (dtype == ARHIP_F32)
-                hipLaunchKernelGGL((quant_rows_kernel<float, true>), rgrid, dim3(256), 0, dev->stream,
-                                   (const float *)x, x8, scales, mean, (int)N, (int)D, rows, lay);
-            else
-                hipLaunchKernelGGL((quant_rows_kernel<uint16_t, true>), rgrid, dim3(256), 0, dev->stream,
-                                   (const uint16_t *)x, x8, scales, mean, (int)N, (int)D, rows, lay);
-        } else {
-            if (dtype == ARHIP_F32)
-                hipLaunchKernelGGL((quant_rows_kernel<float, false>), rgrid, dim3(256), 0, dev->stream,
-                                   (const float *)x, x8, scales, nullptr, (int)N, (int)D, rows, lay);
-            else
-                hipLaunchKernelGGL((quant_rows_kernel<uint16_t, false>), rgrid, dim3(256), 0, dev->stream,
-                                   (const uint16_t *)x, x8, scales, nullptr, (int)N, (int)D, rows, lay);
-        }
-    } else if (smooth) {
-        if (dtype == ARHIP_F32)
-            hipLaunchKernelGGL((quant_blocks_kernel<float, true>), qgrid, dim3(256), 0, dev->stream,
-                               (const float *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk, lay);
-        else
-            hipLaunchKernelGGL((quant_blocks_kernel<uint16_t, true>), qgrid, dim3(256), 0, dev->stream,
-                               (const uint16_t *)x, x8, scales, mean, (int)N, (int)D, (int)block, nblk, lay);
+    const long rows = (long)(B * H * N);
+    if (dtype == ARHIP_F32) {
+        if (smooth) fp8 ? launch_quant<float, true, true>(dev, x, x8, scales, mean, N, D, block, nblk, rows, B * H, lay)
+                        : launch_quant<float, true, false>(dev, x, x8, scales, mean, N, D, block, nblk, rows, B * H, lay);
+        else fp8 ? launch_quant<float, false, true>(dev, x, x8, scales, nullptr, N, D, block, nblk, rows, B * H, lay)
+                 : launch_quant<float, false, false>(dev, x, x8, scales, nullptr, N, D, block, nblk, rows, B * H, lay);
     } else {
-        if (dtype == ARHIP_F32)
-            hipLaunchKernelGGL((quant_blocks_kernel<float, false>), qgrid, dim3(256), 0, dev->stream,
-                               (const float *)x, x8, scales, nullptr, (int)N, (int)D, (int)block, nblk, lay);
-        else
-            hipLaunchKernelGGL((quant_blocks_kernel<uint16_t, false>), qgrid, dim3(256), 0, dev->stream,
-                               (const uint16_t *)x, x8, scales, nullptr, (int)N, (int)D, (int)block, nblk, lay);
+        if (smooth) fp8 ? launch_quant<uint16_t, true, true>(dev, x, x8, scales, mean, N, D, block, nblk, rows, B * H, lay)
+                        : launch_quant<uint16_t, true, false>(dev, x, x8, scales, mean, N, D, block, nblk, rows, B * H, lay);
+        else fp8 ? launch_quant<uint16_t, false, true>(dev, x, x8, scales, nullptr, N, D, block, nblk, rows, B * H, lay)
+                 : launch_quant<uint16_t, false, false>(dev, x, x8, scales, nullptr, N, D, block, nblk, rows, B * H, lay);
     }
     arhip_note_selected(ARHIP_K_SAGE_QUANT);
     return t.end();
@@ -133,6 +125,14 @@ extern "C" int arhip_sage_quant_strided(arhip_device *dev, const void *x, const 
     ARHIP_REQUIRE(x_strides != nullptr, "arhip_sage_quant_strided: null strides");
     return sage_quant_impl(dev, x, x_strides, x8, scales, mean, workspace, B, H, N, D, block, dtype, smooth, wait, secs,
                            ARHIP_K_SAGE_QUANT);
+}
+
+extern "C" int arhip_sage_quant_fp8(arhip_device *dev, const void *x, uint8_t *x8, float *scales, float *mean,
+                                    void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
+                                    int64_t block, int dtype, int smooth, int wait, double *secs)
+{
+    return sage_quant_impl(dev, x, nullptr, (int8_t *)x8, scales, mean, workspace, B, H, N, D, block, dtype, smooth, wait, secs,
+                           ARHIP_K_SAGE_QUANT, true);
 }
 
 extern "C" size_t arhip_sage_quant_static_limit(void) { return STATIC_SCRATCH_FLOATS * sizeof(float); }

@@ -101,10 +101,45 @@ __global__ void k_mean_final_kernel(const float *part, float *mean, int N, int D
     k_mean_final_body(part, mean, N, D, nchunk, blockIdx);
 }
 
+// FP8 E4M3 (OCP "FN" flavour: bias 7, no infinities, largest finite 448) of the reference's AR_FP8
+// branch: `__nv_cvt_float2_to_fp8x2(..., __NV_SATFINITE, __NV_E4M3)`, src/runtime/cuda_flash_sage.rs:125-128,
+// with scale = absmax / 448 (:9).  The hardware conversion rounds to nearest even; the operands
+// are clamped to +-448 first, which is what SATFINITE does to anything larger (values in
+// (448, 464) round down to 448 either way).
+template <bool FP8>
+struct QFormat {
+    static constexpr float QMAX = FP8 ? 448.0f : 127.0f;
+};
+template <bool FP8>
+__device__ __forceinline__ uint2 quantise8(const float (&v)[8], float inv)
+{
+    uint32_t w[2] = {0u, 0u};
+    if constexpr (FP8) {
+        float c[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) c[i] = fminf(fmaxf(v[i] * inv, -448.0f), 448.0f);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            int r = 0;
+            r = __builtin_amdgcn_cvt_pk_fp8_f32(c[4 * j + 0], c[4 * j + 1], r, false);
+            r = __builtin_amdgcn_cvt_pk_fp8_f32(c[4 * j + 2], c[4 * j + 3], r, true);
+            w[j] = (uint32_t)r;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int iv = (int)rintf(v[i] * inv);
+            iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
+            w[i >> 2] |= ((uint32_t)iv & 0xffu) << ((i & 3) * 8);
+        }
+    }
+    return make_uint2(w[0], w[1]);
+}
+
 // One workgroup per (block of `blk` tokens, head).  Blocks of up to 256*64 elements are kept
 // in registers between the absmax pass and the quantising pass (one trip to memory); larger
 // ones are read twice.
-template <typename T, bool SMOOTH>
+template <typename T, bool SMOOTH, bool FP8 = false>
 __device__ __forceinline__ void quant_blocks_body(const T *x, int8_t *x8, float *scales, const float *mean,
                                                   int N, int D, int blk, int nblk, const XLayout lay, const dim3 bid)
 {
@@ -156,20 +191,11 @@ __device__ __forceinline__ void quant_blocks_body(const T *x, int8_t *x8, float 
     __syncthreads();
     mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 
-    const float scale = (mx > 0.f) ? mx / 127.0f : 1.f;
+    const float scale = (mx > 0.f) ? mx / QFormat<FP8>::QMAX : 1.f;
     const float inv = 1.f / scale;
     if (tid == 0) scales[(size_t)bh * nblk + bi] = scale;
 
-    auto quant8 = [&](const float (&v)[8]) {
-        uint32_t w[2] = {0u, 0u};
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            int iv = (int)rintf(v[i] * inv);
-            iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
-            w[i >> 2] |= ((uint32_t)iv & 0xffu) << ((i & 3) * 8);
-        }
-        return make_uint2(w[0], w[1]);
-    };
+    auto quant8 = [&](const float (&v)[8]) { return quantise8<FP8>(v, inv); };
     if (keep) {
 #pragma unroll
         for (int it = 0; it < KEEP; ++it) {
@@ -190,17 +216,17 @@ __device__ __forceinline__ void quant_blocks_body(const T *x, int8_t *x8, float 
     }
 }
 
-template <typename T, bool SMOOTH>
+template <typename T, bool SMOOTH, bool FP8 = false>
 __global__ void __launch_bounds__(256) quant_blocks_kernel(const T *x, int8_t *x8, float *scales, const float *mean,
                                                            int N, int D, int blk, int nblk, const XLayout lay)
 {
-    quant_blocks_body<T, SMOOTH>(x, x8, scales, mean, N, D, blk, nblk, lay, blockIdx);
+    quant_blocks_body<T, SMOOTH, FP8>(x, x8, scales, mean, N, D, blk, nblk, lay, blockIdx);
 }
 
 // The reference's own granularity, one scale per token row (block == 1): D/8 lanes share a row,
 // so a workgroup of 256 threads quantises 256/(D/8) rows and the absmax is a shuffle reduction
 // inside the lane group.  Same arithmetic, same order of operations per element.
-template <typename T, bool SMOOTH>
+template <typename T, bool SMOOTH, bool FP8 = false>
 __device__ __forceinline__ void quant_rows_body(const T *x, int8_t *x8, float *scales, const float *mean,
                                                 int N, int D, long rows_total, const XLayout lay, const dim3 bid)
 {
@@ -221,26 +247,19 @@ __device__ __forceinline__ void quant_rows_body(const T *x, int8_t *x8, float *s
 #pragma unroll
     for (int i = 0; i < 8; ++i) mx = fmaxf(mx, fabsf(v[i]));
     for (int off = gpr >> 1; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    const float scale = (mx > 0.f) ? mx / 127.0f : 1.f;
+    const float scale = (mx > 0.f) ? mx / QFormat<FP8>::QMAX : 1.f;
     const float inv = 1.f / scale;
     if (live) {
         if (g == 0) scales[row] = scale;
-        uint32_t w[2] = {0u, 0u};
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            int iv = (int)rintf(v[i] * inv);
-            iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
-            w[i >> 2] |= ((uint32_t)iv & 0xffu) << ((i & 3) * 8);
-        }
-        *(uint2 *)(x8 + (size_t)row * D + g * 8) = make_uint2(w[0], w[1]);
+        *(uint2 *)(x8 + (size_t)row * D + g * 8) = quantise8<FP8>(v, inv);
     }
 }
 
-template <typename T, bool SMOOTH>
+template <typename T, bool SMOOTH, bool FP8 = false>
 __global__ void __launch_bounds__(256) quant_rows_kernel(const T *x, int8_t *x8, float *scales, const float *mean,
                                                          int N, int D, long rows_total, const XLayout lay)
 {
-    quant_rows_body<T, SMOOTH>(x, x8, scales, mean, N, D, rows_total, lay, blockIdx);
+    quant_rows_body<T, SMOOTH, FP8>(x, x8, scales, mean, N, D, rows_total, lay, blockIdx);
 }
 
 __device__ __forceinline__ void cast_bf16_body(const float *x, uint16_t *y, size_t n, const dim3 bid)

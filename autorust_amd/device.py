@@ -210,6 +210,24 @@ class Device:
                                                     int(smooth), int(wait), ctypes.byref(s)))
         return s.value if wait else None
 
+    def sage_quant_fp8(self, x, x8, scales, B, H, N, D, block, dtype, mean=None, workspace=None, smooth=False, wait=True):
+        """sage_quant with FP8 E4M3 codes (scale = absmax / 448) instead of int8 values."""
+        s = ctypes.c_double()
+        check(self.lib.arhip_sage_quant_fp8(self.handle, self._ptr(x), self._ptr(x8), self._ptr(scales), self._ptr(mean),
+                                            self._ptr(workspace), B, H, N, D, block, dtype, int(smooth), int(wait),
+                                            ctypes.byref(s)))
+        return s.value if wait else None
+
+    def sage_fwd_fp8(self, q8, k8, sq, sk, v, o, B, Hq, Hkv, N, D, bq, bk, out_dtype=F32, mask=None, kv_len=None,
+                     causal=False, scale=None, wait=True):
+        scale = float(1.0 / np.sqrt(np.float32(D))) if scale is None else float(scale)
+        s = ctypes.c_double()
+        check(self.lib.arhip_sage_fwd_fp8(self.handle, self._ptr(q8), self._ptr(k8), self._ptr(sq), self._ptr(sk),
+                                          self._ptr(v), self._ptr(o), self._ptr(mask), self._ptr(kv_len),
+                                          B, Hq, Hkv, N, D, bq, bk, int(causal), out_dtype, scale, int(wait),
+                                          ctypes.byref(s)))
+        return s.value if wait else None
+
     def sage_quant_static(self, x, x8, scales, B, H, N, D, block, dtype, mean=None, smooth=False, wait=True):
         """sage_quant with the partial sums in the library's own device array (no allocation)."""
         s = ctypes.c_double()

@@ -215,6 +215,22 @@ int arhip_sage_quant_static(arhip_device *dev, const void *x, int8_t *x8, float 
                             int64_t B, int64_t H, int64_t N, int64_t D,
                             int64_t block, int dtype, int smooth, int wait, double *secs);
 
+/* FP8 E4M3 variant of the quantised path: the reference's AR_FP8 branch
+ *   (src/runtime/cuda_flash_sage.rs:9, 92-147: `mma ... e4m3.e4m3.f32`, scale = max/448,
+ *   `__nv_cvt_float2_to_fp8x2(..., __NV_SATFINITE, __NV_E4M3)`).  Same arguments and semantics as
+ *   arhip_sage_quant / arhip_sage_fwd with x8 holding OCP E4M3 codes instead of int8 values; the
+ *   logits are accumulated in f32 by v_mfma_f32_32x32x16_fp8_fp8, so there is no int32 export.
+ *   Runs on the general kernel (any mask, any block sizes incl. per-row scales). */
+int arhip_sage_quant_fp8(arhip_device *dev, const void *x, uint8_t *x8, float *scales, float *mean,
+                         void *workspace, int64_t B, int64_t H, int64_t N, int64_t D,
+                         int64_t block, int dtype, int smooth, int wait, double *secs);
+int arhip_sage_fwd_fp8(arhip_device *dev, const uint8_t *q8, const uint8_t *k8,
+                       const float *sq, const float *sk, const uint16_t *v, void *o,
+                       const float *mask, const int32_t *kv_len,
+                       int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D,
+                       int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
+                       int wait, double *secs);
+
 /* arhip_cast_bf16: f32 -> bf16 round-to-nearest-even of n elements (the V
  *   operand of the Sage kernel: cuda_flash_sage.rs:99-103, 257-262). */
 int arhip_cast_bf16(arhip_device *dev, const float *x, uint16_t *y, int64_t n, int wait, double *secs);

@@ -233,6 +233,92 @@ def quant_blocks(x, blk, sub=None, use_div=False):
     return q, s
 
 
+def fp8_e4m3_bits(x):
+    """float32 -> FP8 E4M3 codes (OCP "FN": bias 7, subnormal step 2^-9, largest finite 448, no
+    infinities), round to nearest even, saturating: the reference's
+    `__nv_cvt_float2_to_fp8x2(..., __NV_SATFINITE, __NV_E4M3)` (src/runtime/cuda_flash_sage.rs:125-128)."""
+    x = np.asarray(x, np.float32)
+    sign = (np.signbit(x).astype(np.uint8) << 7)
+    a = np.minimum(np.abs(x).astype(np.float64), 448.0)   # SATFINITE; (448, 464) rounds to 448 anyway
+    e = np.floor(np.log2(np.where(a > 0, a, 1.0))).astype(np.int64)
+    e = np.maximum(e, -6)
+    q = np.rint(a / np.exp2(e - 3.0))                      # numpy rint is half-to-even; 0..16
+    up = q >= 16                                           # rounded up into the next binade
+    e = np.where(up, e + 1, e)
+    q = np.where(up, 8.0, q)
+    normal = q >= 8
+    code = np.where(normal, ((e + 7) << 3) | (q.astype(np.int64) - 8), q.astype(np.int64))
+    code = np.where(np.isnan(x), 0x7f, code)
+    return (sign | code.astype(np.uint8)).astype(np.uint8)
+
+
+def fp8_e4m3_value(bits):
+    """FP8 E4M3 codes -> float32 values (exact)."""
+    b = np.asarray(bits, np.uint8).astype(np.int64)
+    e, m = (b >> 3) & 15, b & 7
+    v = np.where(e == 0, m * 2.0 ** -9, (8 + m) * np.exp2(e - 10.0))
+    v = np.where((b & 0x7f) == 0x7f, np.nan, v)
+    return np.where(b & 0x80, -v, v).astype(np.float32)
+
+
+def quant_blocks_fp8(x, blk, sub=None):
+    """quant_blocks with FP8 E4M3 codes and scale = absmax / 448 (cuda_flash_sage.rs:9, 209-222):
+    returns (codes uint8 [B,H,N,D], scales f32 [B,H,ceil(N/blk)])."""
+    x = _f32(x)
+    B, H, N, D = x.shape
+    if sub is not None:
+        x = (x - _f32(sub)[:, :, None, :]).astype(np.float32)
+    nblk = (N + blk - 1) // blk
+    codes = np.empty(x.shape, np.uint8)
+    scales = np.empty((B, H, nblk), np.float32)
+    for i in range(nblk):
+        seg = x[:, :, i * blk:(i + 1) * blk]
+        mx = np.abs(seg).max(axis=(2, 3)).astype(np.float32)
+        sc = np.where(mx > 0, mx / np.float32(448.0), np.float32(1.0)).astype(np.float32)
+        inv = (np.float32(1.0) / sc).astype(np.float32)
+        scales[:, :, i] = sc
+        codes[:, :, i * blk:(i + 1) * blk] = fp8_e4m3_bits((seg * inv[:, :, None, None]).astype(np.float32))
+    return codes, scales
+
+
+def sage_fp8(qc, kc, sq, sk, v, bq, bk, mask=None, causal=False, kv_len=None, scale=None, round_out=False):
+    """The quantised kernel's arithmetic with FP8 operands (the AR_FP8 branch of
+    src/runtime/cuda_flash_sage.rs:280-412): logits = sum of exact FP8 products, accumulated here in
+    binary64 and rounded to f32 once (the matrix instruction's f32 accumulation can differ in the last
+    place), s = logits * ((sq*sk)*scale), masks, f32 softmax, P and V rounded to bf16, f32 accumulate."""
+    qv, kv = fp8_e4m3_value(qc).astype(np.float64), fp8_e4m3_value(kc).astype(np.float64)
+    v = _f32(v)
+    B, Hq, N, D = qv.shape
+    Hkv = kv.shape[1]
+    group = Hq // Hkv
+    scale = np.float32(1.0 / np.sqrt(np.float32(D))) if scale is None else np.float32(scale)
+    out = np.zeros((B, Hq, N, D), np.float32)
+    i, j = np.arange(N)[:, None], np.arange(N)[None, :]
+    vb = bf16_round(v)
+    for b in range(B):
+        dead = np.zeros((N, N), bool)
+        if causal:
+            dead |= j > i
+        if kv_len is not None:
+            dead |= j >= int(kv_len[b])
+        for h in range(Hq):
+            kh = h // group
+            acc = (qv[b, h] @ kv[b, kh].T).astype(np.float32)
+            f = ((_f32(sq)[b, h][np.arange(N) // bq][:, None] * _f32(sk)[b, kh][np.arange(N) // bk][None, :]) * scale).astype(np.float32)
+            s = (acc * f).astype(np.float32)
+            if mask is not None:
+                s = (s + np.broadcast_to(_f32(mask), (N, N))).astype(np.float32)
+            s = np.where(dead, np.float32(-1e30), s)
+            m = s.max(axis=1, keepdims=True)
+            p = np.exp((s - m).astype(np.float32)).astype(np.float32)
+            p = np.where(dead, np.float32(0), p) if (causal or kv_len is not None) else p
+            l = p.sum(axis=1, keepdims=True, dtype=np.float32)
+            o = (bf16_round(p).astype(np.float64) @ vb[b, kh].astype(np.float64)).astype(np.float32)
+            o = np.where(l > 0, o / np.where(l > 0, l, 1), 0).astype(np.float32)
+            out[b, h] = bf16_round(o) if round_out else o
+    return out
+
+
 def logits_i32(q8_head, k8_head, i0, i1, j0, j1):
     """int32 QK^T of one head for rows [i0,i1) x keys [j0,j1)."""
     q8 = np.ascontiguousarray(q8_head, dtype=np.int8)

@@ -426,3 +426,31 @@ def test_backward_reference_closed_forms():
     b2 = oracle.attention_backward_f64(q, k, v, 3.0 * do)
     for x, y in zip(a[2:], b2[2:]):
         assert np.abs(3.0 * x - y).max() < 1e-4
+
+
+def test_fp8_e4m3_against_torch_and_closed_forms():
+    """oracle.fp8_e4m3_bits against torch.float8_e4m3fn casts on every representable value, on the
+    midpoints between neighbours (ties to even), on subnormals and on random data; saturation and
+    the known code points by hand (OCP FP8 specification: 448 = 0x7e, 2^-9 = 0x01, 1.0 = 0x38)."""
+    import torch
+    codes = np.arange(256, dtype=np.uint8)
+    vals = oracle.fp8_e4m3_value(codes)
+    finite = ~np.isnan(vals)
+    tv = torch.tensor(codes).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    assert np.array_equal(vals[finite], tv[finite]) and np.isnan(tv[~finite]).all()
+    assert np.array_equal(oracle.fp8_e4m3_bits(vals[finite]), codes[finite])
+    pos = np.sort(vals[finite & (vals >= 0)])
+    mids = ((pos[:-1].astype(np.float64) + pos[1:].astype(np.float64)) / 2).astype(np.float32)
+    rnd = synth.normal(5, (4096,)) * np.float32(100.0)
+    for x in (mids, -mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)), rnd[np.abs(rnd) <= 448],
+              synth.normal(6, (4096,)) * np.float32(0.01)):
+        want = torch.tensor(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        assert np.array_equal(oracle.fp8_e4m3_bits(x), want)
+    assert oracle.fp8_e4m3_bits(np.float32([448, 460, 1e9, -1e9, 1.0, 2.0 ** -9, 2.0 ** -10, 0.0])).tolist() == \
+        [0x7e, 0x7e, 0x7e, 0xfe, 0x38, 0x01, 0x00, 0x00]
+    # the quantiser: the block maximum maps to +-448 exactly, a zero block gets scale 1
+    x = synth.normal(7, (1, 2, 64, 64))
+    x[0, 1] = 0
+    c, sc = oracle.quant_blocks_fp8(x, 32)
+    assert np.abs(oracle.fp8_e4m3_value(c[0, 0, :32])).max() == 448 and sc[0, 1].tolist() == [1.0, 1.0]
+    assert np.abs(oracle.fp8_e4m3_value(c[0, 0]) * np.repeat(sc[0, 0], 32)[:, None] - x[0, 0]).max() <= np.abs(x[0, 0]).max() / 16
