@@ -360,7 +360,9 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         }
     };
 
-    uint4 pb[2];     // P of the block about to be multiplied with V
+    // P (bf16, B-operand layout) of two consecutive blocks: while the O^T MFMAs of block j read one,
+    // the softmax of block j+1 fills the other
+    uint4 p_a[2], p_b[2];
     float rs = 0.f;  // its row sum
     // The softmax of an unmasked block as a list of single vector instructions, so that they can be
     // dealt out between the matrix instructions by hand.  Per half of 8 keys: [convert (int8 only)]
@@ -412,10 +414,10 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     // the next LDS stage holds; those results are never used.
     constexpr int R2_SLOTS = DB * 2 - 2;  // S is not ready under the first two O^T MFMAs
     constexpr int SM_SPLIT = (MODE == MODE_I8) ? (SM_OPS * R2_SLOTS) / (R2_SLOTS + KSTEPS) : SM_HALF;
-    uint4 pn[2];  // P of the block whose softmax is in progress
     // mc / mn: block j / block j+1 has masked keys (causal diagonal, key-length edge); rel_cur /
     // rel_next are their mask offsets (see lim4h).
-    auto pipe_block = [&](auto mc, auto mn, acc_t &s_old, acc_t &s_new, const unsigned char *sc, int cb,
+    auto pipe_block = [&](auto mc, auto mn, acc_t &s_old, acc_t &s_new, uint4 (&p_cur)[2], uint4 (&p_nxt)[2],
+                          const unsigned char *sc, int cb,
                           const unsigned char *sv, int vb, const unsigned char *sk, int kb, float c_cur, float c_next,
                           int rel_cur, int rel_next) __attribute__((always_inline)) {
         // ---- R1 ----
@@ -430,15 +432,13 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
                 s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s_new, 0, 0, 0);
             ARHIP_FENCE();
             constexpr int lo = SM_SPLIT + st * (SM_OPS - SM_SPLIT) / KSTEPS, hi = SM_SPLIT + (st + 1) * (SM_OPS - SM_SPLIT) / KSTEPS;
-            static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mc, ic, s_old, c_cur, rel_cur, pn); });
+            static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mc, ic, s_old, c_cur, rel_cur, p_cur); });
             kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
             ARHIP_FENCE();
         });
         rs = sm_half[0] + sm_half[1];
-        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(mc, sc, cb, c_cur, rel_cur, pn, rs);
+        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(mc, sc, cb, c_cur, rel_cur, p_cur, rs);
         l_run += rs;
-        pb[0] = pn[0];
-        pb[1] = pn[1];
         ARHIP_FENCE();
         // ---- R2 ----
         static_for<0, DB * 2>([&](auto gi) __attribute__((always_inline)) {
@@ -446,11 +446,11 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
             constexpr int db = g / 2, ks = g % 2;
             const uint4 a = make_uint4(vf[db][ks][0].x, vf[db][ks][0].y, vf[db][ks][1].x, vf[db][ks][1].y);
             oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                               __builtin_bit_cast(bf16x8, pb[ks]), oacc[db], 0, 0, 0);
+                                                               __builtin_bit_cast(bf16x8, p_cur[ks]), oacc[db], 0, 0, 0);
             ARHIP_FENCE();
             if constexpr (g >= 2) {
                 constexpr int lo = (g - 2) * SM_SPLIT / R2_SLOTS, hi = (g - 1) * SM_SPLIT / R2_SLOTS;
-                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mn, ic, s_new, c_next, rel_next, pn); });
+                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mn, ic, s_new, c_next, rel_next, p_nxt); });
             }
             if constexpr (ks == 1) {
 #pragma unroll
@@ -499,9 +499,9 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         load_vf(lds, 0);
         const float c0 = tile_c(0, 0);
         if (nfull > 0)
-            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(PLAIN, ic, s_a, c0, 0, pn); });
+            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(PLAIN, ic, s_a, c0, 0, p_a); });
         else
-            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(MASKED, ic, s_a, c0, lim4h, pn); });
+            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(MASKED, ic, s_a, c0, lim4h, p_a); });
     }
 
     // one tile: its two blocks; m0 / m1 / m2 say whether the first block, the second block and the
@@ -514,8 +514,8 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         advance_sk_group(it);
         const float c_cur = tile_c(it, it), c_nxt = tile_c(it + 1, it);
         const int rel0 = lim4h - it * BK;
-        pipe_block(m0, m1, s_a, s_b, st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, c_cur, rel0, rel0 - 32);
-        pipe_block(m1, m2, s_b, s_a, st_cur, 1, st_nxt, 0, st_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64);
+        pipe_block(m0, m1, s_a, s_b, p_a, p_b, st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, c_cur, rel0, rel0 - 32);
+        pipe_block(m1, m2, s_b, s_a, p_b, p_a, st_cur, 1, st_nxt, 0, st_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64);
         wait_vmem_le<XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
         __syncthreads();
     };
