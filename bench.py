@@ -28,6 +28,7 @@ from autorust_amd import _lib, synth  # noqa: E402
 from autorust_amd.device import BF16, F32, Device  # noqa: E402
 
 PEAK_BF16 = 2500.0   # TFLOP/s, MI355X dense bf16 MFMA
+PEAK_F32 = 157.3     # TFLOP/s, MI355X dense fp32 MFMA
 PEAK_INT8 = 5000.0   # TOP/s, MI355X dense int8 MFMA
 PEAK_HBM = 8000.0    # GB/s, MI355X HBM3E
 
@@ -174,12 +175,49 @@ class FlashWorkload:
                 b.free()
 
 
+class TrainWorkload:
+    """fp32 training step of one attention layer: forward with the saved log-sum-exp, then the
+    backward (prep + dQ + dK/dV): src/runtime/cuda_flash_train.rs.  14 B H S^2 D flops per step:
+    2 products forward, 5 backward (S and dP are each computed by both backward kernels)."""
+
+    def __init__(self, dev, B, H, S, D, causal, cfg):
+        self.dev, self.B, self.H, self.S, self.D, self.causal = dev, B, H, S, D, causal
+        self.name = "train_f32_b%d_h%d_s%d_d%d%s" % (B, H, S, D, "_causal" if causal else "")
+        n = B * H * S * D
+        arrs = [synth.normal(1000 * cfg + i, (B, H, S, D)) for i in (1, 2, 3, 8)]
+        self.host = dict(zip("qkv", arrs[:3]))
+        self.dq, self.dk, self.dv, self.ddo = (dev.from_numpy(a) for a in arrs)
+        self.o, self.gq, self.gk, self.gv = (dev.alloc(n * 4) for _ in range(4))
+        self.lse, self.delta = dev.alloc(B * H * S * 4), dev.alloc(B * H * S * 4)
+        self.ops = 14.0 * B * H * S * S * D * (0.5 if causal else 1.0)
+        self.kernel = _lib.K_FLASH_BWD
+        self.kernel_bytes = 8 * n * 4   # backward: q, k, v, o, dO in; dq, dk, dv out
+        self.dtype = "f32"
+
+    def step(self):
+        d, B, H, S, D = self.dev, self.B, self.H, self.S, self.D
+        d.flash_fwd_lse(self.dq, self.dk, self.dv, self.o, self.lse, B, H, H, S, D, F32, causal=self.causal, wait=False)
+        d.flash_bwd(self.dq, self.dk, self.dv, self.o, self.lse, self.ddo, self.gq, self.gk, self.gv, self.delta,
+                    B, H, H, S, D, causal=self.causal, wait=False)
+
+    def roofline(self, secs):
+        bwd_ops = self.ops * 10.0 / 14.0
+        ach = bwd_ops / secs / 1e12
+        return {"bound": "mfma", "achieved": ach, "peak": PEAK_F32, "unit": "TFLOP/s", "frac": ach / PEAK_F32,
+                "traffic": None, "kernel": "bwd_prep + bwd_dq + bwd_dkv (f32)", "launch_ms": secs * 1e3,
+                "ops_per_launch": bwd_ops, "peak_note": "dense fp32 MFMA"}
+
+    def free(self):
+        for b in (self.dq, self.dk, self.dv, self.ddo, self.o, self.gq, self.gk, self.gv, self.lse, self.delta):
+            b.free()
+
+
 def measure(dev, w, steps, warmup):
     for _ in range(warmup):
         w.step()
     dev.sync()
     dev.kprof_enable(True)
-    for k in range(_lib.K_SAGE_QUANT + 1):
+    for k in range(_lib.K_FLASH_BWD + 1):
         dev.kprof_collect(k)
     dev.timer_start()
     for _ in range(steps):
@@ -297,6 +335,8 @@ def build_workload(dev, name):
     if name == "vit_f32":
         return FlashWorkload(dev, 1, 12, 197, 64, False, F32, cfg=1)
     # the shape the reference publishes its own kernel times on (B8 H6 N789 D64, PERFORMANCE.md:314-317)
+    if name == "train_f32":   # the ViT-B/16 layer shape at batch 8, fp32 (the reference's training kernels are f32 only)
+        return TrainWorkload(dev, 8, 12, 197, 64, False, cfg=8)
     if name == "ref_bf16":
         return FlashWorkload(dev, 8, 6, 789, 64, False, BF16, cfg=7)
     if name == "ref_f32":
@@ -318,7 +358,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="sage",
                     choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32", "flash_long", "ref_bf16",
-                             "ref_f32", "ref_sage"])
+                             "ref_f32", "ref_sage", "train_f32"])
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="one step of the workload plus one plain 1 GiB copy kernel and nothing else: "
@@ -360,7 +400,7 @@ def main():
     secondary = []
     if not args.no_secondary:
         for name in ("vit", "decoder", "flash_long", "vit_f32", "sage", "sage_causal_long", "ref_bf16", "ref_f32",
-                     "ref_sage"):
+                     "ref_sage", "train_f32"):
             if name == args.workload:
                 continue
             sw = build_workload(dev, name)
