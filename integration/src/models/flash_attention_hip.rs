@@ -28,6 +28,11 @@
 //! `Tensor::empty(..).to_param()` replaces the `from_slice(&vec![0.0; ..])` of `:514-530`.
 //!
 //! In `ViT::forward_with` (`vit.rs:119-121`): `|| d.starts_with("HIP")`.
+//!
+//! In `fused_attention_train` / `fused_attention_backward` (`:789-977`): accept `dev.starts_with("HIP")`
+//! beside `"CUDA"`, `supports(n, d)` becomes `d == 64 || d == 128`, and the launches become
+//! `hip_flash::host_call_train_fwd` / `hip_flash::host_calls_train_bwd` (same buffers, same order;
+//! `dk`/`dv` need no zero fill: the GQA sum happens inside the kernel).
 
 use crate::engine::session::HostCall;
 use crate::runtime::buffer::Buffer;

@@ -233,3 +233,30 @@ pub fn host_calls_sage(
     }
     calls
 }
+
+// ---- training (counterpart of `cuda_flash_train::{run_fwd, run_prep, run_dq, run_dkv}`,
+// src/runtime/cuda_flash_train.rs:336-541): f32 tensors, dense `[b, h, n, d]` ----
+
+/// Forward that also writes `lse [b*h, n]`: `bufs = [q, k, v, o, lse, mask-or-o]`.
+pub fn host_call_train_fwd(bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
+    let f = dtype::FLOAT32;
+    call("ar_fl_fwd", bufs, &[f, f, f, f, f, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+}
+
+/// The three launches of the backward, in order.  `delta` is a scratch tensor `[b*h, n]`; `mask` is
+/// the additive mask or `dq` again (the reference's dummy, cuda_flash_train.rs:442-449).
+#[allow(clippy::too_many_arguments)]
+pub fn host_calls_train_bwd(
+    q: Buffer, k: Buffer, v: Buffer, o: Buffer, lse: Buffer, dout: Buffer, mask: Buffer, delta: Buffer,
+    dq: Buffer, dk: Buffer, dv: Buffer, b: i64, h: i64, n: i64, d: i64, opts: Options,
+) -> Vec<HostCall> {
+    let f = dtype::FLOAT32;
+    let tiles = (n + 127) / 128;
+    vec![
+        call("ar_fl_prep", vec![o, dout.clone(), delta.clone()], &[f, f, f], [(n + 3) / 4, b * h, 1], [256, 1, 1], vec![n, d], &[]),
+        call("ar_fl_bwd_dq", vec![q.clone(), k.clone(), v.clone(), dout.clone(), lse.clone(), delta.clone(), mask.clone(), dq],
+             &[f, f, f, f, f, f, f, f], [tiles, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[]),
+        call("ar_fl_bwd_dkv", vec![q, k, v, dout, lse, delta, mask, dk, dv],
+             &[f, f, f, f, f, f, f, f, f], [tiles, b * opts.h_kv, 1], [256, 1, 1], vals(n, d, h, opts), &[]),
+    ]
+}
