@@ -391,7 +391,7 @@ def main():
     log(json.dumps(res))
     cpu = None
     if not args.no_cpu:
-        heads = {"sage": 2, "sage_causal_long": 1, "decoder": 16, "vit": 96, "vit_f32": 12, "flash_long": 2}.get(
+        heads = {"sage": 32, "sage_causal_long": 2, "decoder": 128, "vit": 96, "vit_f32": 12, "flash_long": 32}.get(
             args.workload, 48)
         cpu = cpu_baseline(w, heads)
         log(json.dumps(cpu))
