@@ -42,6 +42,7 @@ SIGNATURES = {
     "arhip_timer_stop": (c_int, [c_void_p, _pd]),
     "arhip_kprof_enable": (c_int, [c_void_p, c_int]),
     "arhip_kprof_collect": (c_int, [c_void_p, c_int, _pd, ctypes.POINTER(ctypes.c_uint64)]),
+    "arhip_kprof_collect_stats": (c_int, [c_void_p, c_int, _pd, ctypes.POINTER(ctypes.c_uint64), _pd, _pd]),
     "arhip_graph_begin": (c_int, [c_void_p]),
     "arhip_graph_end": (c_int, [c_void_p, ctypes.POINTER(c_void_p)]),
     "arhip_graph_launch": (c_int, [c_void_p, c_void_p, c_int, _pd]),

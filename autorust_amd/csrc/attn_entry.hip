@@ -215,12 +215,13 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long(const uint1
     }
 }
 
-extern "C" __global__ void __launch_bounds__(256) ar_flash_sage(const int8_t *Q8, const int8_t *K8, const uint16_t *V, float *O,
-                                                                 const float *M, const float *SQ, const float *SK, int N,
-                                                                 int head_dim, int causal, int has_mask, int hq, int hkv,
-                                                                 int bq, int bk)
+namespace {
+// ar_flash_sage / ar_flash_sage_fp8: the general kernel on pre-quantised operands, QMODE = MODE_I8 or MODE_FP8
+template <int QMODE>
+__device__ __forceinline__ void flash_sage_entry(unsigned char *lds, const void *Q8, const void *K8, const uint16_t *V, float *O,
+                                                 const float *M, const float *SQ, const float *SK, int N, int head_dim, int causal,
+                                                 int has_mask, int hq, int hkv, int bq, int bk)
 {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_I8, true>()];
     AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, has_mask, hq, hkv);
     p.sq = SQ; p.sk = SK;
     p.bq = bq; p.bk = bk;
@@ -234,11 +235,11 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_sage(const int8_t *Q8
 #define AR_SAGE(DD, PK)                                                                                 \
     do {                                                                                                \
         if (has_mask) {                                                                                 \
-            if (causal) attn_fwd_body<DD, 4, true, true, MODE_I8, PK, true, false>(p, lds, wg);         \
-            else attn_fwd_body<DD, 4, false, true, MODE_I8, PK, true, false>(p, lds, wg);               \
+            if (causal) attn_fwd_body<DD, 4, true, true, QMODE, PK, true, false>(p, lds, wg);           \
+            else attn_fwd_body<DD, 4, false, true, QMODE, PK, true, false>(p, lds, wg);                 \
         } else {                                                                                        \
-            if (causal) attn_fwd_body<DD, 4, true, false, MODE_I8, PK, true, false>(p, lds, wg);        \
-            else attn_fwd_body<DD, 4, false, false, MODE_I8, PK, true, false>(p, lds, wg);              \
+            if (causal) attn_fwd_body<DD, 4, true, false, QMODE, PK, true, false>(p, lds, wg);          \
+            else attn_fwd_body<DD, 4, false, false, QMODE, PK, true, false>(p, lds, wg);                \
         }                                                                                               \
     } while (0)
     if (head_dim == 64) {
@@ -249,6 +250,27 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_sage(const int8_t *Q8
         else AR_SAGE(128, false);
     }
 #undef AR_SAGE
+}
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_sage(const int8_t *Q8, const int8_t *K8, const uint16_t *V, float *O,
+                                                                 const float *M, const float *SQ, const float *SK, int N,
+                                                                 int head_dim, int causal, int has_mask, int hq, int hkv,
+                                                                 int bq, int bk)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_I8, true>()];
+    flash_sage_entry<MODE_I8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
+}
+
+// the FP8 E4M3 variant (the reference's AR_FP8 = 1 source, src/runtime/cuda_flash_sage.rs:82-84): same
+// arguments, Q8 / K8 hold E4M3 codes
+extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_fp8(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
+                                                                     float *O, const float *M, const float *SQ, const float *SK,
+                                                                     int N, int head_dim, int causal, int has_mask, int hq,
+                                                                     int hkv, int bq, int bk)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_FP8, true>()];
+    flash_sage_entry<MODE_FP8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
 }
 
 extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
@@ -329,6 +351,24 @@ extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_bf16(const 
     if (smooth) quant_rows_body<uint16_t, true>(x, x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);
     else quant_rows_body<uint16_t, false>(x, x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);
 }
+// FP8 E4M3 quantiser entries: same arguments, x8 receives E4M3 codes, scale = absmax / 448
+#define AR_QUANT_FP8(SUFFIX, T)                                                                                              \
+    extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_blocks_fp8_##SUFFIX(                                     \
+        const T *x, uint8_t *x8, float *scales, const float *mean, int N, int D, int blk, int nblk, int smooth)              \
+    {                                                                                                                        \
+        if (smooth) quant_blocks_body<T, true, true>(x, (int8_t *)x8, scales, mean, N, D, blk, nblk, XLayout::dense(1, N, D), blockIdx);  \
+        else quant_blocks_body<T, false, true>(x, (int8_t *)x8, scales, mean, N, D, blk, nblk, XLayout::dense(1, N, D), blockIdx);        \
+    }                                                                                                                        \
+    extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_fp8_##SUFFIX(                                       \
+        const T *x, uint8_t *x8, float *scales, const float *mean, int N, int D, long rows_total, int smooth)                \
+    {                                                                                                                        \
+        if (smooth) quant_rows_body<T, true, true>(x, (int8_t *)x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);   \
+        else quant_rows_body<T, false, true>(x, (int8_t *)x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);         \
+    }
+AR_QUANT_FP8(f32, float)
+AR_QUANT_FP8(bf16, uint16_t)
+#undef AR_QUANT_FP8
+
 extern "C" __global__ void __launch_bounds__(256) ar_cast_bf16(const float *x, uint16_t *y, long n)
 {
     cast_bf16_body(x, y, (size_t)n, blockIdx);

@@ -5,6 +5,7 @@
 // encoding (:888-1019).  One stream per handle, default priority.
 #include "arhip_internal.h"
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
@@ -286,10 +287,17 @@ extern "C" int arhip_kprof_enable(arhip_device *dev, int on)
 
 extern "C" int arhip_kprof_collect(arhip_device *dev, int kernel, double *total_secs, uint64_t *launches)
 {
+    return arhip_kprof_collect_stats(dev, kernel, total_secs, launches, nullptr, nullptr);
+}
+
+extern "C" int arhip_kprof_collect_stats(arhip_device *dev, int kernel, double *total_secs, uint64_t *launches,
+                                         double *min_secs, double *median_secs)
+{
     ARHIP_DEV(dev);
     ARHIP_HIP(hipStreamSynchronize(dev->stream));
     double tot = 0.0;
     uint64_t n = 0;
+    std::vector<double> each;
     std::vector<arhip_device::prof_entry> keep;
     for (auto &e : dev->prof_log) {
         if (e.kernel != kernel) {
@@ -299,6 +307,7 @@ extern "C" int arhip_kprof_collect(arhip_device *dev, int kernel, double *total_
         float ms = 0.f;
         ARHIP_HIP(hipEventElapsedTime(&ms, e.e0, e.e1));
         tot += (double)ms * 1e-3;
+        each.push_back((double)ms * 1e-3);
         ++n;
         dev->prof_pool.push_back(e.e0);
         dev->prof_pool.push_back(e.e1);
@@ -306,6 +315,9 @@ extern "C" int arhip_kprof_collect(arhip_device *dev, int kernel, double *total_
     dev->prof_log.swap(keep);
     if (total_secs) *total_secs = tot;
     if (launches) *launches = n;
+    std::sort(each.begin(), each.end());
+    if (min_secs) *min_secs = each.empty() ? 0.0 : each.front();
+    if (median_secs) *median_secs = each.empty() ? 0.0 : 0.5 * (each[(each.size() - 1) / 2] + each[each.size() / 2]);
     return ARHIP_OK;
 }
 

@@ -43,6 +43,7 @@ Settings Settings::from_env()
     if (const char *a = getenv("AUTORUST_ATTN")) s.attention = attention_kind_from_str(a);
     s.tensor_cores = env_flag("AUTORUST_TENSOR_CORES", env_flag("AUTORUST_TC", true));
     s.async_pipeline = env_flag("AUTORUST_ASYNC", true);
+    if (const char *f = getenv("AUTORUST_SAGE_FP8")) s.sage_fp8 = f[0] == '1';
     if (const char *m = getenv("AUTORUST_MATH")) {
         if (std::string(m) == "exact") {  // settings.rs:202-208: exact mode turns the matrix units off
             s.math_exact = true;
@@ -412,7 +413,9 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     Tensor sq = Tensor::empty(dev, {b, h, nqb}, F), sk = Tensor::empty(dev, {b, hk, nkb}, F);
     Tensor mean = Tensor::empty(dev, {b, hk, d}, F);
     const std::string part_name = std::string("ar_sage_kmean_partial_") + sfx;
-    const std::string rows_name = std::string("ar_sage_quant_rows_") + sfx, blocks_name = std::string("ar_sage_quant_blocks_") + sfx;
+    const std::string q8fmt = st.sage_fp8 ? "fp8_" : "";
+    const std::string rows_name = "ar_sage_quant_rows_" + q8fmt + sfx, blocks_name = "ar_sage_quant_blocks_" + q8fmt + sfx;
+    const char *general = st.sage_fp8 ? "ar_flash_sage_fp8" : "ar_flash_sage";
     auto quant = [&](const Tensor &x, const Tensor &x8, const Tensor &sc, int64_t heads, int64_t blk, int64_t nblk, bool smooth) {
         if (blk == 1) {
             const int64_t rows = b * heads * n, rpb = 256 / (d / 8);
@@ -445,19 +448,19 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     int shift = 0;
     while (((int64_t)64 << shift) < bk) ++shift;
     const bool tile_uniform = ((int64_t)64 << shift) == bk;
-    if (!has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
+    if (!st.sage_fp8 && !has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
         svals.push_back(bf16_in ? 0 : 1);  // out_f32
         calls.push_back(make_call(dev, "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
                                   {(n + 255) / 256, b * h, 1}, {512, 1, 1}, svals));
     } else if (!bf16_in) {
-        calls.push_back(make_call(dev, "ar_flash_sage", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, F, F, F, F},
+        calls.push_back(make_call(dev, general, {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, F, F, F, F},
                                   {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
     } else {
         // ar_flash_sage stores f32 (the reference's convention); bf16 tensors get their bf16 result
         // through one more cast
         Tensor o32 = Tensor::empty(dev, {b, h, n, d}, F);
         const Tensor m2 = has_mask ? *attn_mask : o32;
-        calls.push_back(make_call(dev, "ar_flash_sage", {q8, k8, vb, o32, m2, sq, sk}, {I8, I8, BF, F, F, F, F},
+        calls.push_back(make_call(dev, general, {q8, k8, vb, o32, m2, sq, sk}, {I8, I8, BF, F, F, F, F},
                                   {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
         const int64_t no = b * h * n * d;
         calls.push_back(make_call(dev, "ar_cast_bf16", {o32, out}, {F, BF}, {std::min<int64_t>((no + 255) / 256, 16384), 1, 1},

@@ -47,6 +47,10 @@ struct Settings {
     // Sage extension of this build (the reference quantises per row and does not smooth K)
     int64_t sage_block_q = 128, sage_block_k = 64;
     bool sage_smooth_k = true;
+    // `cuda_flash_sage::Options::fp8` (cuda_flash_sage.rs:53-54): E4M3 codes and the FP8 matrix instruction
+    // instead of int8.  The reference switches it on wherever the device has FP8 tensor cores; here it
+    // is opt-in (AUTORUST_SAGE_FP8=1) because the int8 path is the measured one.
+    bool sage_fp8 = false;
     static Settings from_env();                      // settings.rs:174-282
 };
 

@@ -13,6 +13,7 @@ struct arh_settings {
     int attention, tensor_cores, async_pipeline, math_exact;
     int64_t sage_block_q, sage_block_k;
     int sage_smooth_k;
+    int sage_fp8;
 };
 
 static Settings to_settings(const arh_settings *s)
@@ -26,6 +27,7 @@ static Settings to_settings(const arh_settings *s)
     st.sage_block_q = s->sage_block_q;
     st.sage_block_k = s->sage_block_k;
     st.sage_smooth_k = s->sage_smooth_k != 0;
+    st.sage_fp8 = s->sage_fp8 != 0;
     return st;
 }
 
@@ -52,12 +54,12 @@ const char *arh_last_error(void) { return g_err.c_str(); }
 void arh_settings_default(arh_settings *out)
 {
     const Settings s;
-    *out = {(int)s.attention, s.tensor_cores, s.async_pipeline, s.math_exact, s.sage_block_q, s.sage_block_k, s.sage_smooth_k};
+    *out = {(int)s.attention, s.tensor_cores, s.async_pipeline, s.math_exact, s.sage_block_q, s.sage_block_k, s.sage_smooth_k, s.sage_fp8};
 }
 void arh_settings_from_env(arh_settings *out)
 {
     const Settings s = Settings::from_env();
-    *out = {(int)s.attention, s.tensor_cores, s.async_pipeline, s.math_exact, s.sage_block_q, s.sage_block_k, s.sage_smooth_k};
+    *out = {(int)s.attention, s.tensor_cores, s.async_pipeline, s.math_exact, s.sage_block_q, s.sage_block_k, s.sage_smooth_k, s.sage_fp8};
 }
 const char *arh_attention_kind_name(int k) { return name((AttentionKind)k); }
 int arh_attention_kind_from_str(const char *s) { return (int)attention_kind_from_str(s); }

@@ -97,6 +97,13 @@ class Device:
     def kprof_enable(self, on=True):
         check(self.lib.arhip_kprof_enable(self.handle, int(on)))
 
+    def kprof_collect_stats(self, kernel):
+        """(total seconds, launches, shortest, median) of `kernel` since the last collect."""
+        s, n, lo, med = ctypes.c_double(), ctypes.c_uint64(), ctypes.c_double(), ctypes.c_double()
+        check(self.lib.arhip_kprof_collect_stats(self.handle, kernel, ctypes.byref(s), ctypes.byref(n), ctypes.byref(lo),
+                                                 ctypes.byref(med)))
+        return s.value, n.value, lo.value, med.value
+
     def kprof_collect(self, kernel):
         """(total seconds, launches) of `kernel` since the last collect."""
         s, n = ctypes.c_double(), ctypes.c_uint64()

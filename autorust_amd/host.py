@@ -33,7 +33,7 @@ class AttentionKind:
 class Settings(ctypes.Structure):
     _fields_ = [("attention", ctypes.c_int), ("tensor_cores", ctypes.c_int), ("async_pipeline", ctypes.c_int),
                 ("math_exact", ctypes.c_int), ("sage_block_q", ctypes.c_int64), ("sage_block_k", ctypes.c_int64),
-                ("sage_smooth_k", ctypes.c_int)]
+                ("sage_smooth_k", ctypes.c_int), ("sage_fp8", ctypes.c_int)]
 
     @staticmethod
     def default():

@@ -223,13 +223,15 @@ def measure(dev, w, steps, warmup):
     for _ in range(steps):
         w.step()
     total = dev.timer_stop()
-    ksecs, kn = dev.kprof_collect(w.kernel)
+    ksecs, kn, kmin, kmed = dev.kprof_collect_stats(w.kernel)
     qsecs, qn = dev.kprof_collect(_lib.K_SAGE_QUANT)
     dev.kprof_enable(False)
     ms = total / steps * 1e3
     res = {"workload": w.name, "ms_per_step": ms, "ops_per_step": w.ops,
            "tops": w.ops / (total / steps) / 1e12,
            "roofline": w.roofline(ksecs / max(kn, 1))}
+    res["roofline"]["launch_ms_min"] = kmin * 1e3
+    res["roofline"]["launch_ms_median"] = kmed * 1e3
     if qn:
         res["prepass_ms_per_step"] = qsecs / steps * 1e3
     if w.S < 1024:

@@ -88,6 +88,9 @@ int arhip_timer_stop(arhip_device *dev, double *secs); /* records, waits, return
  *      the last collect, and forgets them. ---- */
 int arhip_kprof_enable(arhip_device *dev, int on);
 int arhip_kprof_collect(arhip_device *dev, int kernel, double *total_secs, uint64_t *launches);
+/* the same, also returning the shortest and the median launch (NULL: not wanted) */
+int arhip_kprof_collect_stats(arhip_device *dev, int kernel, double *total_secs, uint64_t *launches,
+                              double *min_secs, double *median_secs);
 
 /* ---- launch graphs: captured replay (`Session::capture_host` + `Jit::replay`,
  *      src/engine/session.rs:138-146, src/engine/jit.rs:186-195) as one device submission.

@@ -194,3 +194,30 @@ def test_training_kernels_by_name(dev, kernels, case):
     for name, g, w in zip(("o", "lse", "dq", "dk", "dv"), got, want):
         assert np.abs(g - w).max() < 2e-3, name
         assert np.abs(g - w).max() <= 3e-5 * max(1.0, np.abs(w).max()), name
+
+
+def test_ar_flash_sage_fp8_by_name(dev, kernels):
+    """The FP8 entries by name: codes and scales bit-exact against the oracle's E4M3 quantiser, output
+    within 2e-3 of the emulation (tests/sage_int8.rs:148)."""
+    b, hq, hkv, n, d, bq, bk = 1, 4, 2, 200, 64, 128, 64
+    q, k, v = fill_qkv(b, hq, hkv, n, d)
+    with Bufs(dev) as bufs:
+        def quant(x, blk, heads):
+            dx, x8 = bufs.put(x), bufs.new(x.size)
+            nblk = (n + blk - 1) // blk
+            sc, mean = bufs.new(b * heads * nblk * 4), bufs.new(b * heads * d * 4)
+            dev.launch(kernels, "ar_sage_quant_blocks_fp8_f32", (nblk, b * heads, 1), (256, 1, 1), [dx, x8, sc, mean],
+                       [n, d, blk, nblk, 0])
+            return x8, sc, x8.copyout(np.uint8, x.shape), sc.copyout(np.float32, (b, heads, nblk))
+        q8, sq, h_q8, h_sq = quant(q, bq, hq)
+        k8, sk, h_k8, h_sk = quant(k, bk, hkv)
+        dv = bufs.put(synth.to_bf16_bits(v))
+        do = bufs.new(q.size * 4)
+        dev.launch(kernels, "ar_flash_sage_fp8", _grid(n, 128, b, hq), (256, 1, 1), [q8, k8, dv, do, do, sq, sk],
+                   [n, d, 1, 0, hq, hkv, bq, bk])
+        got = do.copyout(np.float32, q.shape)
+    w_q8, w_sq = oracle.quant_blocks_fp8(q, bq)
+    w_k8, w_sk = oracle.quant_blocks_fp8(k, bk)
+    assert np.array_equal(h_q8, w_q8) and np.array_equal(h_sq, w_sq) and np.array_equal(h_k8, w_k8) and np.array_equal(h_sk, w_sk)
+    want = oracle.sage_fp8(w_q8, w_k8, w_sq, w_sk, v, bq, bk, causal=True)
+    assert np.abs(got - want).max() < 2e-3

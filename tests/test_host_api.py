@@ -194,6 +194,24 @@ def test_fused_attention_wrappers(hdev):
 
 
 @gpu
+def test_sage_fp8_setting(hdev):
+    """Settings.sage_fp8 (the reference's `Options::fp8`, cuda_flash_sage.rs:53-54) routes the quantised
+    path through the FP8 entries."""
+    b, h, n, d = 1, 4, 300, 128
+    q, k, v = _fill((b, h, n, d), 3), _fill((b, h, n, d), 11), _fill((b, h, n, d), 19)
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v))
+    st = Settings.default()
+    st.sage_fp8 = 1
+    sess = Session()
+    sess.begin_capture()
+    out = tq.sage_attention_with(tk, tv, None, 0.0, True, sess, st)
+    n_calls = sess.end_capture()
+    names = [sess.step(i)[0] for i in range(n_calls)]
+    assert names[0] == "ar_sage_quant_blocks_fp8_f32" and "ar_flash_sage_fp8" in names
+    assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v, causal=True)).max()) < 6e-2
+
+
+@gpu
 def test_fused_attention_train_and_backward(hdev):
     """The reference's own differential test of the training path (tests/flash_train_cuda.rs:40-106):
     fused forward (out, lse) then fused backward (dq, dk, dv) within 2e-3 of the gradients of SDPA
