@@ -4,8 +4,9 @@
 // O^T += V^T . P^T), different plumbing:
 //
 //   HBM -> LDS   K and V tiles of 64 keys go straight to LDS (buffer_load ... lds, 16 bytes per
-//                lane, no registers in between), four stages deep, so a tile is requested two
-//                iterations before its first use.  Rows past the last visible key come back as
+//                lane, no registers in between), four stages deep, so a tile is requested three
+//                iterations before the one that computes on it (two before the look-ahead
+//                first touches it).  Rows past the last visible key come back as
 //                zeros from the buffer bounds check; nothing is clamped or branched on.
 //   LDS layout   A transfer writes 64 x 16 bytes to consecutive addresses, so rows cannot be padded.
 //                Rows are cut into 64-byte pieces and stored [piece][row][64 B]; inside a block of
@@ -26,7 +27,9 @@
 //                K(j+1) and V(j) fragments.
 //   reference    lazy exponent reference as in attn_fwd.h; it is checked between R1 and R2 (the
 //                rare case recomputes the block's logits from K, which is still in LDS).
-//   masked tiles (causal diagonal, key-length edge) run block by block without look-ahead.
+//   masked tiles (causal diagonal, key-length edge) run the same pipeline with the mask applied inside
+//                the softmax instructions; a wave past its last query only keeps feeding the
+//                transfers and barriers.
 //
 // 8 waves of 32 queries per workgroup, two waves per SIMD.
 #pragma once
