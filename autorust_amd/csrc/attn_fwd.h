@@ -146,15 +146,22 @@ constexpr int attn_fwd_lds_bytes()
 // The kernel body.  lds: attn_fwd_lds_bytes<...>() bytes of workgroup memory, 16-byte aligned;
 // wg_linear: this workgroup's index in [0, p.total) (the entry points below and the named entry
 // points of the loadable code object derive it from their grids).
-template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false>
+template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false,
+          int KSPLIT = 1>
 __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
+    // KSPLIT = 2 (with SMALL): waves w and w + NW/2 own the same 32 queries and take the even / odd
+    // key tiles; their (m, l, O) are merged through LDS at the end.  A short sequence gives a wave
+    // only a handful of blocks, each a serial MFMA -> softmax -> MFMA chain: two waves per SIMD on
+    // half the blocks each overlap those chains and halve their length.
+    static_assert(KSPLIT == 1 || (KSPLIT == 2 && SMALL && NW % 2 == 0), "key splitting is built for the preloading variant");
+    constexpr int QW = NW / KSPLIT;  // waves that own distinct queries
     // SMALL: the whole sequence (at most 4 tiles) is brought into LDS up front, all global loads
     // in flight at once and a single barrier: short sequences are latency bound, not math bound.
     constexpr int NSTAGE = SMALL ? 4 : 2;
     constexpr int NSLOT = SMALL ? 4 : 1;  // register sets for tiles in flight
     constexpr int T = NW * 64;
-    constexpr int BQ = NW * 32;
+    constexpr int BQ = QW * 32;
     constexpr int QK_BYTES = (MODE != MODE_BF16) ? 1 : 2;        // bytes per q/k element
     constexpr int KROW = D * QK_BYTES + 16;                    // padded K row in LDS
     constexpr int K_TILE = BK * KROW;
@@ -208,7 +215,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     const int N = p.N;
 
     const int qblk = qt * BQ;
-    const int wq0 = qblk + wave * 32;  // first query of this wave
+    const int qwave = wave % QW, kpart = wave / QW;
+    const int wq0 = qblk + qwave * 32;  // first query of this wave
     const int q_row = wq0 + i32;
 
     int kvl = N;
@@ -506,11 +514,37 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
             if (t < ntiles) store_tile(t, t);
         __syncthreads();
         auto nothing = [] {};
-        for (int it = 0; it < my_tiles; ++it) {
+        for (int it = kpart; it < my_tiles; it += KSPLIT) {
             const int k0 = it * BK;
             const bool masked = (k0 + BK > kend) || (CAUSAL && (k0 + BK - 1 > wq0));
             if (HAS_MASK || masked) tile_body(std::true_type{}, it, nothing);
             else tile_body(std::false_type{}, it, nothing);
+        }
+        if constexpr (KSPLIT == 2) {
+            // merge the two key halves: m = max, l and O rescaled by 2^(m_part - m)
+            constexpr int SLAB = DB * 16 * 64 + 128;  // floats per query group: O, then m and l, lane-major
+            static_assert(QW * SLAB * 4 <= NSTAGE * STAGE, "merge buffer fits the tile stages");
+            __syncthreads();  // every wave is done with the tiles
+            float *mb = (float *)lds + qwave * SLAB;
+            if (kpart == 1) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mb[(db * 16 + r) * 64 + lane] = oacc[db][r];
+                mb[DB * 16 * 64 + lane] = m_run;
+                mb[DB * 16 * 64 + 64 + lane] = l_run;
+            }
+            __syncthreads();
+            if (kpart == 1) return;
+            const float m1 = mb[DB * 16 * 64 + lane], l1 = mb[DB * 16 * 64 + 64 + lane];
+            const float m = fmaxf(m_run, m1);
+            const float f0 = __builtin_amdgcn_exp2f(m_run - m), f1 = __builtin_amdgcn_exp2f(m1 - m);
+            l_run = l_run * f0 + l1 * f1;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[db][r] = oacc[db][r] * f0 + mb[(db * 16 + r) * 64 + lane] * f1;
+            m_run = m;
         }
     } else {
     // Staging runs two tiles ahead of the math with one set of registers: in the middle of the
@@ -587,11 +621,12 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     }
 }
 
-template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false>
+template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false,
+          int KSPLIT = 1>
 __global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd_kernel(const AttnParams p)
 {
     __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<D, NW, MODE, PER_KEY, SMALL>()];
-    attn_fwd_body<D, NW, CAUSAL, HAS_MASK, MODE, PER_KEY, OUT_F32, DBG, SMALL>(p, lds, (int)blockIdx.x);
+    attn_fwd_body<D, NW, CAUSAL, HAS_MASK, MODE, PER_KEY, OUT_F32, DBG, SMALL, KSPLIT>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

@@ -212,13 +212,14 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
         // short sequence: bring all of K/V into LDS at once (128 queries per workgroup)
         p.nq = (int)((N + 127) / 128);
         p.total = (int)(p.nq * B * Hq);
-        const dim3 grid((unsigned)p.total), block(256);
+        // 8 waves: two per 32 queries, one on the even and one on the odd key tiles
+        const dim3 grid((unsigned)p.total), block(512);
         if (D == 64) {
-            if (c) hipLaunchKernelGGL((attn_fwd_kernel<64, 4, true, false, MODE_BF16, false, false, false, true>), grid, block, 0, dev->stream, p);
-            else hipLaunchKernelGGL((attn_fwd_kernel<64, 4, false, false, MODE_BF16, false, false, false, true>), grid, block, 0, dev->stream, p);
+            if (c) hipLaunchKernelGGL((attn_fwd_kernel<64, 8, true, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
+            else hipLaunchKernelGGL((attn_fwd_kernel<64, 8, false, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
         } else {
-            if (c) hipLaunchKernelGGL((attn_fwd_kernel<128, 4, true, false, MODE_BF16, false, false, false, true>), grid, block, 0, dev->stream, p);
-            else hipLaunchKernelGGL((attn_fwd_kernel<128, 4, false, false, MODE_BF16, false, false, false, true>), grid, block, 0, dev->stream, p);
+            if (c) hipLaunchKernelGGL((attn_fwd_kernel<128, 8, true, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
+            else hipLaunchKernelGGL((attn_fwd_kernel<128, 8, false, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
         }
     } else if (D == 64) {
         if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
