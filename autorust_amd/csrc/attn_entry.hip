@@ -14,6 +14,7 @@
 //   ar_flash_f32        [256,1,1]  [ceil(n/128), B*hq, 1]    fp32 exact (cuda_flash.rs)
 //   ar_flash_bf16       [256,1,1]  [ceil(n/128), B*hq, 1]    bf16 (cuda_flash_bf16.rs), any mask
 //   ar_flash_bf16_long  [512,1,1]  [ceil(n/256), B*hq, 1]    bf16 pipelined, has_mask must be 0
+//   ar_flash_bf16_short [512,1,1]  [ceil(n/128), B*hq, 1]    bf16, n <= 256, has_mask must be 0
 //   ar_flash_sage       [256,1,1]  [ceil(n/128), B*hq, 1]    int8 (cuda_flash_sage.rs), any mask, any
 //                                                            block sizes incl. per-row scales; O f32
 //   ar_flash_sage_long  [512,1,1]  [ceil(n/256), B*hq, 1]    int8 pipelined: has_mask 0, bk = 64 * 2^n
@@ -196,6 +197,25 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16(const uint16_t *
     if (head_dim == 64) AR_BF16(64);
     else if (head_dim == 128) AR_BF16(128);
 #undef AR_BF16
+}
+
+// sequences of at most 256 keys: all of K/V of the head in LDS at once, 8 waves (two per 32 queries on
+// the even / odd key tiles).  has_mask must be 0 and N <= 256; anything else returns without writing.
+extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_short(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                       uint16_t *O, const float *M, int N, int head_dim,
+                                                                       int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 8, MODE_BF16, false, true>()];
+    if (has_mask || N > 256) return;
+    AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, 0, hq, hkv);
+    const int wg = linear_wg();
+    if (head_dim == 64) {
+        if (causal) attn_fwd_body<64, 8, true, false, MODE_BF16, false, false, false, true, 2>(p, lds, wg);
+        else attn_fwd_body<64, 8, false, false, MODE_BF16, false, false, false, true, 2>(p, lds, wg);
+    } else if (head_dim == 128) {
+        if (causal) attn_fwd_body<128, 8, true, false, MODE_BF16, false, false, false, true, 2>(p, lds, wg);
+        else attn_fwd_body<128, 8, false, false, MODE_BF16, false, false, false, true, 2>(p, lds, wg);
+    }
 }
 
 extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long(const uint16_t *Q, const uint16_t *K, const uint16_t *V,

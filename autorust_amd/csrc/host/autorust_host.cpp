@@ -393,7 +393,10 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
         return calls;
     }
     if (kern == Kernel::FlashBf16) {
-        if (!has_mask && long_variant(dev, b, h, n, d))
+        if (!has_mask && n <= 256 && b * h * ((n + 127) / 128) <= 4 * (int64_t)dev->compute_units())
+            calls.push_back(make_call(dev, "ar_flash_bf16_short", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
+                                      {(n + 127) / 128, b * h, 1}, {512, 1, 1}, vals));
+        else if (!has_mask && long_variant(dev, b, h, n, d))
             calls.push_back(make_call(dev, "ar_flash_bf16_long", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 255) / 256, b * h, 1}, {512, 1, 1}, vals));
         else

@@ -48,6 +48,9 @@
 /* the software-pipelined variant for long sequences: same arguments, has_mask must be 0,
  * (N + 320) * head_dim * 2 < 2^31; long tiling. */
 #define ARHIP_KERNEL_FLASH_BF16_LONG "ar_flash_bf16_long"
+/* the variant for sequences of at most 256 keys (all of K/V of a head in LDS at once): same
+ * arguments, has_mask must be 0, N <= 256; block [512,1,1], grid [ceil(N/128), B*hq, 1]. */
+#define ARHIP_KERNEL_FLASH_BF16_SHORT "ar_flash_bf16_short"
 
 /* Sage int8: replaces `ar_flash_sage`, src/runtime/cuda_flash_sage.rs:168-414, on pre-quantised
  * operands (the quantiser is the pre-pass below):

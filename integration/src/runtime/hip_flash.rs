@@ -134,7 +134,10 @@ pub fn host_call_f32(bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Op
 /// bf16: `bufs = [q, k, v, o, mask-or-o]`, q/k/v/o bf16, mask f32 `[n, n]`.
 pub fn host_call_bf16(dev: &str, bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
     let (bf, f) = (dtype::BFLOAT16, dtype::FLOAT32);
-    if !opts.has_mask && long_variant(dev, b, h, n, d) {
+    if !opts.has_mask && n <= 256 && b * h * ((n + 127) / 128) <= 4 * crate::runtime::ops_hip::compute_units(dev) {
+        // all of K/V of a head in LDS at once: the ViT sequence lengths
+        call("ar_flash_bf16_short", bufs, &[bf, bf, bf, bf, f], [(n + 127) / 128, b * h, 1], [512, 1, 1], vals(n, d, h, opts), &[])
+    } else if !opts.has_mask && long_variant(dev, b, h, n, d) {
         call("ar_flash_bf16_long", bufs, &[bf, bf, bf, bf, f], [(n + 255) / 256, b * h, 1], [512, 1, 1], vals(n, d, h, opts), &[])
     } else {
         call("ar_flash_bf16", bufs, &[bf, bf, bf, bf, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])

@@ -221,3 +221,19 @@ def test_ar_flash_sage_fp8_by_name(dev, kernels):
     assert np.array_equal(h_q8, w_q8) and np.array_equal(h_sq, w_sq) and np.array_equal(h_k8, w_k8) and np.array_equal(h_sk, w_sk)
     want = oracle.sage_fp8(w_q8, w_k8, w_sq, w_sk, v, bq, bk, causal=True)
     assert np.abs(got - want).max() < 2e-3
+
+
+@pytest.mark.parametrize("n,d,causal,hkv", [(197, 64, False, 6), (256, 128, True, 3), (1, 64, False, 6), (130, 128, False, 1)])
+def test_ar_flash_bf16_short_by_name(dev, kernels, n, d, causal, hkv):
+    """The variant for sequences of at most 256 keys (8 waves, two per 32 queries on the even / odd
+    key tiles), at the ViT length among others."""
+    b, hq = 2, 6
+    q, k, v = fill_qkv(b, hq, hkv, n, d)
+    with Bufs(dev) as bufs:
+        dq, dk, dv = (bufs.put(synth.to_bf16_bits(t)) for t in (q, k, v))
+        do = bufs.new(q.size * 2)
+        dev.launch(kernels, "ar_flash_bf16_short", _grid(n, 128, b, hq), (512, 1, 1), [dq, dk, dv, do, do],
+                   [n, d, int(causal), 0, hq, hkv])
+        got = synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+    want = oracle.attn_bf16(q, k, v, causal=causal)
+    assert np.abs(got - want).max() < 5e-3

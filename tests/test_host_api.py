@@ -252,6 +252,22 @@ def test_attention_debug_line_and_kernel_info(hdev, capfd, monkeypatch):
 
 
 @gpu
+def test_short_sequences_take_the_short_kernel(hdev):
+    """ViT-B/16's sequence length through the host API: the dispatcher's HostCall names the
+    short-sequence entry (all of K/V of a head in LDS at once)."""
+    b, h, n, d = 2, 12, 197, 64
+    q, k, v = (synth.normal(710 + i, (b, h, n, d)) for i in range(3))
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape, BFLOAT16) for a in (q, k, v))
+    sess = Session()
+    sess.begin_capture()
+    out = tq.attention_with(tk, tv, None, 0.0, False, sess)
+    assert sess.end_capture() == 1
+    name, grid, vals = sess.step(0)
+    assert name == "ar_flash_bf16_short" and grid == [2, b * h, 1] and sess.step_detail(0)[1] == [512, 1, 1]
+    assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v)).max()) < 2e-2
+
+
+@gpu
 def test_capture_and_replay(hdev):
     """Session::capture_host + Jit replay (session.rs:138-146, jit.rs:186-195): the captured launch
     re-runs on the same buffers and reproduces the result; the allocator serves repeats from its
