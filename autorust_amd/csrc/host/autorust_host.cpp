@@ -366,11 +366,12 @@ HostCall make_call(const std::shared_ptr<Device> &dev, const char *name, const s
     return c;
 }
 
-// The pipelined kernels want enough workgroups of 256 queries to fill the chip twice and address
-// K/V with 32-bit byte offsets.
+// The pipelined kernels want enough workgroups of 256 queries to fill the chip twice (or, from 8
+// tiles per workgroup on, half of it once) and address K/V with 32-bit byte offsets.
 bool long_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int64_t n, int64_t d)
 {
-    return b * h * ((n + 255) / 256) >= 2 * (int64_t)dev->compute_units() && (n + 320) * d * 2 < ((int64_t)1 << 31);
+    const int64_t cus = dev->compute_units(), wgs = b * h * ((n + 255) / 256);
+    return (wgs >= 2 * cus || (n >= 512 && 2 * wgs >= cus)) && (n + 320) * d * 2 < ((int64_t)1 << 31);
 }
 
 }  // namespace

@@ -118,11 +118,12 @@ fn vals(n: i64, d: i64, h: i64, opts: Options) -> Vec<i64> {
     vec![n, d, opts.causal as i64, opts.has_mask as i64, h, opts.h_kv]
 }
 
-/// The pipelined kernels want enough workgroups of 256 queries to fill the chip twice and
-/// address K/V with 32-bit byte offsets.
+/// The pipelined kernels want enough workgroups of 256 queries to fill the chip twice (or, from 8
+/// tiles per workgroup on, half of it once) and address K/V with 32-bit byte offsets.
 fn long_variant(dev: &str, b: i64, h: i64, n: i64, d: i64) -> bool {
     let cus = crate::runtime::ops_hip::compute_units(dev);
-    b * h * ((n + 255) / 256) >= 2 * cus && (n + 320) * d * 2 < 1 << 31
+    let wgs = b * h * ((n + 255) / 256);
+    (wgs >= 2 * cus || (n >= 512 && 2 * wgs >= cus)) && (n + 320) * d * 2 < 1 << 31
 }
 
 /// fp32 exact mode: `bufs = [q, k, v, o, mask-or-o]`, all f32 `[b, h, n, d]`.
