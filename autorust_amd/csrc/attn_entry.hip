@@ -18,6 +18,7 @@
 //   ar_flash_sage       [256,1,1]  [ceil(n/128), B*hq, 1]    int8 (cuda_flash_sage.rs), any mask, any
 //                                                            block sizes incl. per-row scales; O f32
 //   ar_flash_sage_long  [512,1,1]  [ceil(n/256), B*hq, 1]    int8 pipelined: has_mask 0, bk = 64 * 2^n
+//   ar_flash_sage_fp8_long  the same on E4M3 codes
 // The Sage entries take pre-quantised operands (the quantiser is the pre-pass below, not part of
 // the attention kernel as in the reference):
 //     (Q8, K8, V, O, M, SQ, SK,  N, head_dim, causal, has_mask, hq, hkv, bq, bk [, out_f32])
@@ -293,15 +294,15 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_fp8(const uint8_
     flash_sage_entry<MODE_FP8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
 }
 
-extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
-                                                                      void *O, const float *M, const float *SQ, const float *SK,
-                                                                      int N, int head_dim, int causal, int has_mask, int hq,
-                                                                      int hkv, int bq, int bk, int out_f32)
+// ar_flash_sage_long / ar_flash_sage_fp8_long: the pipelined kernel on pre-quantised operands
+template <int QMODE>
+__device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const void *Q8, const void *K8, const uint16_t *V, void *O,
+                                                      const float *M, const float *SQ, const float *SK, int N, int head_dim,
+                                                      int causal, int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8>()];
     int shift = 0;
     while ((64 << shift) < bk) ++shift;
-    if (has_mask || (64 << shift) != bk) return;  // ar_flash_sage covers those
+    if (has_mask || (64 << shift) != bk) return;  // the general kernels cover those
     AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, 0, hq, hkv);
     p.sq = SQ; p.sk = SK;
     p.bq = bq; p.bk = bk;
@@ -310,16 +311,34 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_
 #define AR_SAGE_LONG(DD)                                                                  \
     do {                                                                                  \
         if (out_f32) {                                                                    \
-            if (causal) attn_pipe_body<DD, true, MODE_I8, true>(p, lds, wg);              \
-            else attn_pipe_body<DD, false, MODE_I8, true>(p, lds, wg);                    \
+            if (causal) attn_pipe_body<DD, true, QMODE, true>(p, lds, wg);                \
+            else attn_pipe_body<DD, false, QMODE, true>(p, lds, wg);                      \
         } else {                                                                          \
-            if (causal) attn_pipe_body<DD, true, MODE_I8, false>(p, lds, wg);             \
-            else attn_pipe_body<DD, false, MODE_I8, false>(p, lds, wg);                   \
+            if (causal) attn_pipe_body<DD, true, QMODE, false>(p, lds, wg);               \
+            else attn_pipe_body<DD, false, QMODE, false>(p, lds, wg);                     \
         }                                                                                 \
     } while (0)
     if (head_dim == 64) AR_SAGE_LONG(64);
     else if (head_dim == 128) AR_SAGE_LONG(128);
 #undef AR_SAGE_LONG
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
+                                                                      void *O, const float *M, const float *SQ, const float *SK,
+                                                                      int N, int head_dim, int causal, int has_mask, int hq,
+                                                                      int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8>()];
+    flash_sage_long_entry<MODE_I8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
+                                                                          void *O, const float *M, const float *SQ, const float *SK,
+                                                                          int N, int head_dim, int causal, int has_mask, int hq,
+                                                                          int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8>()];
+    flash_sage_long_entry<MODE_FP8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
 // ---- Sage pre-pass (the quantiser the reference runs inside its attention kernel,

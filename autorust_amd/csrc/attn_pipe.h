@@ -61,7 +61,7 @@ __device__ __forceinline__ void static_for(F &&f)
 template <int D, int MODE>
 constexpr int attn_pipe_lds_bytes()
 {
-    return 4 * 4096 * (D * ((MODE == MODE_I8) ? 1 : 2) / 64 + D * 2 / 64);
+    return 4 * 4096 * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64 + D * 2 / 64);
 }
 
 // The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
@@ -71,7 +71,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
 {
     constexpr int NW = 8;
     constexpr int BQ = NW * 32;
-    constexpr int QK_BYTES = (MODE == MODE_I8) ? 1 : 2;
+    constexpr int QK_BYTES = (MODE != MODE_BF16) ? 1 : 2;
     constexpr int KP = D * QK_BYTES / 64;  // 64-byte pieces per K row
     constexpr int VP = D * 2 / 64;         // 64-byte pieces per V row
     constexpr int K_TILE = KP * 4096;      // [piece][64 rows][64 B]
@@ -81,7 +81,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     constexpr int XFERS = (KP + VP) * 4;          // 1 KB transfers per tile
     constexpr int XPW = (XFERS + NW - 1) / NW;    // at most this many per wave
     constexpr int XPW_MIN = XFERS / NW;           // at least this many per wave
-    constexpr int KSTEPS = (MODE == MODE_I8) ? D / 32 : D / 16;
+    constexpr int KSTEPS = (MODE != MODE_BF16) ? D / 32 : D / 16;
     constexpr int DB = D / 32;
     static_assert(KP >= 1 && XFERS >= NW, "tile too small for 8 waves");
 
@@ -210,8 +210,8 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     float m_run = NEG_SENTINEL;
     float l_run = 0.f;
     float sq_lane = 1.f;
-    const int nkb = (MODE == MODE_I8) ? (N + p.bk - 1) / p.bk : 0;
-    if (MODE == MODE_I8) {
+    const int nkb = (MODE != MODE_BF16) ? (N + p.bk - 1) / p.bk : 0;
+    if (MODE != MODE_BF16) {
         const int nqb = (N + p.bq - 1) / p.bq;
         sq_lane = p.sq[(size_t)bh * nqb + min(q_row, N - 1) / p.bq];
     }
@@ -229,7 +229,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     // exponent factor of the keys of tile t (in the group of tile `it` or the next one): scale log2(e),
     // times sq sk for int8 (s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322)
     auto tile_c = [&](int t, int it) __attribute__((always_inline)) -> float {
-        if constexpr (MODE == MODE_I8) {
+        if constexpr (MODE != MODE_BF16) {
             const int a = __builtin_amdgcn_readlane(__float_as_int(skv_cur), t & 63);
             const int bnext = __builtin_amdgcn_readlane(__float_as_int(skv_nxt), t & 63);
             const float f = __int_as_float(((t >> 6) == (it >> 6)) ? a : bnext);
@@ -242,7 +242,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     // wait makes the new vector's arrival explicit (once per 64 tiles) so that no wait for it is
     // left at its uses.
     auto advance_sk_group = [&](int it) __attribute__((always_inline)) {
-        if constexpr (MODE == MODE_I8) {
+        if constexpr (MODE != MODE_BF16) {
             if ((it & 63) == 0 && it > 0) {
                 skv_cur = skv_nxt;
                 skv_nxt = load_sk_group((it >> 6) + 1);
@@ -267,17 +267,37 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
                 vf[db][ks][1] = lds_read_tr16(st + v_addr[1] + db * 4096 + (blk * 2 + ks) * 1024);
             }
     };
+    // One step of S^T += K-fragment . Q-fragment.  int8: v_mfma_i32_32x32x32_i8 on the 16-byte
+    // fragments of step st.  FP8 (E4M3): the same fragments, two steps at a time, on
+    // v_mfma_f32_32x32x64_f8f6f4 (32 bytes per lane, the int8 rate): the call for an even step does
+    // nothing, the call for the odd step multiplies the fragments of both (the contraction order is
+    // free as long as Q and K agree).  bf16: v_mfma_f32_32x32x16_bf16.
+    auto qk_step = [&](auto si, acc_t &acc, const uint4 &a_prev, const uint4 &a, const uint4 &b_prev, const uint4 &b)
+                       __attribute__((always_inline)) {
+        constexpr int st = decltype(si)::value;
+        if constexpr (MODE == MODE_I8) {
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a), __builtin_bit_cast(i32x4, b), acc, 0, 0, 0);
+        } else if constexpr (MODE == MODE_FP8) {
+            if constexpr (st % 2 == 1) {
+                typedef __attribute__((ext_vector_type(8))) int i32x8;
+                const i32x8 av = {(int)a_prev.x, (int)a_prev.y, (int)a_prev.z, (int)a_prev.w, (int)a.x, (int)a.y, (int)a.z, (int)a.w};
+                const i32x8 bv = {(int)b_prev.x, (int)b_prev.y, (int)b_prev.z, (int)b_prev.w, (int)b.x, (int)b.y, (int)b.z, (int)b.w};
+                acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 0, 0, 0, 0, 0, 0);
+            }
+        } else {
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+        }
+    };
+    static_assert(MODE != MODE_FP8 || KSTEPS % 2 == 0, "FP8 steps come in pairs");
     auto mfma_qk = [&]() __attribute__((always_inline)) -> acc_t {
         acc_t s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0;
-#pragma unroll
-        for (int st = 0; st < KSTEPS; ++st) {
-            if constexpr (MODE == MODE_I8)
-                s = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kf[st]), __builtin_bit_cast(i32x4, qreg[st]), s, 0, 0, 0);
-            else
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s, 0, 0, 0);
-        }
+        static_for<0, KSTEPS>([&](auto si) __attribute__((always_inline)) {
+            constexpr int st = decltype(si)::value;
+            constexpr int pv = st > 0 ? st - 1 : 0;
+            qk_step(si, s, kf[pv], kf[st], qreg[pv], qreg[st]);
+        });
         return s;
     };
     auto move_reference = [&](float mx) __attribute__((always_inline)) {
@@ -318,14 +338,14 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         acc_t s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0;
+        uint4 kt[KSTEPS];
 #pragma unroll
-        for (int q = 0; q < KSTEPS; ++q) {
-            const uint4 kt = *(const uint4 *)(st + k_addr[q & 1] + (q >> 1) * 4096 + blk * 2048);
-            if constexpr (MODE == MODE_I8)
-                s = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kt), __builtin_bit_cast(i32x4, qreg[q]), s, 0, 0, 0);
-            else
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kt), __builtin_bit_cast(bf16x8, qreg[q]), s, 0, 0, 0);
-        }
+        for (int q = 0; q < KSTEPS; ++q) kt[q] = *(const uint4 *)(st + k_addr[q & 1] + (q >> 1) * 4096 + blk * 2048);
+        static_for<0, KSTEPS>([&](auto qi) __attribute__((always_inline)) {
+            constexpr int q = decltype(qi)::value;
+            constexpr int pv = q > 0 ? q - 1 : 0;
+            qk_step(qi, s, kt[pv], kt[q], qreg[pv], qreg[q]);
+        });
         // max3 is inline assembly, which the compiler leaves out when it pads the distance between a
         // matrix instruction and the first vector read of its result: the scaled copies below are
         // ordinary vector instructions, so the result has landed by the time max3 runs
@@ -416,7 +436,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     // the wave issues in order.  Past the last pipelined block the look-ahead works on whatever
     // the next LDS stage holds; those results are never used.
     constexpr int R2_SLOTS = DB * 2 - 2;  // S is not ready under the first two O^T MFMAs
-    constexpr int SM_SPLIT = (MODE == MODE_I8) ? (SM_OPS * R2_SLOTS) / (R2_SLOTS + KSTEPS) : SM_HALF;
+    constexpr int SM_SPLIT = (MODE != MODE_BF16) ? (SM_OPS * R2_SLOTS) / (R2_SLOTS + KSTEPS) : SM_HALF;
     // mc / mn: block j / block j+1 has masked keys (causal diagonal, key-length edge); rel_cur /
     // rel_next are their mask offsets (see lim4h).
     auto pipe_block = [&](auto mc, auto mn, acc_t &s_old, acc_t &s_new, uint4 (&p_cur)[2], uint4 (&p_nxt)[2],
@@ -429,14 +449,20 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         ARHIP_FENCE();
         static_for<0, KSTEPS>([&](auto si) __attribute__((always_inline)) {
             constexpr int st = decltype(si)::value;
-            if constexpr (MODE == MODE_I8)
-                s_new = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, kf[st]), __builtin_bit_cast(i32x4, qreg[st]), s_new, 0, 0, 0);
-            else
-                s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[st]), __builtin_bit_cast(bf16x8, qreg[st]), s_new, 0, 0, 0);
+            constexpr int pv = st > 0 ? st - 1 : 0;
+            qk_step(si, s_new, kf[pv], kf[st], qreg[pv], qreg[st]);
             ARHIP_FENCE();
             constexpr int lo = SM_SPLIT + st * (SM_OPS - SM_SPLIT) / KSTEPS, hi = SM_SPLIT + (st + 1) * (SM_OPS - SM_SPLIT) / KSTEPS;
             static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mc, ic, s_old, c_cur, rel_cur, p_cur); });
-            kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
+            // refill behind the MFMA that read the fragment (FP8: behind the odd step, both halves)
+            if constexpr (MODE == MODE_FP8) {
+                if constexpr (st % 2 == 1) {
+                    kf[st - 1] = *(const uint4 *)(sk + k_addr[(st - 1) & 1] + ((st - 1) >> 1) * 4096 + kb * 2048);
+                    kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
+                }
+            } else {
+                kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
+            }
             ARHIP_FENCE();
         });
         rs = sm_half[0] + sm_half[1];
@@ -484,7 +510,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         for (int s = 0; s < KSTEPS; ++s) qreg[s] = *(const uint4 *)(qb + s * 32 + h * 16);
     }
 
-    if constexpr (MODE == MODE_I8) {
+    if constexpr (MODE != MODE_BF16) {
         skv_cur = load_sk_group(0);
         skv_nxt = load_sk_group(1);
     }

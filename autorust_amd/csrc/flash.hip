@@ -293,7 +293,7 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
     while (((int64_t)64 << shift) < bk) ++shift;
     const bool per_key = ((int64_t)64 << shift) != bk;
     p.bk_tile_shift = shift;
-    int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg || fp8);   // FP8 runs on the general kernel
+    int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg);
     if (nw == 1) nw = 4;
     if (nw == 8 && !pipe_addressable(N, std::max<int64_t>(D, v_strides ? v_strides[2] : D), 2)) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
@@ -329,7 +329,10 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
         if (f32o) launch_attn<DD, 4, MODE_FP8, PK, true, false, true>(dev->stream, p, c, hm);          \
         else launch_attn<DD, 4, MODE_FP8, PK, false, false, true>(dev->stream, p, c, hm);              \
     } while (0)
-    if (fp8) {
+    if (fp8 && nw == 8 && !per_key) {
+        if (D == 64) { if (f32o) launch_pipe<64, MODE_FP8, true>(dev->stream, p, c); else launch_pipe<64, MODE_FP8, false>(dev->stream, p, c); }
+        else { if (f32o) launch_pipe<128, MODE_FP8, true>(dev->stream, p, c); else launch_pipe<128, MODE_FP8, false>(dev->stream, p, c); }
+    } else if (fp8) {
         if (D == 64) { if (per_key) SAGE_F(64, true); else SAGE_F(64, false); }
         else { if (per_key) SAGE_F(128, true); else SAGE_F(128, false); }
     } else if (D == 64) SAGE_D(64);

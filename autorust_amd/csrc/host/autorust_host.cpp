@@ -452,9 +452,9 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     int shift = 0;
     while (((int64_t)64 << shift) < bk) ++shift;
     const bool tile_uniform = ((int64_t)64 << shift) == bk;
-    if (!st.sage_fp8 && !has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
+    if (!has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
         svals.push_back(bf16_in ? 0 : 1);  // out_f32
-        calls.push_back(make_call(dev, "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
+        calls.push_back(make_call(dev, st.sage_fp8 ? "ar_flash_sage_fp8_long" : "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
                                   {(n + 255) / 256, b * h, 1}, {512, 1, 1}, svals));
     } else if (!bf16_in) {
         calls.push_back(make_call(dev, general, {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, F, F, F, F},

@@ -29,7 +29,7 @@ from autorust_amd.device import BF16, F32, Device  # noqa: E402
 
 PEAK_BF16 = 2500.0   # TFLOP/s, MI355X dense bf16 MFMA
 PEAK_F32 = 157.3     # TFLOP/s, MI355X dense fp32 MFMA
-PEAK_INT8 = 5000.0   # TOP/s, MI355X dense int8 MFMA
+PEAK_INT8 = 5000.0   # TOP/s, MI355X dense int8 MFMA (dense fp8 MFMA: the same 5000 TFLOP/s)
 PEAK_HBM = 8000.0    # GB/s, MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
@@ -49,13 +49,14 @@ class SageWorkload:
     """SageAttention INT8 forward: Q ~ N(0,1), K = N(0,1) + per-(head,channel) bias ~ N(0, sigma),
     V ~ N(0,1); all three stored as bf16; O bf16."""
 
-    def __init__(self, dev, B, H, S, D, causal, sigma, outliers, cfg, bq=128, bk=64, f32_io=False):
+    def __init__(self, dev, B, H, S, D, causal, sigma, outliers, cfg, bq=128, bk=64, f32_io=False, fp8=False):
         self.dev, self.B, self.H, self.S, self.D, self.causal = dev, B, H, S, D, causal
         self.bq, self.bk = bq, bk
+        self.fp8 = fp8  # E4M3 codes instead of int8 (the reference's AR_FP8 build of the same kernel)
         # f32_io: the reference's own convention (f32 tensors in, f32 out, per-row scales, no smoothing)
         self.f32_io = f32_io
-        self.name = "sage_int8_b%d_h%d_s%d_d%d%s%s" % (B, H, S, D, "_causal" if causal else "",
-                                                        "_f32io_rowscales" if f32_io else "")
+        self.name = "sage_%s_b%d_h%d_s%d_d%d%s%s" % ("fp8" if fp8 else "int8", B, H, S, D, "_causal" if causal else "",
+                                                      "_f32io_rowscales" if f32_io else "")
         n = B * H * S * D
         base = 1000 * cfg
         q = synth.normal(base + 1, (B, H, S, D))
@@ -90,11 +91,18 @@ class SageWorkload:
         self.kernel = _lib.K_SAGE
         # dominant kernel: int8 Q, K (1 B), bf16 V and O (2 B), block scales
         self.kernel_bytes = n * (1 + 1 + 2 + 2) + 4 * B * H * (S // bq + S // bk)
-        self.dtype = "int8"
+        self.dtype = "fp8" if fp8 else "int8"
 
     def step(self):
         d, B, H, S, D = self.dev, self.B, self.H, self.S, self.D
         io = F32 if self.f32_io else BF16
+        if self.fp8:
+            d.sage_quant_fp8(self.dq, self.q8, self.sq, B, H, S, D, self.bq, io, wait=False)
+            d.sage_quant_fp8(self.dk, self.k8, self.sk, B, H, S, D, self.bk, io, mean=self.mean, workspace=self.ws,
+                             smooth=True, wait=False)
+            d.sage_fwd_fp8(self.q8, self.k8, self.sq, self.sk, self.dv, self.do, B, H, H, S, D, self.bq, self.bk,
+                           out_dtype=io, causal=self.causal, wait=False)
+            return
         d.sage_quant(self.dq, self.q8, self.sq, B, H, S, D, self.bq, io, wait=False)
         d.sage_quant(self.dk, self.k8, self.sk, B, H, S, D, self.bk, io, mean=self.mean, workspace=self.ws,
                      smooth=not self.f32_io, wait=False)
@@ -109,8 +117,8 @@ class SageWorkload:
         ach = self.ops / secs / 1e12
         return {"bound": "mfma", "achieved": ach, "peak": PEAK_INT8, "unit": "TOP/s", "frac": ach / PEAK_INT8,
                 "traffic": MEASURED_TRAFFIC.get(self.name), "traffic_source": "rocprofv3 --pmc profile (profiles/), not this run",
-                "kernel": "attn_fwd_kernel<int8>" if self.bk == 1 else "attn_pipe_kernel<int8>", "launch_ms": secs * 1e3,
-                "ops_per_launch": self.ops, "peak_note": "dense int8 MFMA; half of the ops are bf16 (P.V)",
+                "kernel": "attn_fwd_kernel<int8>" if self.bk == 1 else "attn_pipe_kernel<%s>" % self.dtype, "launch_ms": secs * 1e3,
+                "ops_per_launch": self.ops, "peak_note": "dense %s MFMA; half of the ops are bf16 (P.V)" % self.dtype,
                 "frac_of_mixed_int8_bf16_bound": t_min / secs}
 
     def free(self):
@@ -328,6 +336,8 @@ def build_workload(dev, name):
         return SageWorkload(dev, 4, 32, 8192, 128, False, 3.0, 0.0, cfg=4)
     if name == "sage_causal_long":
         return SageWorkload(dev, 1, 64, 32768, 128, True, 5.0, 0.01, cfg=5)
+    if name == "sage_fp8":   # the headline shape on E4M3 codes
+        return SageWorkload(dev, 4, 32, 8192, 128, False, 3.0, 0.0, cfg=4, fp8=True)
     if name == "vit":
         return FlashWorkload(dev, 8, 12, 197, 64, False, BF16, cfg=2)
     if name == "flash_long":
@@ -360,7 +370,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="sage",
                     choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32", "flash_long", "ref_bf16",
-                             "ref_f32", "ref_sage", "train_f32"])
+                             "ref_f32", "ref_sage", "train_f32", "sage_fp8"])
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="one step of the workload plus one plain 1 GiB copy kernel and nothing else: "
@@ -402,7 +412,7 @@ def main():
     secondary = []
     if not args.no_secondary:
         for name in ("vit", "decoder", "flash_long", "vit_f32", "sage", "sage_causal_long", "ref_bf16", "ref_f32",
-                     "ref_sage", "train_f32"):
+                     "ref_sage", "train_f32", "sage_fp8"):
             if name == args.workload:
                 continue
             sw = build_workload(dev, name)
@@ -419,13 +429,13 @@ def main():
 
     line = {
         "metric": "attention fwd TFLOPS/TOPS + % MFMA peak, ViT-B/16 and S=8192 D=128 shapes",
-        "value": res["tops"], "unit": "TOP/s" if w.dtype == "int8" else "TFLOP/s",
+        "value": res["tops"], "unit": "TOP/s" if w.dtype in ("int8", "fp8") else "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": res["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic",
         "config": {"workload": w.name, "B": w.B, "H": w.H, "S": w.S, "D": w.D, "causal": bool(w.causal),
-                   "step": "quantise Q (128-token blocks) + smooth and quantise K (64-token blocks) + int8 attention"
-                           if w.dtype == "int8" else "attention forward"},
+                   "step": "quantise Q (128-token blocks) + smooth and quantise K (64-token blocks) + %s attention" % w.dtype
+                           if w.dtype in ("int8", "fp8") else "attention forward"},
         "roofline": res["roofline"],
         "cpu_baseline": cpu,
     }
@@ -436,7 +446,7 @@ def main():
         line["power_limit_probe"] = {"kernel": "probe_mfma_rate (bf16 32x32x16 MFMAs only, 2 waves per SIMD)",
                                      "constant_operands": power["constant"], "random_operands": power["random"]}
         line["roofline"]["frac_of_sustained_bf16_mfma_rate"] = (
-            (res["ops_per_step"] / 2 / (PEAK_INT8 / PEAK_BF16) + res["ops_per_step"] / 2) if w.dtype == "int8"
+            (res["ops_per_step"] / 2 / (PEAK_INT8 / PEAK_BF16) + res["ops_per_step"] / 2) if w.dtype in ("int8", "fp8")
             else res["ops_per_step"]) / (line["roofline"]["launch_ms"] * 1e-3) / 1e12 / power["random"]["tflops"]
     if "ms_per_step_graph_replay" in res:
         line["ms_per_step_graph_replay"] = res["ms_per_step_graph_replay"]

@@ -90,6 +90,7 @@
  * the same argument lists as ar_flash_sage / ar_sage_quant_{blocks,rows}_*, with E4M3 codes
  * (scale = absmax / 448) in place of int8 values. */
 #define ARHIP_KERNEL_FLASH_SAGE_FP8 "ar_flash_sage_fp8"
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_LONG "ar_flash_sage_fp8_long"   /* as ar_flash_sage_long */
 #define ARHIP_KERNEL_SAGE_QUANT_BLOCKS_FP8_F32 "ar_sage_quant_blocks_fp8_f32"
 #define ARHIP_KERNEL_SAGE_QUANT_BLOCKS_FP8_BF16 "ar_sage_quant_blocks_fp8_bf16"
 #define ARHIP_KERNEL_SAGE_QUANT_ROWS_FP8_F32 "ar_sage_quant_rows_fp8_f32"

@@ -14,6 +14,7 @@
 //! | `ar_flash_bf16_long` | 512   | `[ceil(n/256), b*h, 1]` | same (`has_mask` must be 0)                  |
 //! | `ar_flash_sage`      | 256   | `[ceil(n/128), b*h, 1]` | same `+ bq, bk`; buffers `+ SQ, SK`; O is f32|
 //! | `ar_flash_sage_long` | 512   | `[ceil(n/256), b*h, 1]` | same `+ bq, bk, out_f32`                     |
+//! | `ar_flash_sage_fp8`, `ar_flash_sage_fp8_long` | as the int8 pair, on E4M3 codes (`SageOptions::fp8`)        |
 //!
 //! Unlike the CUDA Sage kernel, which quantises inside the attention kernel (K once per query
 //! block, `cuda_flash_sage.rs:248-278`), the quantiser is a pre-pass of its own here, with K
@@ -51,11 +52,13 @@ pub struct SageOptions {
     pub block_q: i64,
     pub block_k: i64,
     pub smooth_k: bool,
+    /// E4M3 codes instead of int8 (the CUDA source's `fp8` flag, `cuda_flash_sage.rs:82-84`).
+    pub fp8: bool,
 }
 
 impl Default for SageOptions {
     fn default() -> Self {
-        SageOptions { block_q: 128, block_k: 64, smooth_k: true }
+        SageOptions { block_q: 128, block_k: 64, smooth_k: true, fp8: false }
     }
 }
 
@@ -180,6 +183,8 @@ pub fn host_calls_sage(
     let (f, bf, i8t) = (dtype::FLOAT32, dtype::BFLOAT16, dtype::INT8);
     let x = if bf16_in { bf } else { f };
     let sfx = if bf16_in { "bf16" } else { "f32" };
+    let q8fmt = if sage.fp8 { "fp8_" } else { "" };
+    let (general, long) = if sage.fp8 { ("ar_flash_sage_fp8", "ar_flash_sage_fp8_long") } else { ("ar_flash_sage", "ar_flash_sage_long") };
     let hk = opts.h_kv;
     let (bq, bk) = (sage.block_q, sage.block_k);
     let (nqb, nkb, nchunk) = ((n + bq - 1) / bq, (n + bk - 1) / bk, (n + 63) / 64);
@@ -189,10 +194,10 @@ pub fn host_calls_sage(
         if blk == 1 {
             let rows = b * heads * n;
             let rpb = 256 / (d / 8);
-            calls.push(call(&format!("ar_sage_quant_rows_{sfx}"), bufs, &[x, i8t, f, f], [(rows + rpb - 1) / rpb, 1, 1], [256, 1, 1],
+            calls.push(call(&format!("ar_sage_quant_rows_{q8fmt}{sfx}"), bufs, &[x, i8t, f, f], [(rows + rpb - 1) / rpb, 1, 1], [256, 1, 1],
                             vec![n, d, rows, smooth as i64], &[2]));
         } else {
-            calls.push(call(&format!("ar_sage_quant_blocks_{sfx}"), bufs, &[x, i8t, f, f], [nblk, b * heads, 1], [256, 1, 1],
+            calls.push(call(&format!("ar_sage_quant_blocks_{q8fmt}{sfx}"), bufs, &[x, i8t, f, f], [nblk, b * heads, 1], [256, 1, 1],
                             vec![n, d, blk, nblk, smooth as i64], &[]));
         }
     };
@@ -220,17 +225,17 @@ pub fn host_calls_sage(
     let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
     if !opts.has_mask && tile_uniform && long_variant(dev, b, h, n, d) {
         sv.push(!bf16_in as i64); // out_f32
-        calls.push(call("ar_flash_sage_long", vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f],
+        calls.push(call(long, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f],
                         [(n + 255) / 256, b * h, 1], [512, 1, 1], sv, &[]));
     } else if !bf16_in {
-        calls.push(call("ar_flash_sage", vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f],
+        calls.push(call(general, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f],
                         [(n + 127) / 128, b * h, 1], [256, 1, 1], sv, &[]));
     } else {
         // the general kernel stores f32 (the CUDA kernel's convention); bf16 tensors get their
         // bf16 result through one more cast
         let o32 = s.o32.expect("o32 scratch for bf16 tensors");
         let m2 = if opts.has_mask { mask } else { o32.clone() };
-        calls.push(call("ar_flash_sage", vec![s.q8, s.k8, vb, o32.clone(), m2, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f],
+        calls.push(call(general, vec![s.q8, s.k8, vb, o32.clone(), m2, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f],
                         [(n + 127) / 128, b * h, 1], [256, 1, 1], sv, &[]));
         let no = b * h * n * d;
         calls.push(call("ar_cast_bf16", vec![o32, o], &[f, bf], [((no + 255) / 256).min(16384), 1, 1], [256, 1, 1], vec![no], &[0]));

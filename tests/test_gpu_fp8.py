@@ -81,6 +81,34 @@ def test_fp8_attention_matches_emulation(dev, bq, bk, smooth, in_dtype, causal, 
     assert np.abs(out - want).max() < 2e-3
 
 
+@pytest.mark.parametrize("d,bk", [(128, 64), (64, 128)])
+@pytest.mark.parametrize("causal,use_len", [(False, False), (True, False), (True, True), (False, True)])
+def test_fp8_long_sequence_kernel_matches_emulation(dev, d, bk, causal, use_len):
+    """Shapes with enough 256-query workgroups for the software-pipelined kernel, which multiplies
+    E4M3 operands 64 at a time (v_mfma_f32_32x32x64_f8f6f4); ragged length, grouped heads, per-batch
+    key lengths.  The same 2e-3 against the emulation as the general kernel, three runs bit-equal."""
+    b, hq, hkv, n = 2, 16, 8, 1024 + 40
+    q, k, v = fill_qkv(b, hq, hkv, n, d)
+    k = k + np.float32(0.5) * synth.normal(7, (1, hkv, 1, d))
+    kv_len = np.array([n, 700], np.int32) if use_len else None
+    runs = [run_fp8(dev, q, k, v, 128, bk, True, F32, kv_len=kv_len, causal=causal) for _ in range(3)]
+    q8, k8, sq, sk, out = runs[0]
+    assert np.array_equal(out, runs[1][4]) and np.array_equal(out, runs[2][4])
+    w_q8, w_sq = oracle.quant_blocks_fp8(q, 128)
+    w_k8, w_sk = oracle.quant_blocks_fp8(k, bk, sub=oracle.k_mean(k))
+    assert np.array_equal(q8, w_q8) and np.array_equal(k8, w_k8)
+    assert np.array_equal(sq, w_sq) and np.array_equal(sk, w_sk)
+    want = oracle.sage_fp8(w_q8, w_k8, w_sq, w_sk, v, 128, bk, causal=causal, kv_len=kv_len)
+    assert np.abs(out - want).max() < 2e-3
+    # bf16 tensors in and out: the same function of the rounded inputs, plus the output rounding
+    qb, kb = oracle.bf16_round(q), oracle.bf16_round(k)
+    out16 = run_fp8(dev, qb, kb, v, 128, bk, True, BF16, out_dtype=BF16, kv_len=kv_len, causal=causal)[4]
+    b_q8, b_sq = oracle.quant_blocks_fp8(qb, 128)
+    b_k8, b_sk = oracle.quant_blocks_fp8(kb, bk, sub=oracle.k_mean(kb))
+    want16 = oracle.sage_fp8(b_q8, b_k8, b_sq, b_sk, v, 128, bk, causal=causal, kv_len=kv_len)
+    assert np.abs(out16 - want16).max() < 2e-3 + 2.0 ** -8 * np.abs(want16).max()
+
+
 def test_fp8_attention_against_exact(dev):
     """N(0,1) data at D = 128: three mantissa bits cost more than int8's seven; the bound asserted is
     what the format gives (measured: maximum 3.8e-2, median 1.8e-3, 99th percentile 9e-3; int8 on the

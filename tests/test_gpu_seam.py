@@ -223,6 +223,38 @@ def test_ar_flash_sage_fp8_by_name(dev, kernels):
     assert np.abs(got - want).max() < 2e-3
 
 
+@pytest.mark.parametrize("d,causal,out_f32", [(128, True, 1), (64, False, 0)])
+def test_ar_flash_sage_fp8_long_by_name(dev, kernels, d, causal, out_f32):
+    """The software-pipelined FP8 entry by name, on codes from the by-name quantiser, against the
+    general FP8 entry on the same codes (both within 2e-3 of the emulation)."""
+    b, hq, hkv, n, bq, bk = 1, 4, 2, 700, 128, 64
+    q, k, v = fill_qkv(b, hq, hkv, n, d)
+    with Bufs(dev) as bufs:
+        def quant(x, blk, heads):
+            dx, x8 = bufs.put(x), bufs.new(x.size)
+            nblk = (n + blk - 1) // blk
+            sc, mean = bufs.new(b * heads * nblk * 4), bufs.new(b * heads * d * 4)
+            dev.launch(kernels, "ar_sage_quant_blocks_fp8_f32", (nblk, b * heads, 1), (256, 1, 1), [dx, x8, sc, mean],
+                       [n, d, blk, nblk, 0])
+            return x8, sc
+        q8, sq = quant(q, bq, hq)
+        k8, sk = quant(k, bk, hkv)
+        dv = bufs.put(synth.to_bf16_bits(v))
+        do, dg = bufs.new(q.size * 4), bufs.new(q.size * 4)
+        dev.launch(kernels, "ar_flash_sage_fp8_long", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, do, do, sq, sk],
+                   [n, d, int(causal), 0, hq, hkv, bq, bk, out_f32])
+        dev.launch(kernels, "ar_flash_sage_fp8", _grid(n, 128, b, hq), (256, 1, 1), [q8, k8, dv, dg, dg, sq, sk],
+                   [n, d, int(causal), 0, hq, hkv, bq, bk])
+        got = do.copyout(np.float32, q.shape) if out_f32 else synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+        general = dg.copyout(np.float32, q.shape)
+    w_q8, w_sq = oracle.quant_blocks_fp8(q, bq)
+    w_k8, w_sk = oracle.quant_blocks_fp8(k, bk)
+    want = oracle.sage_fp8(w_q8, w_k8, w_sq, w_sk, v, bq, bk, causal=causal)
+    tol = 2e-3 if out_f32 else 2e-3 + 2.0 ** -8 * np.abs(want).max()
+    assert np.abs(got - want).max() < tol
+    assert np.abs(got - general).max() < 2 * tol
+
+
 @pytest.mark.parametrize("n,d,causal,hkv", [(197, 64, False, 6), (256, 128, True, 3), (1, 64, False, 6), (130, 128, False, 1)])
 def test_ar_flash_bf16_short_by_name(dev, kernels, n, d, causal, hkv):
     """The variant for sequences of at most 256 keys (8 waves, two per 32 queries on the even / odd

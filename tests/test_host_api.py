@@ -209,6 +209,16 @@ def test_sage_fp8_setting(hdev):
     names = [sess.step(i)[0] for i in range(n_calls)]
     assert names[0] == "ar_sage_quant_blocks_fp8_f32" and "ar_flash_sage_fp8" in names
     assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v, causal=True)).max()) < 6e-2
+    # enough 256-query workgroups: the pipelined FP8 entry, as for int8
+    b, h, n = 2, 32, 1024
+    q, k, v = _fill((b, h, n, d), 3), _fill((b, h, n, d), 11), _fill((b, h, n, d), 19)
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v))
+    sess.begin_capture()
+    out = tq.sage_attention_with(tk, tv, None, 0.0, False, sess, st)
+    n_calls = sess.end_capture()
+    assert "ar_flash_sage_fp8_long" in [sess.step(i)[0] for i in range(n_calls)]
+    rows = np.array([0, 255, 256, 777, 1023])
+    assert float(np.abs(out.to_list()[:, :, rows] - oracle.sdpa_f64(q, k, v, rows=rows)).max()) < 6e-2
 
 
 @gpu
