@@ -36,6 +36,11 @@
 
 #include "attn_fwd.h"
 
+// 1: the int8 pipeline reads its int32 logit accumulators as biased floats (no conversions)
+#ifndef ARHIP_PIPE_INT_BIAS
+#define ARHIP_PIPE_INT_BIAS 1
+#endif
+
 namespace arhip {
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -64,11 +69,28 @@ constexpr int attn_pipe_lds_bytes()
     return 4 * 4096 * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64 + D * 2 / 64);
 }
 
-// The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
-// aligned; wg_linear: this workgroup's index in [0, p.total).
-template <int D, bool CAUSAL, int MODE, bool OUT_F32>
-__device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned char *lds, int wg_linear)
+// workgroup index -> (batch * heads + head, query tile of 256), as in attn_fwd_kernel
+template <bool CAUSAL>
+__device__ __forceinline__ void pipe_work_item(const AttnParams &p, int wg, int &bh, int &qt)
 {
+    if (CAUSAL && p.lpt) {
+        const int nbh = p.total / p.nq;
+        qt = p.nq - 1 - wg / nbh;
+        bh = wg % nbh;
+    } else {
+        if ((p.total & 7) == 0) wg = (wg & 7) * (p.total >> 3) + (wg >> 3);
+        bh = wg / p.nq;
+        qt = wg - bh * p.nq;
+        if (CAUSAL) qt = p.nq - 1 - qt;
+    }
+}
+
+// The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
+// aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below.
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS>
+__device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
+{
+    static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
     constexpr int NW = 8;
     constexpr int BQ = NW * 32;
     constexpr int QK_BYTES = (MODE != MODE_BF16) ? 1 : 2;
@@ -93,19 +115,8 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     const int i32 = lane & 31;
     const int h = lane >> 5;
 
-    // workgroup -> (head, query tile), as in attn_fwd_kernel
-    int wg = wg_linear;
     int bh, qt;
-    if (CAUSAL && p.lpt) {
-        const int nbh = p.total / p.nq;
-        qt = p.nq - 1 - wg / nbh;
-        bh = wg % nbh;
-    } else {
-        if ((p.total & 7) == 0) wg = (wg & 7) * (p.total >> 3) + (wg >> 3);
-        bh = wg / p.nq;
-        qt = wg - bh * p.nq;
-        if (CAUSAL) qt = p.nq - 1 - qt;
-    }
+    pipe_work_item<CAUSAL>(p, wg_linear, bh, qt);
     const int b = bh / p.Hq;
     const int head = bh - b * p.Hq;
     const int kvh = head / (p.Hq / p.Hkv);
@@ -209,6 +220,29 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
     float m_run = NEG_SENTINEL;
     float l_run = 0.f;
+    // int8: the int32 accumulators start at 0x4B400000, the bit pattern of the float 12582912 = 1.5 * 2^23,
+    // whose unit in the last place is 1: with |sum| <= 128 * 128^2 = 2^21 < 2^22 the accumulator's bits,
+    // read as a float, ARE the value 12582912 + sum, so no int -> float conversion is needed; the softmax
+    // subtracts m_bias = m_run + 12582912 c instead of m_run (one fused multiply-add per block).
+    // m_bias is rounded at the magnitude of 12582912 c, so the exponent is off by at most 0.75 c,
+    // c being the logit of ONE integer step (attn_pipe_body picks this variant only where that is
+    // below 2^-10 * 0.75).
+    constexpr float BIAS_F = 12582912.0f;
+    acc_t s_init;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s_init[r] = 0;
+    if constexpr (BIAS) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_init[r] = 0x4B400000;
+        asm volatile("" : "+v"(s_init));  // a register block of its own: the matrix instruction's C operand
+    }
+    float m_bias = NEG_SENTINEL;  // what the pipelined softmax subtracts for the block it works on
+    auto set_bias = [&](float c) __attribute__((always_inline)) { m_bias = BIAS ? __builtin_fmaf(BIAS_F, c, m_run) : m_run; };
+    // a logit accumulator as a float (before the factor c)
+    auto as_logit = [&](const acc_t &a, int r) __attribute__((always_inline)) -> float {
+        if constexpr (BIAS) return __builtin_bit_cast(float, (int)a[r]);
+        else return (float)a[r];
+    };
     float sq_lane = 1.f;
     const int nkb = (MODE != MODE_BF16) ? (N + p.bk - 1) / p.bk : 0;
     if (MODE != MODE_BF16) {
@@ -290,9 +324,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     };
     static_assert(MODE != MODE_FP8 || KSTEPS % 2 == 0, "FP8 steps come in pairs");
     auto mfma_qk = [&]() __attribute__((always_inline)) -> acc_t {
-        acc_t s;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0;
+        acc_t s = s_init;
         static_for<0, KSTEPS>([&](auto si) __attribute__((always_inline)) {
             constexpr int st = decltype(si)::value;
             constexpr int pv = st > 0 ? st - 1 : 0;
@@ -390,7 +422,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
     // The softmax of an unmasked block as a list of single vector instructions, so that they can be
     // dealt out between the matrix instructions by hand.  Per half of 8 keys: [convert (int8 only)]
     // 8 x fma(s, c, -m), 8 x exp2, 7 adds (row sum of the unrounded values), 4 bf16 packs.
-    constexpr int SM_CVT = (MODE == MODE_I8) ? 8 : 0;
+    constexpr int SM_CVT = (MODE == MODE_I8 && !BIAS) ? 8 : 0;
     constexpr int SM_HALF = SM_CVT + 8 + 8 + 7 + 4;
     constexpr int SM_OPS = 2 * SM_HALF;
     float sm_t[8], sm_x[8], sm_a[6], sm_half[2];
@@ -402,7 +434,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
             sm_t[k] = (float)s[ks * 8 + k];
         } else if constexpr (k < SM_CVT + 8) {
             constexpr int r = k - SM_CVT;
-            sm_t[r] = __builtin_fmaf((MODE == MODE_I8) ? sm_t[r] : (float)s[ks * 8 + r], c, -m_run);
+            sm_t[r] = __builtin_fmaf(SM_CVT ? sm_t[r] : as_logit(s, ks * 8 + r), c, -m_bias);
             // a masked key: exp2 of the sentinel is exactly 0
             if (M && 8 * ((ks * 8 + r) >> 2) + (r & 3) > rel) sm_t[r] = NEG_SENTINEL;
         } else if constexpr (k < SM_CVT + 16) {
@@ -444,8 +476,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
                           const unsigned char *sv, int vb, const unsigned char *sk, int kb, float c_cur, float c_next,
                           int rel_cur, int rel_next) __attribute__((always_inline)) {
         // ---- R1 ----
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s_new[r] = 0;
+        s_new = s_init;
         ARHIP_FENCE();
         static_for<0, KSTEPS>([&](auto si) __attribute__((always_inline)) {
             constexpr int st = decltype(si)::value;
@@ -468,6 +499,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         rs = sm_half[0] + sm_half[1];
         if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(mc, sc, cb, c_cur, rel_cur, p_cur, rs);
         l_run += rs;
+        set_bias(c_next);  // the reference is final for block j+1 from here to the end of its softmax
         ARHIP_FENCE();
         // ---- R2 ----
         static_for<0, DB * 2>([&](auto gi) __attribute__((always_inline)) {
@@ -527,6 +559,7 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
         load_kf(lds, 1);
         load_vf(lds, 0);
         const float c0 = tile_c(0, 0);
+        set_bias(c0);
         if (nfull > 0)
             static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(PLAIN, ic, s_a, c0, 0, p_a); });
         else
@@ -616,6 +649,43 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
             const uint4 w = *(const uint4 *)(ob + r * OROW + cl * 16);
             if (wq0 + r < N) *(uint4 *)(obase + (size_t)(wq0 + r) * p.os[2] + cl * 8) = w;
         }
+    }
+}
+
+// int8: the variant with biased accumulators saves 16 conversions per 32-key block but rounds the
+// exponent reference at the magnitude of 12582912 c (error <= 0.75 c in the exponent, c = the logit
+// of one integer step = sq sk scale log2(e)).  A workgroup takes it only if c <= 2^-10 for every
+// (query block, key block) pair it can meet, so that a probability moves by less than 2^-11 relative
+// (a quarter of the rounding step of P to bf16); coarser quantisations (outliers stretching a
+// block's scale) run the converting variant, whose logits are exact.  The choice is uniform over
+// the workgroup: every wave reduces the same scales.
+template <int D, bool CAUSAL, int MODE, bool OUT_F32>
+__device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned char *lds, int wg_linear)
+{
+    if constexpr (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS) {
+        int bh, qt;
+        pipe_work_item<CAUSAL>(p, wg_linear, bh, qt);
+        const int lane = threadIdx.x & 63;
+        const int N = p.N;
+        const int nqb = (N + p.bq - 1) / p.bq, nkb = (N + p.bk - 1) / p.bk;
+        const int b = bh / p.Hq;
+        const int kv_bh = b * p.Hkv + (bh - b * p.Hq) / (p.Hq / p.Hkv);
+        const int qb0 = (qt * 256) / p.bq, qb1 = min(qt * 256 + 255, N - 1) / p.bq;
+        float mq = 0.f, mk = 0.f;
+        for (int i = qb0 + lane; i <= qb1; i += 64) mq = fmaxf(mq, fabsf(p.sq[(size_t)bh * nqb + i]));
+        for (int i = lane; i < nkb; i += 64) mk = fmaxf(mk, fabsf(p.sk[(size_t)kv_bh * nkb + i]));
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) {
+            mq = fmaxf(mq, __shfl_xor(mq, o));
+            mk = fmaxf(mk, __shfl_xor(mk, o));
+        }
+        const float c_max = ((mq * mk) * fabsf(p.scale)) * LOG2E;
+        // (a NaN or infinite scale fails the comparison and takes the exact variant)
+        const bool fine = __builtin_amdgcn_readfirstlane((int)(c_max <= 0x1p-10f)) != 0;
+        if (fine) attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, true>(p, lds, wg_linear);
+        else attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, false>(p, lds, wg_linear);
+    } else {
+        attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, false>(p, lds, wg_linear);
     }
 }
 
