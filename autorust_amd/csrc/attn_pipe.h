@@ -86,9 +86,10 @@ __device__ __forceinline__ void pipe_work_item(const AttnParams &p, int wg, int 
 }
 
 // The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
-// aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below.
+// aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below;
+// m_grid: the power of two the exponent reference is kept a multiple of (BIAS only).
 template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS>
-__device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
+__device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear, float m_grid)
 {
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
     constexpr int NW = 8;
@@ -223,10 +224,14 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // int8: the int32 accumulators start at 0x4B400000, the bit pattern of the float 12582912 = 1.5 * 2^23,
     // whose unit in the last place is 1: with |sum| <= 128 * 128^2 = 2^21 < 2^22 the accumulator's bits,
     // read as a float, ARE the value 12582912 + sum, so no int -> float conversion is needed; the softmax
-    // subtracts m_bias = m_run + 12582912 c instead of m_run (one fused multiply-add per block).
-    // m_bias is rounded at the magnitude of 12582912 c, so the exponent is off by at most 0.75 c,
-    // c being the logit of ONE integer step (attn_pipe_body picks this variant only where that is
-    // below 2^-10 * 0.75).
+    // subtracts m_bias = m_run + 12582912 c instead of m_run (one fused multiply-add per block), and
+    // fma(12582912 + sum, c, -m_bias) rounds the same real number sum c - m_run as
+    // fma((float)sum, c, -m_run) does PROVIDED m_bias is exact.  Two things make it exact: c is
+    // rounded to 21 significant bits (so that 12582912 c = 3 c 2^22 has at most 23), and m_run only
+    // ever takes multiples of m_grid, a power of two that no unit in the last place of any
+    // 12582912 c + m_run this workgroup can meet exceeds (attn_pipe_body derives it from the largest
+    // scales).  Where m_run outweighs 12582912 c (tiny scales) the sum may still round, by at most
+    // half a unit in the last place of m_run: 2^-16 for references below 256.
     constexpr float BIAS_F = 12582912.0f;
     acc_t s_init;
 #pragma unroll
@@ -238,6 +243,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     }
     float m_bias = NEG_SENTINEL;  // what the pipelined softmax subtracts for the block it works on
     auto set_bias = [&](float c) __attribute__((always_inline)) { m_bias = BIAS ? __builtin_fmaf(BIAS_F, c, m_run) : m_run; };
+    const float m_grid_inv = BIAS ? 1.0f / m_grid : 1.0f;
     // a logit accumulator as a float (before the factor c)
     auto as_logit = [&](const acc_t &a, int r) __attribute__((always_inline)) -> float {
         if constexpr (BIAS) return __builtin_bit_cast(float, (int)a[r]);
@@ -267,7 +273,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             const int a = __builtin_amdgcn_readlane(__float_as_int(skv_cur), t & 63);
             const int bnext = __builtin_amdgcn_readlane(__float_as_int(skv_nxt), t & 63);
             const float f = __int_as_float(((t >> 6) == (it >> 6)) ? a : bnext);
-            return ((sq_lane * f) * p.scale) * LOG2E;
+            const float c = ((sq_lane * f) * p.scale) * LOG2E;
+            // BIAS: to 21 significant bits, round to nearest (a relative change of at most 2^-21)
+            return BIAS ? __uint_as_float((__float_as_uint(c) + 4u) & ~7u) : c;
         } else {
             return c_scale;
         }
@@ -333,7 +341,10 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         return s;
     };
     auto move_reference = [&](float mx) __attribute__((always_inline)) {
-        const float m_new = fmaxf(m_run, mx);
+        float m_new = fmaxf(m_run, mx);
+        // BIAS: up to the next multiple of m_grid (softmax does not depend on the reference; a row
+        // with no visible key yet keeps the sentinel)
+        if (BIAS && m_new > -1e29f) m_new = __builtin_ceilf(m_new * m_grid_inv) * m_grid;
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;
         l_run *= alpha;
@@ -652,13 +663,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     }
 }
 
-// int8: the variant with biased accumulators saves 16 conversions per 32-key block but rounds the
-// exponent reference at the magnitude of 12582912 c (error <= 0.75 c in the exponent, c = the logit
-// of one integer step = sq sk scale log2(e)).  A workgroup takes it only if c <= 2^-10 for every
-// (query block, key block) pair it can meet, so that a probability moves by less than 2^-11 relative
-// (a quarter of the rounding step of P to bf16); coarser quantisations (outliers stretching a
-// block's scale) run the converting variant, whose logits are exact.  The choice is uniform over
-// the workgroup: every wave reduces the same scales.
+// int8: the biased accumulators (see s_init) need the exponent reference on a grid no finer than the
+// unit in the last place of 12582912 c for the largest c = sq sk scale log2(e) the workgroup can
+// meet: every wave reduces the same scales, so the grid is uniform over the workgroup.
 template <int D, bool CAUSAL, int MODE, bool OUT_F32>
 __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
@@ -679,13 +686,18 @@ __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned cha
             mq = fmaxf(mq, __shfl_xor(mq, o));
             mk = fmaxf(mk, __shfl_xor(mk, o));
         }
-        const float c_max = ((mq * mk) * fabsf(p.scale)) * LOG2E;
-        // (a NaN or infinite scale fails the comparison and takes the exact variant)
-        const bool fine = __builtin_amdgcn_readfirstlane((int)(c_max <= 0x1p-10f)) != 0;
-        if (fine) attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, true>(p, lds, wg_linear);
-        else attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, false>(p, lds, wg_linear);
+        // 12582912 c_max < 2^(E+1): the sums stay below 2^(E+2) wherever the bias outweighs the
+        // reference, so their unit in the last place is at most 2^(E-22); the grid is twice that.
+        // (Scales that are not finite, or zero, give a grid of 1: the results are garbage or
+        // trivial either way.)
+        const float x = 12582912.0f * (((mq * mk) * fabsf(p.scale)) * LOG2E);
+        const int e = (int)((__float_as_uint(x) >> 23) & 0xff) - 127;  // floor(log2 x)
+        float grid = 1.0f;
+        if (x > 0x1p-60f && x < 0x1p100f) grid = __uint_as_float((uint32_t)(e - 21 + 127) << 23);
+        grid = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(grid)));
+        attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, true>(p, lds, wg_linear, grid);
     } else {
-        attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, false>(p, lds, wg_linear);
+        attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, false>(p, lds, wg_linear, 1.0f);
     }
 }
 

@@ -79,10 +79,12 @@ def test_block_quantised_smoothed(dev, N, causal, D):
 
 @pytest.mark.parametrize("causal", [False, True])
 def test_long_sequence_kernel_on_fine_and_coarse_scales(dev, causal):
-    """The software-pipelined int8 kernel reads its int32 logit sums as biased floats where the logit
-    of one integer step, c = sq sk scale log2(e), is at most 2^-10 for the whole workgroup, and converts
-    them otherwise.  Heads scaled so that c runs from ~1e-4 to ~2.5e-3 put both variants, and workgroups
-    right at the threshold, into one launch; each head must match the emulation as before."""
+    """The software-pipelined int8 kernel reads its int32 logit sums as biased floats (no conversions)
+    whatever the logit of one integer step, c = sq sk scale log2(e), is: the bias is exact because c
+    is cut to 21 significant bits and the exponent reference sits on a power-of-two grid derived from
+    the workgroup's largest c (tests/test_int_bias_identity.py pins that arithmetic on the CPU).  Heads
+    scaled so that c runs from ~1e-4 to ~2.5e-3 put fine and coarse quantisations into one launch;
+    every head must match the emulation to the bound the bf16 rounding of P sets."""
     B, H, N, D = 1, 32, 1024 + 72, 128
     q, k, v = synth.normal(601, (B, H, N, D)), synth.normal(602, (B, H, N, D)), synth.normal(603, (B, H, N, D))
     gain = np.float32(2.0) ** np.linspace(0.0, 5.0, H, dtype=np.float32)
@@ -92,18 +94,18 @@ def test_long_sequence_kernel_on_fine_and_coarse_scales(dev, causal):
     q8, sq, k8, sk = _check_bits(r, q, k, v, 128, 64, True)
     c = (sq.max(axis=2) * sk.max(axis=2)) * np.float32(1.0 / np.sqrt(128.0)) * np.float32(1.4426950408889634)
     c = c.reshape(-1)
-    assert (c <= 2.0 ** -10).sum() >= 4 and (c > 2.0 ** -10).sum() >= 4      # both variants ran
+    assert (c <= 2.0 ** -12).sum() >= 4 and (c > 2.0 ** -10).sum() >= 4      # fine and coarse steps
     want = oracle.sage(q8, k8, sq, sk, v, 128, 64, causal=causal, kv_len=kv_len)
     err = np.abs(r["out"] - want).reshape(H, -1).max(axis=1)
     # P is rounded to bf16 relative to the kernel's running exponent reference, in the emulation relative
-    # to the final maximum: a relative 2^-9 of |v| <= 4.5 at most, reached where the softmax is nearly
-    # one-hot (the heads with the large gains, which are the converting ones)
-    assert err.max() < 4.5 * 2.0 ** -8, (err, c)
-    fine, coarse = c <= 2.0 ** -10, c > 2.0 ** -10
-    assert err[c <= 2.0 ** -12].max() < 4e-3
-    # no step at the threshold: the biased heads just below it are no further from the emulation
-    # than the converting heads just above it
-    assert err[fine & (c > 2.0 ** -11)].max() <= 1.25 * err[coarse & (c <= 2.0 ** -9)].max(), (err, c)
+    # to the final maximum, and the row sum is taken over the unrounded values on both sides: each side
+    # is off by a relative 2^-9 on every probability, at different rounding points, so where a few keys
+    # carry the row the two differ by up to 2 * 2^-9 * max|v| (the heads with the large gains).
+    bound = 2.0 ** -8 * float(np.abs(v).max())
+    assert err.max() < bound, (err, c, bound)
+    # the heads with the small gains have flat rows, where the rounding errors average out (under the
+    # causal mask the first rows see few keys and stay closer to the bound above)
+    assert err[c <= 2.0 ** -12].max() < (8e-3 if causal else 4e-3)
 
 
 def test_bf16_inputs_and_bf16_output(dev):
