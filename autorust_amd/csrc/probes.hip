@@ -135,3 +135,69 @@ extern "C" __global__ void probe_clock_sampler(long long *ticks, int samples, in
         ticks[2 * i + 1] = r1 - r0;
     }
 }
+
+// What the vector ALU can still issue beside the matrix pipe: every wave runs `iters` times
+// { 1 matrix instruction (bf16 32x32x16 or int8 32x32x32, four accumulators in turn); K independent
+// vector instructions (v_fma_f32 or v_exp_f32) }, two waves per SIMD like the attention kernels, and
+// every wave records the real-time (100 MHz) ticks of its loop.  With K = 0 the loop runs at the
+// matrix rate; the growth with K is what the softmax instructions between the matrix instructions
+// of an attention block cost.  One kernel per (matrix type, vector instruction, K).
+template <int K, bool EXP, bool I8>
+__device__ __forceinline__ void probe_issue_mix_body(const uint4 *src, float *out, long long *ticks, int iters)
+{
+    float d[8], a = threadIdx.x * 0.001f, b = 1.0001f;
+    for (int i = 0; i < 8; ++i) d[i] = i * 0.5f;
+    uint4 fa[4], fb[4];
+    for (int j = 0; j < 4; ++j) {
+        fa[j] = src[(threadIdx.x * 8 + j) & 8191];
+        fb[j] = src[(threadIdx.x * 8 + 4 + j) & 8191];
+    }
+    f32x16 o[4];
+    i32x16 oi[4];
+    for (int n = 0; n < 4; ++n)
+        for (int r = 0; r < 16; ++r) {
+            o[n][r] = 0.f;
+            oi[n][r] = 0;
+        }
+    const long long r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (I8)
+                oi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, fa[j]), __builtin_bit_cast(i32x4, fb[j]), oi[j], 0, 0, 0);
+            else
+                o[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[j]), __builtin_bit_cast(bf16x8, fb[j]), o[j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                if constexpr (EXP) asm volatile("v_exp_f32 %0, %1" : "+v"(d[i & 7]) : "v"(a));
+                else asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(d[i & 7]) : "v"(a), "v"(b));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    const long long r1 = __builtin_amdgcn_s_memrealtime();
+    float r = 0.f;
+    for (int i = 0; i < 8; ++i) r += d[i];
+    for (int n = 0; n < 4; ++n)
+        for (int i = 0; i < 16; ++i) r += o[n][i] + (float)oi[n][i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = r;
+    if ((threadIdx.x & 63) == 0) ticks[blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64] = r1 - r0;
+}
+#define PROBE_ISSUE_MIX(NAME, K, EXP, I8)                                                                              \
+    extern "C" __global__ void __launch_bounds__(512) NAME(const uint4 *src, float *out, long long *ticks, int iters)  \
+    {                                                                                                                  \
+        probe_issue_mix_body<K, EXP, I8>(src, out, ticks, iters);                                                      \
+    }
+#define PROBE_ISSUE_MIX_KS(PREFIX, EXP, I8)     \
+    PROBE_ISSUE_MIX(PREFIX##_k0, 0, EXP, I8)    \
+    PROBE_ISSUE_MIX(PREFIX##_k2, 2, EXP, I8)    \
+    PROBE_ISSUE_MIX(PREFIX##_k4, 4, EXP, I8)    \
+    PROBE_ISSUE_MIX(PREFIX##_k6, 6, EXP, I8)    \
+    PROBE_ISSUE_MIX(PREFIX##_k8, 8, EXP, I8)    \
+    PROBE_ISSUE_MIX(PREFIX##_k10, 10, EXP, I8)  \
+    PROBE_ISSUE_MIX(PREFIX##_k14, 14, EXP, I8)
+PROBE_ISSUE_MIX_KS(probe_mix_bf16_fma, false, false)
+PROBE_ISSUE_MIX_KS(probe_mix_bf16_exp, true, false)
+PROBE_ISSUE_MIX_KS(probe_mix_i8_fma, false, true)
+PROBE_ISSUE_MIX_KS(probe_mix_i8_exp, true, true)

@@ -284,6 +284,34 @@ def sustained_mfma(dev):
     return res
 
 
+def issue_mix(dev):
+    """Time per matrix instruction of a loop of { 1 MFMA ; K vector instructions } for K = 0..14
+    (probe_mix_* in csrc/probes.hip), two waves per SIMD, operands with random mantissas: how much
+    vector work fits beside the matrix pipe before the loop slows down."""
+    mod = _probes(dev)
+    rng = np.random.default_rng(5)
+    bits = (rng.integers(0, 1 << 16, 8192 * 8, dtype=np.uint32) & 0x007F) | 0x3C00     # bf16 values in [0.0078, 0.0156)
+    src = dev.from_numpy(bits.astype(np.uint16))
+    out, ticks = dev.alloc(256 * 512 * 4), dev.alloc(256 * 8 * 8)
+    iters = 2000
+    res = {}
+    for mat in ("bf16", "i8"):
+        for op in ("fma", "exp"):
+            row = {}
+            for k in (0, 2, 4, 6, 8, 10, 14):
+                name = "probe_mix_%s_%s_k%d" % (mat, op, k)
+                dev.launch(mod, name, (256, 1, 1), (512, 1, 1), [src, out, ticks], [iters])
+                dev.launch(mod, name, (256, 1, 1), (512, 1, 1), [src, out, ticks], [iters])
+                t = ticks.copyout(np.int64, (256 * 8,)).astype(np.float64)
+                # real-time ticks are 10 ns; 4 matrix instructions per iteration; two waves share a SIMD
+                row["K=%d" % k] = round(float(t.mean()) * 10.0 / (iters * 4) / 2.0, 2)
+            res["%s_mfma+%s" % (mat, op)] = row
+    src.free()
+    out.free()
+    ticks.free()
+    return res
+
+
 def shader_clock_during(dev, w, steps):
     """Median shader clock (MHz) while `steps` steps of the workload run: a one-wave sampler
     (probe_clock_sampler) on a second stream beside them.  Not part of the timed region."""
@@ -375,12 +403,21 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="one step of the workload plus one plain 1 GiB copy kernel and nothing else: "
                          "the run to put under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`")
+    ap.add_argument("--issue-probe", action="store_true",
+                    help="time loops of one matrix instruction plus K vector instructions (no workload)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-clock", action="store_true", help="skip the shader-clock and sustained-MFMA probes")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
 
+    if args.issue_probe:
+        dev = Device(0)
+        print(json.dumps({"issue_mix_ns_per_mfma_per_simd": issue_mix(dev),
+                          "note": "loop of {1 MFMA (32x32x16 bf16 or 32x32x32 int8); K v_fma_f32 or v_exp_f32}, "
+                                  "two waves per SIMD, 256 workgroups of 512 threads"}))
+        dev.close()
+        return
     dev = Device(0)
     log("device", dev.arch, dev.compute_units, "CUs")
     t0 = time.time()
