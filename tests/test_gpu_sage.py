@@ -108,6 +108,27 @@ def test_long_sequence_kernel_on_fine_and_coarse_scales(dev, causal):
     assert err[c <= 2.0 ** -12].max() < (8e-3 if causal else 4e-3)
 
 
+def test_long_sequence_kernel_on_extreme_scales(dev):
+    """Scales far outside the usual range through the biased-float logits of the pipelined kernel: query
+    gains from 2^-12 to 2^9 give steps c from ~1e-8 (the bias 12582912 c is then smaller than 1) to ~3e-2
+    (logits in the thousands, one-hot rows, an exponent reference near 10^4)."""
+    B, H, N, D = 1, 16, 1024, 128
+    q, k, v = synth.normal(611, (B, H, N, D)), synth.normal(612, (B, H, N, D)), synth.normal(613, (B, H, N, D))
+    gain = np.float32(2.0) ** np.linspace(-12.0, 9.0, H, dtype=np.float32)
+    q = q * gain[None, :, None, None]
+    r = run_sage(dev, q, k, v, 128, 64, smooth=True, causal=False)
+    q8, sq, k8, sk = _check_bits(r, q, k, v, 128, 64, True)
+    c = (sq.max(axis=2) * sk.max(axis=2)) * np.float32(1.0 / np.sqrt(128.0)) * np.float32(1.4426950408889634)
+    assert c.min() < 1e-7 and c.max() > 1e-2
+    want = oracle.sage(q8, k8, sq, sk, v, 128, 64, causal=False)
+    assert np.isfinite(r["out"]).all()
+    err = np.abs(r["out"] - want).reshape(H, -1).max(axis=1)
+    # the bound of test_long_sequence_kernel_on_fine_and_coarse_scales: the two roundings of P to bf16
+    assert err.max() < 2.0 ** -8 * float(np.abs(v).max()), (err, c)
+    # flat rows (tiny logits): the output is close to the mean of V and the rounding errors average out
+    assert err[:4].max() < 1e-3, err
+
+
 def test_bf16_inputs_and_bf16_output(dev):
     B, Hq, Hkv, N, D, bq, bk = 1, 4, 4, 512, 128, 128, 64
     q, k, v = _inputs(B, Hq, Hkv, N, D)
