@@ -21,7 +21,7 @@
 //           With 8 waves per workgroup each SIMD holds two waves, and one of
 //           them can exponentiate while the other multiplies.
 //   lazy  : the exponent reference only moves (and the accumulators are only
-//           rescaled) when a row maximum outgrows it by 2^30; softmax does not
+//           rescaled) when a row maximum outgrows it by 2^60; softmax does not
 //           depend on the reference, so the result is the same function.
 //
 // MFMA shapes (wave64):
@@ -59,8 +59,8 @@ constexpr int MODE_FP8 = 2;   // q, k FP8 E4M3 (OCP) with block scales: the refe
 constexpr int BK = 64;        // keys per tile
 constexpr float NEG_SENTINEL = -1e30f;  // src/runtime/cuda_flash_bf16.rs:106 (AR_NEG)
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr float LAZY_TAU = 30.0f;    // log2 units the running maximum may outgrow the exponent reference
-constexpr float LAZY_LIMIT = 1073741824.0f;  // = 2^LAZY_TAU: the largest probability the lazy reference lets through
+constexpr float LAZY_TAU = 60.0f;    // log2 units the running maximum may outgrow the exponent reference
+constexpr float LAZY_LIMIT = 1152921504606846976.0f;  // = 2^LAZY_TAU: the largest probability the lazy reference lets through
 
 struct AttnParams {
     const void *q;
