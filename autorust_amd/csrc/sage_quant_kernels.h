@@ -61,7 +61,18 @@ __device__ __forceinline__ void k_mean_partial_body(const T *x, float *part, int
     const int j1 = min(N, j0 + MEAN_CHUNK);
     const size_t base = lay.head(bh) + g * 8;
     float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int j = j0; j < j1; ++j) {
+    // eight rows in flight per thread (the loads of a group are issued together), added in token order
+    int j = j0;
+    for (; j + 8 <= j1; j += 8) {
+        float v[8][8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) ld8(x, base + (size_t)(j + u) * lay.st, v[u]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s[i] += v[u][i];
+    }
+    for (; j < j1; ++j) {
         float v[8];
         ld8(x, base + (size_t)j * lay.st, v);
 #pragma unroll
