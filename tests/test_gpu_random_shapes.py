@@ -72,4 +72,9 @@ def test_sage_random_shapes(dev, waves, monkeypatch):
             want = oracle.sage(q8, k8, sq, sk, v, bq, bk, kv_len=kv_len, causal=causal)
             want = np.where(np.isfinite(want), want, 0.0)
             err = float(np.abs(r["out"] - want).max())
-            assert np.isfinite(r["out"]).all() and err < 4e-3, (B, Hq, Hkv, N, D, causal, bq, bk, err)
+            # kernel and emulation round P to bf16 at different points (the running exponent reference
+            # against the final maximum) and both sum the unrounded values: up to 2 * 2^-9 * max|v| where
+            # a few keys carry a row (short key lengths, first causal rows); measured worst over other
+            # seeds: 8e-3
+            bound = 2.0 ** -8 * float(np.abs(v).max())
+            assert np.isfinite(r["out"]).all() and err < bound, (B, Hq, Hkv, N, D, causal, bq, bk, err, bound)
