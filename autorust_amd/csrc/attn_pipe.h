@@ -559,6 +559,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     }
     wait_vmem_le<0>();
     __syncthreads();
+    float c_carry = tile_c(0, 0);  // exponent factor of the tile the next tile_iter works on
     acc_t s_a, s_b;  // logits of the even / odd block of a tile
 #pragma unroll
     for (int r = 0; r < 16; ++r) s_a[r] = s_b[r] = 0;
@@ -585,7 +586,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         // tile it + 3 goes to the stage tile it - 1 vacated at the last barrier
         issue_tile(it + 3, (it + 3) & 3);
         advance_sk_group(it);
-        const float c_cur = tile_c(it, it), c_nxt = tile_c(it + 1, it);
+        // (tile_iter runs on consecutive tiles from 0 on: this tile's factor is last iteration's c_nxt)
+        const float c_cur = c_carry, c_nxt = tile_c(it + 1, it);
+        c_carry = c_nxt;
         const int rel0 = lim4h - it * BK;
         pipe_block(m0, m1, s_a, s_b, p_a, p_b, st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, c_cur, rel0, rel0 - 32);
         pipe_block(m1, m2, s_b, s_a, p_b, p_a, st_cur, 1, st_nxt, 0, st_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64);
