@@ -201,3 +201,31 @@ PROBE_ISSUE_MIX_KS(probe_mix_bf16_fma, false, false)
 PROBE_ISSUE_MIX_KS(probe_mix_bf16_exp, true, false)
 PROBE_ISSUE_MIX_KS(probe_mix_i8_fma, false, true)
 PROBE_ISSUE_MIX_KS(probe_mix_i8_exp, true, true)
+
+// How exactly the 8-bit floating-point matrix instructions add up their products: the dot product of
+// two vectors of 64 E4M3 codes, once with the 64-deep scaled instruction and once with four 16-deep
+// ones (every lane half takes the same bytes of both operands, so every element of the result is the
+// same dot product whatever the operand layout is).  out[0] = 64-deep, out[1] = 4 x 16-deep.
+extern "C" __global__ void probe_fp8_dot64(const unsigned char *a, const unsigned char *b, float *out)
+{
+    typedef __attribute__((ext_vector_type(8))) int i32x8;
+    const int h = threadIdx.x >> 5;
+    i32x8 av, bv;
+    for (int j = 0; j < 8; ++j) {
+        av[j] = ((const int *)(a + 32 * h))[j];
+        bv[j] = ((const int *)(b + 32 * h))[j];
+    }
+    f32x16 acc;
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 0, 0, 0, 0, 0, 0);
+    f32x16 acc2;
+    for (int r = 0; r < 16; ++r) acc2[r] = 0.f;
+    for (int s = 0; s < 4; ++s) {
+        const long a8 = *(const long *)(a + 16 * s + 8 * h), b8 = *(const long *)(b + 16 * s + 8 * h);
+        acc2 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a8, b8, acc2, 0, 0, 0);
+    }
+    if (threadIdx.x == 37) {
+        out[0] = acc[5];
+        out[1] = acc2[5];
+    }
+}

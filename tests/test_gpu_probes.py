@@ -77,3 +77,31 @@ def test_bf16_mfma_layout(dev, probes):
     assert np.array_equal(c.copyout(np.float32, (32, 32)), A @ B)
     for t in (a, b, c):
         t.free()
+
+
+def test_fp8_matrix_instructions_add_their_products_with_about_14_bits(dev, probes):
+    """The E4M3 matrix instructions (64-deep scaled and 16-deep) do not add their exact products in
+    fp32: against the exact dot product of 64 random codes they are off by up to ~6e-5 of the sum of
+    the absolute products (both instructions identically), where an fp32 accumulation would be within
+    1e-7.  This is why the FP8 attention follows a restatement of its own arithmetic only to the
+    extent the logits do (tests/test_gpu_pipe_kernel_order.py); the int8 instruction is exact and the
+    bf16 one is accurate to fp32 rounding (the layout tests above, the kernel-order tests)."""
+    import oracle
+    rng = np.random.default_rng(11)
+    out = dev.alloc(8)
+    worst = 0.0
+    for trial in range(20):
+        codes = rng.integers(0, 256, size=(2, 64)).astype(np.uint8)
+        codes[(codes & 0x7F) == 0x7F] = 0x38                      # no NaN codes
+        if trial >= 10:
+            codes &= 0x7F                                          # all positive: no cancellation
+        a, b = dev.from_numpy(codes[0]), dev.from_numpy(codes[1])
+        dev.launch(probes, "probe_fp8_dot64", (1, 1, 1), (64, 1, 1), [a, b, out])
+        got = out.copyout(np.float32, (2,)).astype(np.float64)
+        prod = oracle.fp8_e4m3_value(codes[0]).astype(np.float64) * oracle.fp8_e4m3_value(codes[1]).astype(np.float64)
+        rel = np.abs(got - prod.sum()) / np.abs(prod).sum()
+        assert got[0] == got[1]                                    # the two instructions agree bit for bit
+        worst = max(worst, float(rel.max()))
+        a.free(); b.free()
+    out.free()
+    assert 1e-6 < worst < 2e-4, worst                              # measured: 6e-5
