@@ -1,4 +1,4 @@
-"""The pipelined kernels (int8, bf16) against a numpy restatement of THEIR OWN order of operations
+"""The attention kernels (pipelined int8, bf16, FP8; short-sequence bf16) against a numpy restatement of THEIR OWN order of operations
 (autorust_amd/csrc/attn_pipe.h), wave by wave: 32-key blocks in sequence, the biased-float logits
 (12582912 + sum) * c' - m_bias with c' cut to 21 bits, the lazy exponent reference on its grid, the
 rescue path (row maximum, reference moved up to the grid, accumulators rescaled, block redone with

@@ -84,7 +84,7 @@ def test_fp8_matrix_instructions_add_their_products_with_about_14_bits(dev, prob
     fp32: against the exact dot product of 64 random codes they are off by up to ~6e-5 of the sum of
     the absolute products (both instructions identically), where an fp32 accumulation would be within
     1e-7.  This is why the FP8 attention follows a restatement of its own arithmetic only to the
-    extent the logits do (tests/test_gpu_pipe_kernel_order.py); the int8 instruction is exact and the
+    extent the logits do (tests/test_gpu_kernel_order.py); the int8 instruction is exact and the
     bf16 one is accurate to fp32 rounding (the layout tests above, the kernel-order tests)."""
     import oracle
     rng = np.random.default_rng(11)
