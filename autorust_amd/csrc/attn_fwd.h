@@ -485,6 +485,9 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
         load_kf(kl, 0);
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
+            // a second block whose keys are all hidden from every query of the wave (past the key length,
+            // or above the causal diagonal) contributes exact zeros and leaves the reference alone
+            if (GENERIC && blk == 1 && (k0 + 32 >= kend || (CAUSAL && k0 + 32 > wq0 + 31))) break;
             uint4 pb[2];
             // ---- P1 ----
             load_vf(vl, blk);
