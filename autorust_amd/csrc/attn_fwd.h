@@ -263,8 +263,9 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
                 if (full) {
                     kst[slot][j] = *(const uint4 *)(kbase + (size_t)gr * k_rs * QK_BYTES + col * 16);
                 } else {
-                    uint4 val = *(const uint4 *)(kbase + (size_t)min(gr, kend - 1) * k_rs * QK_BYTES + col * 16);
-                    if (gr >= kend) val = make_uint4(0, 0, 0, 0);
+                    // rows past the last visible key are zeros and cost no memory transaction
+                    uint4 val = make_uint4(0, 0, 0, 0);
+                    if (gr < kend) val = *(const uint4 *)(kbase + (size_t)gr * k_rs * QK_BYTES + col * 16);
                     kst[slot][j] = val;
                 }
             }
@@ -278,8 +279,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
                 if (full) {
                     vst[slot][j] = *(const uint4 *)(vbase + (size_t)gr * v_rs + col * 8);
                 } else {
-                    uint4 val = *(const uint4 *)(vbase + (size_t)min(gr, kend - 1) * v_rs + col * 8);
-                    if (gr >= kend) val = make_uint4(0, 0, 0, 0);
+                    uint4 val = make_uint4(0, 0, 0, 0);
+                    if (gr < kend) val = *(const uint4 *)(vbase + (size_t)gr * v_rs + col * 8);
                     vst[slot][j] = val;
                 }
             }
@@ -525,28 +526,39 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
         }
         if constexpr (KSPLIT == 2) {
             // merge the two key halves: m = max, l and O rescaled by 2^(m_part - m)
-            constexpr int SLAB = DB * 16 * 64 + 128;  // floats per query group: O, then m and l, lane-major
+            // per query group: O as float4 [DB * 4][64 lanes], then (m, l) as float2 [64 lanes]: 16-byte
+            // accesses at consecutive addresses, lane-major
+            constexpr int SLAB = DB * 16 * 64 + 128;  // floats per query group
             static_assert(QW * SLAB * 4 <= NSTAGE * STAGE, "merge buffer fits the tile stages");
             __syncthreads();  // every wave is done with the tiles
             float *mb = (float *)lds + qwave * SLAB;
+            float4 *mb4 = (float4 *)mb;
+            float2 *ml = (float2 *)(mb + DB * 16 * 64);
             if (kpart == 1) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) mb[(db * 16 + r) * 64 + lane] = oacc[db][r];
-                mb[DB * 16 * 64 + lane] = m_run;
-                mb[DB * 16 * 64 + 64 + lane] = l_run;
+                    for (int g = 0; g < 4; ++g)
+                        mb4[(db * 4 + g) * 64 + lane] = make_float4(oacc[db][4 * g], oacc[db][4 * g + 1], oacc[db][4 * g + 2], oacc[db][4 * g + 3]);
+                ml[lane] = make_float2(m_run, l_run);
             }
             __syncthreads();
             if (kpart == 1) return;
-            const float m1 = mb[DB * 16 * 64 + lane], l1 = mb[DB * 16 * 64 + 64 + lane];
+            const float2 ml1 = ml[lane];
+            const float m1 = ml1.x, l1 = ml1.y;
             const float m = fmaxf(m_run, m1);
             const float f0 = __builtin_amdgcn_exp2f(m_run - m), f1 = __builtin_amdgcn_exp2f(m1 - m);
             l_run = l_run * f0 + l1 * f1;
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[db][r] = oacc[db][r] * f0 + mb[(db * 16 + r) * 64 + lane] * f1;
+                for (int g = 0; g < 4; ++g) {
+                    const float4 o1 = mb4[(db * 4 + g) * 64 + lane];
+                    oacc[db][4 * g + 0] = oacc[db][4 * g + 0] * f0 + o1.x * f1;
+                    oacc[db][4 * g + 1] = oacc[db][4 * g + 1] * f0 + o1.y * f1;
+                    oacc[db][4 * g + 2] = oacc[db][4 * g + 2] * f0 + o1.z * f1;
+                    oacc[db][4 * g + 3] = oacc[db][4 * g + 3] * f0 + o1.w * f1;
+                }
             m_run = m;
         }
     } else {
