@@ -36,6 +36,7 @@ struct FlashBwdParams {
 };
 
 constexpr float BWD_LSE_FLOOR = -5e29f;  // lse at or below: the row saw no key (cuda_flash_train.rs:206)
+constexpr float BWD_LOG2E = 1.44269504088896340736f;
 
 // D[bh, i] = O[i] . dO[i]; one wave per row group: lane l of a wave sums channels l, l + 64, ...
 // in increasing order, then the 64 partial sums are added by a fixed butterfly.
@@ -109,6 +110,8 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
     const float lse = p.lse[(size_t)bh * N + rr];
     const float di = p.delta[(size_t)bh * N + rr];
     const bool row_live = lse > BWD_LSE_FLOOR;
+    // P = exp(x - lse) as v_exp_f32 (base 2) of x * log2(e) - lse * log2(e)
+    const float c2 = p.scale * BWD_LOG2E, lse2 = lse * BWD_LOG2E;
 
     f32x16_t acc[DB];
 #pragma unroll
@@ -168,10 +171,10 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int key = k0 + 8 * (r >> 2) + 4 * h + (r & 3);
-            float xv = s[r] * p.scale;
-            if (p.mask != nullptr && key < N) xv += p.mask[(size_t)rr * N + key];
+            float xv = fmaf(s[r], c2, -lse2);
+            if (p.mask != nullptr && key < N) xv = fmaf(p.mask[(size_t)rr * N + key], BWD_LOG2E, xv);
             const bool dead = key >= kend || (CAUSAL && key > q_row) || !row_live;
-            const float pr = dead ? 0.f : expf(xv - lse);
+            const float pr = dead ? 0.f : __builtin_amdgcn_exp2f(xv);
             ds[r] = pr * (dp[r] - di) * p.scale;
         }
         // dQ^T += K^T dS^T: step (g, t) multiplies key 8 g + 4 h + t
@@ -227,6 +230,7 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
         kvl = kvl < 0 ? 0 : (kvl > N ? N : kvl);
     }
     const bool key_live = key < kvl;
+    const float c2 = p.scale * BWD_LOG2E;
 
     float kr[HALF], vr[HALF];
     {
@@ -286,7 +290,7 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
             *(float4 *)&dos[row * ROW + col] = dx[j];
         }
         if (tid < F32_BK) {
-            stat[tid] = st_l;
+            stat[tid] = st_l * BWD_LOG2E;   // base-2 units: P = 2^(x log2(e) - lse log2(e))
             stat[32 + tid] = st_d;
         }
         if (step + 1 < steps) fetch(step + 1);
@@ -322,10 +326,10 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
             for (int t = 0; t < 4; ++t) {
                 const int r = 4 * gq + t;
                 const int qi = q0 + 8 * gq + 4 * h + t;
-                float xv = s[r] * p.scale;
-                if (p.mask != nullptr && qi < N) xv += p.mask[(size_t)qi * N + jj];
+                float xv = fmaf(s[r], c2, -lv[t]);
+                if (p.mask != nullptr && qi < N) xv = fmaf(p.mask[(size_t)qi * N + jj], BWD_LOG2E, xv);
                 const bool dead = qi >= N || !key_live || (CAUSAL && key > qi) || !(lv[t] > BWD_LSE_FLOOR);
-                pr[r] = dead ? 0.f : expf(xv - lv[t]);
+                pr[r] = dead ? 0.f : __builtin_amdgcn_exp2f(xv);
                 ds[r] = pr[r] * (dp[r] - dvv[t]) * p.scale;
             }
         }

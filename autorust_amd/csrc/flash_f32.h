@@ -1,8 +1,10 @@
 // fp32 exact-mode FlashAttention forward: no reduced precision anywhere.
 //
 // Semantics of the reference's scalar kernel (src/runtime/cuda_flash.rs:53-141): fp32 products
-// and sums, `expf`, finite sentinel -1e30 for masked keys, acc * (l > 0 ? 1/l : 0) at the end;
-// head_dim and scale are parameters here (the reference hard-codes 64 and 0.125).
+// and sums, fp32 exponentials, finite sentinel -1e30 for masked keys, acc * (l > 0 ? 1/l : 0) at
+// the end; head_dim and scale are parameters here (the reference hard-codes 64 and 0.125).  The
+// exponential is v_exp_f32 (base 2, 1 ulp) on logits scaled by scale * log2(e), where the reference
+// calls expf on logits scaled by scale: the same function to a few ulp.
 //
 // The two contractions run on the fp32 matrix instruction v_mfma_f32_32x32x2_f32 (fp32 in,
 // fp32 accumulate) with the same decomposition as the bf16 kernel: a wave owns 32 queries and
@@ -18,6 +20,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace arhip {
 
@@ -63,7 +66,8 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     constexpr int PER_THREAD = (CHUNKS + T - 1) / T;
     static_assert(CHUNKS % T == 0, "tile staging must divide evenly");
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar: tile indices and K/V tile addresses stay scalar
     constexpr int SLAB = F32_BK * KROW + F32_BK * D;
     float *ks = lds + (SPLITK ? wave * SLAB : 0);  // [F32_BK][KROW]
     float *vs = ks + F32_BK * KROW;                // [F32_BK][D]
@@ -91,8 +95,8 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     const int kvh = head / (p.Hq / p.Hkv);
     const size_t kv_off = (size_t)b * p.ks[0] + (size_t)kvh * p.ks[1];
     const size_t k_rs = (size_t)p.ks[2];
-    const float *kp = p.k + kv_off;
-    const float *vp = p.v + kv_off;
+    const char *kp = (const char *)(p.k + kv_off);
+    const char *vp = (const char *)(p.v + kv_off);
 
     // Q: this lane's half of its query row (rows past N read row N-1; never stored)
     float qr[HALF];
@@ -110,41 +114,46 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+    // The softmax runs on base-2 exponentials: logits are scaled by scale * log2(e) and the running
+    // maximum is kept in those units (one multiply-add and one v_exp_f32 per logit).
+    constexpr float LOG2E = 1.44269504088896340736f, LN2 = 0.69314718055994530942f;
+    const float c2 = p.scale * LOG2E;
     float m_run = -1e30f, l_run = 0.f;
 
     // The global loads of a tile are issued one tile ahead of its use, into registers, so that
-    // their latency is spent under the matrix instructions of the tile before.
+    // their latency is spent under the matrix instructions of the tile before.  Thread t stages
+    // rows t / (D/4) + j * RPJ, 16 bytes at column 4 * (t % (D/4)): a per-thread byte offset on top
+    // of a scalar address per (tile, j).
+    constexpr int RPJ = T / (D / 4);
+    const int row0 = stid / (D / 4), col0 = (stid % (D / 4)) * 4;
+    const size_t voff = ((size_t)row0 * k_rs + col0) * sizeof(float);
     float4 kx[PER_THREAD], vx[PER_THREAD];
     auto fetch = [&](int tile) __attribute__((always_inline)) {
+        const size_t t0 = (size_t)tile * F32_BK * k_rs * sizeof(float);
+        if (tile * F32_BK + F32_BK <= kend) {
 #pragma unroll
-        for (int j = 0; j < PER_THREAD; ++j) {
-            const int c = stid + j * T;
-            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-            const int gr = tile * F32_BK + row;
-            kx[j] = vx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (gr < kend) {
-                kx[j] = *(const float4 *)(kp + (size_t)gr * k_rs + col);
-                vx[j] = *(const float4 *)(vp + (size_t)gr * k_rs + col);
+            for (int j = 0; j < PER_THREAD; ++j) {
+                const size_t so = t0 + (size_t)j * RPJ * k_rs * sizeof(float);
+                kx[j] = *(const float4 *)(kp + so + voff);
+                vx[j] = *(const float4 *)(vp + so + voff);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < PER_THREAD; ++j) {
+                const size_t so = t0 + (size_t)j * RPJ * k_rs * sizeof(float);
+                kx[j] = vx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (tile * F32_BK + row0 + j * RPJ < kend) {
+                    kx[j] = *(const float4 *)(kp + so + voff);
+                    vx[j] = *(const float4 *)(vp + so + voff);
+                }
             }
         }
     };
-    constexpr int STEP = SPLITK ? NW : 1;
-    const int first = SPLITK ? wave : 0;
-    if (first < ntiles) fetch(first);
-    for (int it = first; it < ntiles; it += STEP) {
-        const int k0 = it * F32_BK;
-        if (!SPLITK) __syncthreads();  // the previous tile has been consumed
-#pragma unroll
-        for (int j = 0; j < PER_THREAD; ++j) {
-            const int c = stid + j * T;
-            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-            *(float4 *)&ks[row * KROW + col] = kx[j];
-            *(float4 *)&vs[row * D + col] = vx[j];
-        }
-        if (it + STEP < ntiles) fetch(it + STEP);
-        if (!SPLITK) __syncthreads();
-        if (it >= my_tiles) continue;  // under the causal mask this wave is done (it still helps staging)
 
+    // one key tile; GENERIC: additive mask, keys past the end or hidden by the causal mask, or a
+    // negative scale (the plain path takes the maximum before scaling)
+    auto tile_body = [&](auto generic, int k0) __attribute__((always_inline)) {
+        constexpr bool GENERIC = decltype(generic)::value;
         // ---- S^T = K . Q^T ----
         f32x16_t s;
 #pragma unroll
@@ -152,35 +161,45 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
         const float *krow = &ks[i32 * KROW + h * HALF];
 #pragma unroll
         for (int st = 0; st < HALF; st += 4) {
-            const float4 kx = *(const float4 *)(krow + st);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx.x, qr[st + 0], s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx.y, qr[st + 1], s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx.z, qr[st + 2], s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kx.w, qr[st + 3], s, 0, 0, 0);
+            const float4 kq = *(const float4 *)(krow + st);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kq.x, qr[st + 0], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kq.y, qr[st + 1], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kq.z, qr[st + 2], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kq.w, qr[st + 3], s, 0, 0, 0);
         }
 
-        // ---- scale, masks, online softmax (natural exponent, like the reference) ----
+        // ---- scale, masks, online softmax ----
         float x[16];
-        float mx = -1e30f;
+        float m_new;
+        if constexpr (GENERIC) {
+            float mx = -1e30f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int key = k0 + 8 * (r >> 2) + 4 * h + (r & 3);
-            float xv = s[r] * p.scale;
-            if (p.mask != nullptr && key < N && q_row < N) xv += p.mask[(size_t)q_row * N + key];
-            if (key >= kend || (CAUSAL && key > q_row)) xv = -1e30f;
-            x[r] = xv;
-            mx = fmaxf(mx, xv);
+            for (int r = 0; r < 16; ++r) {
+                const int key = k0 + 8 * (r >> 2) + 4 * h + (r & 3);
+                float xv = s[r] * c2;
+                if (p.mask != nullptr && key < N && q_row < N) xv = fmaf(p.mask[(size_t)q_row * N + key], LOG2E, xv);
+                if (key >= kend || (CAUSAL && key > q_row)) xv = -1e30f;
+                x[r] = xv;
+                mx = fmaxf(mx, xv);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            m_new = fmaxf(m_run, mx);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+        } else {
+            float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+            for (int r = 2; r < 16; ++r) mx = fmaxf(mx, s[r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            m_new = fmaxf(m_run, mx * c2);   // c2 >= 0 here: the largest logit is the largest product
+#pragma unroll
+            for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -m_new));
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = expf(m_run - m_new);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;
         float rs = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            x[r] = expf(x[r] - m_new);
-            rs += x[r];
-        }
+        for (int r = 0; r < 16; ++r) rs += x[r];
         l_run = l_run * alpha + rs;
         if (__any(alpha != 1.0f)) {
 #pragma unroll
@@ -197,6 +216,27 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
             for (int db = 0; db < DB; ++db)
                 oacc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[db * 32], x[r], oacc[db], 0, 0, 0);
         }
+    };
+
+    const bool always_generic = p.mask != nullptr || !(c2 >= 0.f);
+    constexpr int STEP = SPLITK ? NW : 1;
+    const int first = SPLITK ? wave : 0;
+    if (first < ntiles) fetch(first);
+    for (int it = first; it < ntiles; it += STEP) {
+        const int k0 = it * F32_BK;
+        if (!SPLITK) __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+        for (int j = 0; j < PER_THREAD; ++j) {
+            *(float4 *)&ks[(row0 + j * RPJ) * KROW + col0] = kx[j];
+            *(float4 *)&vs[(row0 + j * RPJ) * D + col0] = vx[j];
+        }
+        if (it + STEP < ntiles) fetch(it + STEP);
+        if (!SPLITK) __syncthreads();
+        if (it >= my_tiles) continue;  // under the causal mask this wave is done (it still helps staging)
+        if (always_generic || k0 + F32_BK > kend || (CAUSAL && k0 + F32_BK - 1 > wq0))
+            tile_body(std::true_type{}, k0);
+        else
+            tile_body(std::false_type{}, k0);
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
@@ -230,7 +270,7 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
         for (int c = 0; c < CPT; ++c) acc[c] = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
-            const float f = expf(lds[w * SLAB + 32 * OROW + q] - m);
+            const float f = __builtin_amdgcn_exp2f(lds[w * SLAB + 32 * OROW + q] - m);
             l += lds[w * SLAB + 32 * OROW + 32 + q] * f;
 #pragma unroll
             for (int c = 0; c < CPT; c += 4) {
@@ -240,7 +280,7 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
         }
         const float inv = (l > 0.f) ? 1.f / l : 0.f;
         if (row < N) {
-            if (p.lse != nullptr && cg == 0) p.lse[(size_t)bh * N + row] = (l > 0.f) ? m + logf(l) : -1e30f;
+            if (p.lse != nullptr && cg == 0) p.lse[(size_t)bh * N + row] = (l > 0.f) ? m * LN2 + logf(l) : -1e30f;
             float *op = p.o + (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)row * p.os[2] + cg * CPT;
 #pragma unroll
             for (int c = 0; c < CPT; c += 4)
@@ -250,7 +290,7 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     }
     const float inv = (l_tot > 0.f) ? 1.f / l_tot : 0.f;
     if (p.lse != nullptr && h == 0 && q_row < N)
-        p.lse[(size_t)bh * N + q_row] = (l_tot > 0.f) ? m_run + logf(l_tot) : -1e30f;
+        p.lse[(size_t)bh * N + q_row] = (l_tot > 0.f) ? m_run * LN2 + logf(l_tot) : -1e30f;
     if (q_row < N) {
         float *op = p.o + (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)q_row * p.os[2];
 #pragma unroll
@@ -265,7 +305,7 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
 }
 
 template <int D, int NW, bool CAUSAL, bool SPLITK = false>
-__global__ void __launch_bounds__(NW * 64) flash_f32_kernel(const FlashF32Params p)
+__global__ void __launch_bounds__(NW * 64, 2) flash_f32_kernel(const FlashF32Params p)
 {
     __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<D, NW, SPLITK>()];
     flash_f32_body<D, NW, CAUSAL, SPLITK>(p, lds, (int)blockIdx.x);
