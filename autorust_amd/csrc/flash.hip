@@ -389,25 +389,27 @@ extern "C" int arhip_flash_bwd(arhip_device *dev, const float *q, const float *k
     p.scale = scale;
     if (int rc = t.begin()) return rc;
     const long rows = (long)(B * Hq * N);
-    // 4 waves (128 queries / keys) per workgroup when that fills the chip, else 1 wave (32)
-    const int nw = (B * Hkv * ((N + 127) / 128) >= 2 * (int64_t)dev->cus) ? 4 : 1;
-    const int nt = (int)((N + nw * 32 - 1) / (nw * 32));
-    const dim3 block((unsigned)(nw * 64)), grid_prep((unsigned)((rows + 3) / 4)), grid_q((unsigned)(nt * B * Hq)),
+    // 4 waves per workgroup: 128 queries / keys when that still fills the chip, else the same 32
+    // queries / keys with the tiles of the other side dealt out between the waves
+    const bool split = B * Hkv * ((N + 127) / 128) < 2 * (int64_t)dev->cus;
+    const int rows_wg = split ? 32 : 128;
+    const int nt = (int)((N + rows_wg - 1) / rows_wg);
+    const dim3 block(256), grid_prep((unsigned)((rows + 3) / 4)), grid_q((unsigned)(nt * B * Hq)),
         grid_kv((unsigned)(nt * B * Hkv));
     p.nt = nt;
-#define BWD_LAUNCH(DD, NWW)                                                                             \
+#define BWD_LAUNCH(DD, SP)                                                                              \
     do {                                                                                                \
         hipLaunchKernelGGL((bwd_prep_kernel<DD>), grid_prep, dim3(256), 0, dev->stream, o, dout, delta, rows); \
         if (causal) {                                                                                   \
-            hipLaunchKernelGGL((bwd_dq_kernel<DD, NWW, true>), grid_q, block, 0, dev->stream, p);       \
-            hipLaunchKernelGGL((bwd_dkv_kernel<DD, NWW, true>), grid_kv, block, 0, dev->stream, p);     \
+            hipLaunchKernelGGL((bwd_dq_kernel<DD, 4, true, SP>), grid_q, block, 0, dev->stream, p);     \
+            hipLaunchKernelGGL((bwd_dkv_kernel<DD, 4, true, SP>), grid_kv, block, 0, dev->stream, p);   \
         } else {                                                                                        \
-            hipLaunchKernelGGL((bwd_dq_kernel<DD, NWW, false>), grid_q, block, 0, dev->stream, p);      \
-            hipLaunchKernelGGL((bwd_dkv_kernel<DD, NWW, false>), grid_kv, block, 0, dev->stream, p);    \
+            hipLaunchKernelGGL((bwd_dq_kernel<DD, 4, false, SP>), grid_q, block, 0, dev->stream, p);    \
+            hipLaunchKernelGGL((bwd_dkv_kernel<DD, 4, false, SP>), grid_kv, block, 0, dev->stream, p);  \
         }                                                                                               \
     } while (0)
-    if (D == 64) { if (nw == 4) BWD_LAUNCH(64, 4); else BWD_LAUNCH(64, 1); }
-    else { if (nw == 4) BWD_LAUNCH(128, 4); else BWD_LAUNCH(128, 1); }
+    if (D == 64) { if (split) BWD_LAUNCH(64, true); else BWD_LAUNCH(64, false); }
+    else { if (split) BWD_LAUNCH(128, true); else BWD_LAUNCH(128, false); }
 #undef BWD_LAUNCH
     arhip_note_selected(ARHIP_K_FLASH_BWD);
     return t.end();

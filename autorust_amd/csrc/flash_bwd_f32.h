@@ -54,18 +54,24 @@ __device__ __forceinline__ void bwd_prep_body(const float *o, const float *dout,
     if (lane == 0) delta[row] = s;
 }
 
-template <int D>
+// LDS floats of the dQ and dK/dV bodies: two padded 32-row tiles and 64 row statistics (one such slab
+// per wave with SPLIT)
+template <int D, int NW = 1, bool SPLIT = false>
 constexpr int bwd_lds_floats()
 {
-    return 2 * F32_BK * (D + 4) + 64;
+    return (SPLIT ? NW : 1) * (2 * F32_BK * (D + 4) + 64);
 }
 
-// dQ.  lds: bwd_lds_floats<D>() floats.  Workgroup wg_linear in [0, nt * B * Hq): 32 NW queries of one head.
-template <int D, int NW, bool CAUSAL>
+// dQ.  lds: bwd_lds_floats<D, NW, SPLIT>() floats.  Workgroup wg_linear in [0, nt * B * Hq): 32 NW queries
+// of one head.  SPLIT (few, short heads: one wave per workgroup would leave each SIMD a long chain of
+// matrix instructions and most of the chip idle): the NW waves share the same 32 queries and deal the
+// key tiles out between them (wave w takes tiles w, w + NW, ...), each staging its tiles in its own
+// LDS slab with no workgroup barrier; the partial dQ of the waves are added through LDS in wave order.
+template <int D, int NW, bool CAUSAL, bool SPLIT = false>
 __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds, int wg_linear)
 {
-    constexpr int T = NW * 64;
-    constexpr int BQ = NW * 32;
+    constexpr int T = SPLIT ? 64 : NW * 64;   // threads staging one tile
+    constexpr int BQ = SPLIT ? 32 : NW * 32;
     constexpr int HALF = D / 2;
     constexpr int ROW = D + 4;  // padded row: conflict-free 128-bit row reads
     constexpr int DB = D / 32;
@@ -73,9 +79,12 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
     constexpr int PER_THREAD = CHUNKS / T;
     static_assert(CHUNKS % T == 0, "tile staging must divide evenly");
 
-    float *ks = lds;
-    float *vs = lds + F32_BK * ROW;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int SLAB = 2 * F32_BK * ROW + 64;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    float *ks = lds + (SPLIT ? wave * SLAB : 0);
+    float *vs = ks + F32_BK * ROW;
+    const int stid = SPLIT ? lane : tid;      // index among the threads staging a tile
     const int i32 = lane & 31, h = lane >> 5;
     const int bh = wg_linear / p.nt;
     int qt = wg_linear - bh * p.nt;
@@ -83,7 +92,8 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
     const int b = bh / p.Hq, head = bh - b * p.Hq;
     const int N = p.N;
     const int qblk = qt * BQ;
-    const int q_row = qblk + wave * 32 + i32;
+    const int wq0 = qblk + (SPLIT ? 0 : wave * 32);
+    const int q_row = wq0 + i32;
     const int rr = min(q_row, N - 1);
     int kvl = N;
     if (p.kv_len) {
@@ -93,7 +103,7 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
     int kend = kvl;
     if (CAUSAL) kend = min(kend, min(N, qblk + BQ));
     const int ntiles = (kend + F32_BK - 1) / F32_BK;
-    const int my_tiles = CAUSAL ? min(ntiles, (qblk + wave * 32 + 31) / F32_BK + 1) : ntiles;
+    const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / F32_BK + 1) : ntiles;
     const int kvh = head / (p.Hq / p.Hkv);
     const float *kp = p.k + ((size_t)b * p.Hkv + kvh) * (size_t)N * D;
     const float *vp = p.v + ((size_t)b * p.Hkv + kvh) * (size_t)N * D;
@@ -123,7 +133,7 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
     auto fetch = [&](int tile) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < PER_THREAD; ++j) {
-            const int c = tid + j * T;
+            const int c = stid + j * T;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
             const int gr = tile * F32_BK + row;
             kx[j] = vx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -133,19 +143,21 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
             }
         }
     };
-    if (ntiles > 0) fetch(0);
-    for (int it = 0; it < ntiles; ++it) {
+    constexpr int STEP = SPLIT ? NW : 1;
+    const int first = SPLIT ? wave : 0;
+    if (first < ntiles) fetch(first);
+    for (int it = first; it < ntiles; it += STEP) {
         const int k0 = it * F32_BK;
-        __syncthreads();
+        if (!SPLIT) __syncthreads();
 #pragma unroll
         for (int j = 0; j < PER_THREAD; ++j) {
-            const int c = tid + j * T;
+            const int c = stid + j * T;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
             *(float4 *)&ks[row * ROW + col] = kx[j];
             *(float4 *)&vs[row * ROW + col] = vx[j];
         }
-        if (it + 1 < ntiles) fetch(it + 1);
-        __syncthreads();
+        if (it + STEP < ntiles) fetch(it + STEP);
+        if (!SPLIT) __syncthreads();
         if (it >= my_tiles) continue;
 
         // S^T = K Q^T and dP^T = V dO^T: lane = query, register r = key 8 (r / 4) + 4 h + r % 4
@@ -186,6 +198,35 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
                 acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(kcol[db * 32], ds[r], acc[db], 0, 0, 0);
         }
     }
+    if constexpr (SPLIT) {
+        // the waves' partial sums, each as [32 queries][ROW] in its own slab (its tiles are consumed)
+        float *ow = lds + wave * SLAB;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                *(float4 *)&ow[i32 * ROW + db * 32 + 8 * g + 4 * h] =
+                    make_float4(acc[db][4 * g], acc[db][4 * g + 1], acc[db][4 * g + 2], acc[db][4 * g + 3]);
+        __syncthreads();
+        // thread t: query t % 32, channels [cg * CPT, cg * CPT + CPT)
+        constexpr int CPT = D / (NW * 2);
+        static_assert(CPT % 4 == 0, "whole float4s per thread");
+        const int q = tid & 31, cg = tid >> 5;
+        if (qblk + q < N) {
+            float *op = p.dq + ((size_t)bh * N + qblk + q) * D + cg * CPT;
+#pragma unroll
+            for (int c = 0; c < CPT; c += 4) {
+                float4 sum = *(const float4 *)&lds[q * ROW + cg * CPT + c];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) {
+                    const float4 x = *(const float4 *)&lds[w * SLAB + q * ROW + cg * CPT + c];
+                    sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+                }
+                *(float4 *)(op + c) = sum;
+            }
+        }
+        return;
+    }
     if (q_row < N) {
         float *op = p.dq + ((size_t)bh * N + q_row) * D;
 #pragma unroll
@@ -197,12 +238,14 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
     }
 }
 
-// dK and dV.  Workgroup wg_linear in [0, nt * B * Hkv): 32 NW keys of one K/V head.
-template <int D, int NW, bool CAUSAL>
+// dK and dV.  Workgroup wg_linear in [0, nt * B * Hkv): 32 NW keys of one K/V head.  SPLIT: the NW waves
+// share the same 32 keys and deal the (head of the group, query tile) steps out between them, each in
+// its own LDS slab; the partial dK and dV of the waves are added through LDS in wave order.
+template <int D, int NW, bool CAUSAL, bool SPLIT = false>
 __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds, int wg_linear)
 {
-    constexpr int T = NW * 64;
-    constexpr int BKW = NW * 32;  // keys per workgroup
+    constexpr int T = SPLIT ? 64 : NW * 64;   // threads staging one tile
+    constexpr int BKW = SPLIT ? 32 : NW * 32;  // keys per workgroup
     constexpr int HALF = D / 2;
     constexpr int ROW = D + 4;
     constexpr int DB = D / 32;
@@ -210,10 +253,13 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
     constexpr int PER_THREAD = CHUNKS / T;
     static_assert(CHUNKS % T == 0, "tile staging must divide evenly");
 
-    float *qs = lds;
-    float *dos = lds + F32_BK * ROW;
-    float *stat = lds + 2 * F32_BK * ROW;  // lse[32], D[32] of the staged queries
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int SLAB = 2 * F32_BK * ROW + 64;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    float *qs = lds + (SPLIT ? wave * SLAB : 0);
+    float *dos = qs + F32_BK * ROW;
+    float *stat = qs + 2 * F32_BK * ROW;  // lse[32], D[32] of the staged queries
+    const int stid = SPLIT ? lane : tid;      // index among the threads staging a tile
     const int i32 = lane & 31, h = lane >> 5;
     const int kv_bh = wg_linear / p.nt;
     const int kt = wg_linear - kv_bh * p.nt;
@@ -221,7 +267,7 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
     const int group = p.Hq / p.Hkv;
     const int N = p.N;
     const int kblk = kt * BKW;
-    const int wk0 = kblk + wave * 32;
+    const int wk0 = kblk + (SPLIT ? 0 : wave * 32);
     const int key = wk0 + i32;
     const int jj = min(key, N - 1);
     int kvl = N;
@@ -262,7 +308,7 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
         const size_t bh = (size_t)b * p.Hq + (size_t)kvh * group + g;
 #pragma unroll
         for (int j = 0; j < PER_THREAD; ++j) {
-            const int c = tid + j * T;
+            const int c = stid + j * T;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
             const int gr = q0 + row;
             qx[j] = dx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -271,30 +317,32 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
                 dx[j] = *(const float4 *)(p.dout + (bh * N + gr) * D + col);
             }
         }
-        if (tid < F32_BK) {
-            const int gr = q0 + tid;
+        if (stid < F32_BK) {
+            const int gr = q0 + stid;
             st_l = gr < N ? p.lse[bh * N + gr] : -1e30f;
             st_d = gr < N ? p.delta[bh * N + gr] : 0.f;
         }
     };
-    if (steps > 0) fetch(0);
-    for (int step = 0; step < steps; ++step) {
+    constexpr int STEP = SPLIT ? NW : 1;
+    const int first = SPLIT ? wave : 0;
+    if (first < steps) fetch(first);
+    for (int step = first; step < steps; step += STEP) {
         const int g = step / (qtiles - qt0);
         const int q0 = (qt0 + step - g * (qtiles - qt0)) * F32_BK;
-        __syncthreads();
+        if (!SPLIT) __syncthreads();
 #pragma unroll
         for (int j = 0; j < PER_THREAD; ++j) {
-            const int c = tid + j * T;
+            const int c = stid + j * T;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
             *(float4 *)&qs[row * ROW + col] = qx[j];
             *(float4 *)&dos[row * ROW + col] = dx[j];
         }
-        if (tid < F32_BK) {
-            stat[tid] = st_l * BWD_LOG2E;   // base-2 units: P = 2^(x log2(e) - lse log2(e))
-            stat[32 + tid] = st_d;
+        if (stid < F32_BK) {
+            stat[stid] = st_l * BWD_LOG2E;   // base-2 units: P = 2^(x log2(e) - lse log2(e))
+            stat[32 + stid] = st_d;
         }
-        if (step + 1 < steps) fetch(step + 1);
-        __syncthreads();
+        if (step + STEP < steps) fetch(step + STEP);
+        if (!SPLIT) __syncthreads();
         if (CAUSAL && q0 + F32_BK - 1 < wk0) continue;  // every query of the tile precedes this wave's keys
 
         // S = Q K^T and dP = dO V^T: lane = key, register r = query 8 (r / 4) + 4 h + r % 4 of the tile
@@ -346,6 +394,41 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
             }
         }
     }
+    if constexpr (SPLIT) {
+        // the waves' partial sums: dK as [32 keys][ROW] in the first tile of the slab, dV in the second
+        float *ow = lds + wave * SLAB;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = db * 32 + 8 * g + 4 * h;
+                *(float4 *)&ow[i32 * ROW + d] = make_float4(dk[db][4 * g], dk[db][4 * g + 1], dk[db][4 * g + 2], dk[db][4 * g + 3]);
+                *(float4 *)&ow[(F32_BK + i32) * ROW + d] = make_float4(dv[db][4 * g], dv[db][4 * g + 1], dv[db][4 * g + 2], dv[db][4 * g + 3]);
+            }
+        __syncthreads();
+        // thread t: key t % 32, channels [cg * CPT, cg * CPT + CPT) of dK and of dV
+        constexpr int CPT = D / (NW * 2);
+        static_assert(CPT % 4 == 0, "whole float4s per thread");
+        const int kq = tid & 31, cg = tid >> 5;
+        if (kblk + kq < N) {
+            const size_t orow = ((size_t)kv_bh * N + kblk + kq) * D + cg * CPT;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                float *op = (half ? p.dv : p.dk) + orow;
+#pragma unroll
+                for (int c = 0; c < CPT; c += 4) {
+                    float4 sum = *(const float4 *)&lds[(half * F32_BK + kq) * ROW + cg * CPT + c];
+#pragma unroll
+                    for (int w = 1; w < NW; ++w) {
+                        const float4 x = *(const float4 *)&lds[w * SLAB + (half * F32_BK + kq) * ROW + cg * CPT + c];
+                        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+                    }
+                    *(float4 *)(op + c) = sum;
+                }
+            }
+        }
+        return;
+    }
     if (key < N) {
         float *okp = p.dk + ((size_t)kv_bh * N + key) * D;
         float *ovp = p.dv + ((size_t)kv_bh * N + key) * D;
@@ -366,18 +449,18 @@ __global__ void __launch_bounds__(256) bwd_prep_kernel(const float *o, const flo
     bwd_prep_body<D>(o, dout, delta, rows, (long)blockIdx.x * 4);
 }
 
-template <int D, int NW, bool CAUSAL>
+template <int D, int NW, bool CAUSAL, bool SPLIT>
 __global__ void __launch_bounds__(NW * 64) bwd_dq_kernel(const FlashBwdParams p)
 {
-    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<D>()];
-    bwd_dq_body<D, NW, CAUSAL>(p, lds, (int)blockIdx.x);
+    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<D, NW, SPLIT>()];
+    bwd_dq_body<D, NW, CAUSAL, SPLIT>(p, lds, (int)blockIdx.x);
 }
 
-template <int D, int NW, bool CAUSAL>
+template <int D, int NW, bool CAUSAL, bool SPLIT>
 __global__ void __launch_bounds__(NW * 64) bwd_dkv_kernel(const FlashBwdParams p)
 {
-    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<D>()];
-    bwd_dkv_body<D, NW, CAUSAL>(p, lds, (int)blockIdx.x);
+    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<D, NW, SPLIT>()];
+    bwd_dkv_body<D, NW, CAUSAL, SPLIT>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

@@ -70,6 +70,19 @@ def test_backward_random_inputs(dev, D, causal, use_len, hkv):
         assert err <= 3e-5 * max(1.0, np.abs(w).max()), (name, err)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_backward_on_a_shape_that_fills_the_chip(dev, causal):
+    """B * Hkv * ceil(N / 128) = 512 workgroups: the variant with 128 queries / keys per workgroup
+    (shorter shapes deal the tiles of 32 queries / keys out between the four waves instead)."""
+    B, Hq, Hkv, N, D = 16, 8, 8, 512, 64
+    q, k, v, do = (synth.normal(s, (B, H, N, D)) for s, H in ((71, Hq), (72, Hkv), (73, Hkv), (74, Hq)))
+    want = oracle.attention_backward_f64(q, k, v, do, causal=causal)
+    got = run_fwd_bwd(dev, q, k, v, do, causal=causal)
+    for name, g, w in zip(("o", "lse", "dq", "dk", "dv"), got, want):
+        err = np.abs(g - w).max()
+        assert err <= 3e-5 * max(1.0, np.abs(w).max()), (name, err)
+
+
 def test_backward_is_deterministic_and_linear_in_dout(dev):
     B, Hq, Hkv, N, D = 1, 4, 2, 300, 64
     q, k, v, do = (synth.normal(s, (B, H, N, D)) for s, H in ((61, Hq), (62, Hkv), (63, Hkv), (64, Hq)))

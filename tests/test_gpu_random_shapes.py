@@ -1,7 +1,8 @@
 """Seeded random sweep over shapes, head groupings, masks and tiling variants: every case is
 compared with the float64 oracle.  The tiling variant does not change the function, so the
-same case is also run with the workgroup size forced (1, 4 and 8 waves)."""
-import os
+same case is also run with the workgroup size forced (1, 4 and 8 waves): ARHIP_ATTN_WAVES is read
+when a device is opened, so those runs open a device handle of their own."""
+import contextlib
 
 import numpy as np
 import pytest
@@ -12,6 +13,21 @@ from autorust_amd.device import BF16, F32
 from gpu_util import run_flash, run_sage
 
 pytestmark = pytest.mark.gpu
+
+
+@contextlib.contextmanager
+def _device_with_waves(dev, waves, monkeypatch):
+    """The session's device when nothing is forced, else a second handle opened under the override."""
+    if waves is None:
+        yield dev
+        return
+    from autorust_amd.device import Device
+    monkeypatch.setenv("ARHIP_ATTN_WAVES", waves)
+    forced = Device(0)
+    try:
+        yield forced
+    finally:
+        forced.close()
 
 
 def _cases(seed, count):
@@ -32,10 +48,11 @@ def _cases(seed, count):
 
 @pytest.mark.parametrize("waves", [None, "1", "4", "8"])
 def test_flash_random_shapes(dev, waves, monkeypatch):
-    if waves is None:
-        monkeypatch.delenv("ARHIP_ATTN_WAVES", raising=False)
-    else:
-        monkeypatch.setenv("ARHIP_ATTN_WAVES", waves)
+    with _device_with_waves(dev, waves, monkeypatch) as d:
+        _flash_random_shapes(d)
+
+
+def _flash_random_shapes(dev):
     worst = {BF16: 0.0, F32: 0.0}
     for (B, Hq, Hkv, N, D, causal, kv_len, seed) in _cases(1234, 24):
         q, k, v = (synth.normal(seed + i, s) for i, s in enumerate(((B, Hq, N, D), (B, Hkv, N, D), (B, Hkv, N, D))))
@@ -54,10 +71,11 @@ def test_flash_random_shapes(dev, waves, monkeypatch):
 
 @pytest.mark.parametrize("waves", [None, "4", "8"])
 def test_sage_random_shapes(dev, waves, monkeypatch):
-    if waves is None:
-        monkeypatch.delenv("ARHIP_ATTN_WAVES", raising=False)
-    else:
-        monkeypatch.setenv("ARHIP_ATTN_WAVES", waves)
+    with _device_with_waves(dev, waves, monkeypatch) as d:
+        _sage_random_shapes(d)
+
+
+def _sage_random_shapes(dev):
     for (B, Hq, Hkv, N, D, causal, kv_len, seed) in _cases(4321, 12):
         q, k, v = (synth.normal(seed + i, s) for i, s in enumerate(((B, Hq, N, D), (B, Hkv, N, D), (B, Hkv, N, D))))
         k = (k + np.float32(2.0) * synth.normal(seed + 9, (1, Hkv, 1, D))).astype(np.float32)
