@@ -166,23 +166,26 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
             fp.ks[i] = (long)kv_strides[i];
             fp.os[i] = (long)o_strides[i];
         }
-        // 4 waves per workgroup: 128 queries when that still fills the chip, else the same 32
-        // queries with the key tiles dealt out between the waves
+        // 128 queries per workgroup of 4 waves when that still fills the chip, else 32 queries whose key
+        // tiles are dealt out between the waves of the workgroup: 4 waves, or 2 when that lets every
+        // workgroup be resident at once (8 waves per CU) and 4 would need a second round
         const bool splitk = B * Hq * ((N + 127) / 128) < 2 * (int64_t)dev->cus;
         const int bq = splitk ? 32 : 128;
         fp.nq = (int)((N + bq - 1) / bq);
         fp.scale = scale;
+        const int64_t wgs = fp.nq * B * Hq;
+        const bool two = splitk && D == 64 && wgs > 2 * (int64_t)dev->cus && wgs <= 4 * (int64_t)dev->cus;
         if (int rc = t.begin()) return rc;
-        const dim3 grid((unsigned)(fp.nq * B * Hq)), block(256);
-#define F32_LAUNCH(DD, SK)                                                                            \
+        const dim3 grid((unsigned)wgs), block(two ? 128 : 256);
+#define F32_LAUNCH(DD, NWW, SK)                                                                         \
     do {                                                                                              \
-        if (causal) hipLaunchKernelGGL((flash_f32_kernel<DD, 4, true, SK>), grid, block, 0, dev->stream, fp);  \
-        else hipLaunchKernelGGL((flash_f32_kernel<DD, 4, false, SK>), grid, block, 0, dev->stream, fp); \
+        if (causal) hipLaunchKernelGGL((flash_f32_kernel<DD, NWW, true, SK>), grid, block, 0, dev->stream, fp);  \
+        else hipLaunchKernelGGL((flash_f32_kernel<DD, NWW, false, SK>), grid, block, 0, dev->stream, fp); \
     } while (0)
         if (D == 64) {
-            if (splitk) F32_LAUNCH(64, true); else F32_LAUNCH(64, false);
+            if (two) F32_LAUNCH(64, 2, true); else if (splitk) F32_LAUNCH(64, 4, true); else F32_LAUNCH(64, 4, false);
         } else {
-            if (splitk) F32_LAUNCH(128, true); else F32_LAUNCH(128, false);
+            if (splitk) F32_LAUNCH(128, 4, true); else F32_LAUNCH(128, 4, false);
         }
 #undef F32_LAUNCH
         arhip_note_selected(ARHIP_K_FLASH_F32);

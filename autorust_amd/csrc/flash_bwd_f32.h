@@ -449,15 +449,17 @@ __global__ void __launch_bounds__(256) bwd_prep_kernel(const float *o, const flo
     bwd_prep_body<D>(o, dout, delta, rows, (long)blockIdx.x * 4);
 }
 
+// D = 64: registers held to 256 per lane so that a SIMD holds two waves (the split dK/dV variant would
+// spill at that limit and keeps one)
 template <int D, int NW, bool CAUSAL, bool SPLIT>
-__global__ void __launch_bounds__(NW * 64) bwd_dq_kernel(const FlashBwdParams p)
+__global__ void __launch_bounds__(NW * 64, (D == 64 ? 2 : 1)) bwd_dq_kernel(const FlashBwdParams p)
 {
     __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<D, NW, SPLIT>()];
     bwd_dq_body<D, NW, CAUSAL, SPLIT>(p, lds, (int)blockIdx.x);
 }
 
 template <int D, int NW, bool CAUSAL, bool SPLIT>
-__global__ void __launch_bounds__(NW * 64) bwd_dkv_kernel(const FlashBwdParams p)
+__global__ void __launch_bounds__(NW * 64, (D == 64 && !SPLIT ? 2 : 1)) bwd_dkv_kernel(const FlashBwdParams p)
 {
     __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<D, NW, SPLIT>()];
     bwd_dkv_body<D, NW, CAUSAL, SPLIT>(p, lds, (int)blockIdx.x);

@@ -304,7 +304,7 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     }
 }
 
-// D = 64: two workgroups per CU (registers held to 256 per lane); D = 128 needs more than that
+// D = 64: two waves per SIMD (registers held to 256 per lane); D = 128 needs more than that
 template <int D, int NW, bool CAUSAL, bool SPLITK = false>
 __global__ void __launch_bounds__(NW * 64, (D == 64 ? 2 : 1)) flash_f32_kernel(const FlashF32Params p)
 {
