@@ -105,6 +105,27 @@ def test_edge_cases(dev):
     assert np.abs(got - truth).max() < 1e-5
 
 
+@pytest.mark.parametrize("N", [70, 333])
+def test_f32_scale_signs_wide_logits_and_additive_mask(dev, N):
+    """The fp32 kernel takes the row maximum before scaling on plain tiles, which only holds for a
+    scale >= 0: negative and zero scales, logits tens of units wide, and an additive mask (with -inf
+    entries) on top of the causal mask and key lengths all have to give the float64 result."""
+    B, Hq, Hkv, D = 2, 4, 2, 64
+    q, k, v = (synth.normal(s, (B, H, N, D)) for s, H in ((301, Hq), (302, Hkv), (303, Hkv)))
+    for scale, tol in ((-0.125, 1e-5), (0.0, 1e-5), (-1.5, 5e-5), (3.0, 5e-5)):
+        got = run_flash(dev, q, k, v, F32, scale=scale)
+        truth = oracle.sdpa_f64(q, k, v, scale=scale)
+        assert np.isfinite(got).all()
+        assert (np.abs(got - truth) / np.maximum(np.abs(truth), 1)).max() <= tol, scale
+    mask = (synth.normal(304, (N, N)) * np.float32(3.0)).astype(np.float32)
+    mask[::7, 1::3] = -np.inf          # every row keeps visible keys (column 0 is never masked)
+    kv_len = np.array([N, max(1, N // 2)], np.int32)
+    for causal in (False, True):
+        got = run_flash(dev, q, k, v, F32, mask=mask, kv_len=kv_len, causal=causal, scale=0.2)
+        truth = oracle.sdpa_f64(q, k, v, mask=mask, kv_len=kv_len, causal=causal, scale=0.2)
+        assert (np.abs(got - truth) / np.maximum(np.abs(truth), 1)).max() <= 1e-5, causal
+
+
 def test_unsupported_shapes_are_declined_not_faked(dev):
     # head_dim 32: the dispatcher's cue to use the general path (flash_attention.rs:470-472)
     q = dev.alloc(4096)
