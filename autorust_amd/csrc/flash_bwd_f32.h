@@ -131,6 +131,17 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
 
     float4 kx[PER_THREAD], vx[PER_THREAD];
     auto fetch = [&](int tile) __attribute__((always_inline)) {
+        if (tile * F32_BK + F32_BK <= kend) {  // a full tile: no row tests, no zero fill
+#pragma unroll
+            for (int j = 0; j < PER_THREAD; ++j) {
+                const int c = stid + j * T;
+                const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+                const size_t off = (size_t)(tile * F32_BK + row) * D + col;
+                kx[j] = *(const float4 *)(kp + off);
+                vx[j] = *(const float4 *)(vp + off);
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < PER_THREAD; ++j) {
             const int c = stid + j * T;
@@ -306,15 +317,26 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
         const int g = step / (qtiles - qt0);
         const int q0 = (qt0 + step - g * (qtiles - qt0)) * F32_BK;
         const size_t bh = (size_t)b * p.Hq + (size_t)kvh * group + g;
+        if (q0 + F32_BK <= N) {  // a full tile: no row tests, no zero fill
 #pragma unroll
-        for (int j = 0; j < PER_THREAD; ++j) {
-            const int c = stid + j * T;
-            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-            const int gr = q0 + row;
-            qx[j] = dx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (gr < N) {
-                qx[j] = *(const float4 *)(p.q + (bh * N + gr) * D + col);
-                dx[j] = *(const float4 *)(p.dout + (bh * N + gr) * D + col);
+            for (int j = 0; j < PER_THREAD; ++j) {
+                const int c = stid + j * T;
+                const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+                const size_t off = (bh * N + q0 + row) * D + col;
+                qx[j] = *(const float4 *)(p.q + off);
+                dx[j] = *(const float4 *)(p.dout + off);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < PER_THREAD; ++j) {
+                const int c = stid + j * T;
+                const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+                const int gr = q0 + row;
+                qx[j] = dx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (gr < N) {
+                    qx[j] = *(const float4 *)(p.q + (bh * N + gr) * D + col);
+                    dx[j] = *(const float4 *)(p.dout + (bh * N + gr) * D + col);
+                }
             }
         }
         if (stid < F32_BK) {
