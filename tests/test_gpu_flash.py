@@ -126,6 +126,22 @@ def test_f32_scale_signs_wide_logits_and_additive_mask(dev, N):
         assert (np.abs(got - truth) / np.maximum(np.abs(truth), 1)).max() <= 1e-5, causal
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_f32_tiling_variants_by_workgroup_count(dev, causal):
+    """The fp32 kernel picks its tiling from the number of workgroups: 32 queries with the key tiles
+    dealt out over four waves (few workgroups), over two waves (more than two and at most four
+    workgroups per CU: B8 H12 S197 gives 672 on 256 CUs), or 128 queries per workgroup (many).  All
+    are the same function."""
+    D = 64
+    for B, H, N in ((1, 12, 197), (8, 12, 197), (8, 24, 640)):
+        q, k, v = (synth.normal(s, (B, H, N, D)) for s in (311, 312, 313))
+        kv_len = np.full(B, N, np.int32)
+        kv_len[-1] = N - 37
+        got = run_flash(dev, q, k, v, F32, kv_len=kv_len, causal=causal)
+        truth = oracle.sdpa_f64(q, k, v, kv_len=kv_len, causal=causal)
+        assert (np.abs(got - truth) / np.maximum(np.abs(truth), 1)).max() <= 1e-5, (B, H, N)
+
+
 def test_unsupported_shapes_are_declined_not_faked(dev):
     # head_dim 32: the dispatcher's cue to use the general path (flash_attention.rs:470-472)
     q = dev.alloc(4096)
