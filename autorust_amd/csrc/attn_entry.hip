@@ -12,6 +12,7 @@
 //
 //   entry               block      grid                      covers
 //   ar_flash_f32        [256,1,1]  [ceil(n/128), B*hq, 1]    fp32 exact (cuda_flash.rs)
+//   ar_flash_f32_short  [256,1,1]  [ceil(n/32), B*hq, 1]     fp32 exact for few, short heads; head_dim 64
 //   ar_flash_bf16       [256,1,1]  [ceil(n/128), B*hq, 1]    bf16 (cuda_flash_bf16.rs), any mask
 //   ar_flash_bf16_long  [512,1,1]  [ceil(n/256), B*hq, 1]    bf16 pipelined, has_mask must be 0
 //   ar_flash_bf16_short [512,1,1]  [ceil(n/128), B*hq, 1]    bf16, n <= 256, has_mask must be 0
@@ -28,6 +29,8 @@
 //   ar_fl_prep     [256,1,1]  [ceil(n/4), B*hq, 1]     (O, dO, D,  N, head_dim)
 //   ar_fl_bwd_dq   [256,1,1]  [ceil(n/128), B*hq, 1]   (Q, K, V, dO, LSE, D, M, dQ,  N, head_dim, causal, has_mask, hq, hkv)
 //   ar_fl_bwd_dkv  [256,1,1]  [ceil(n/128), B*hkv, 1]  (Q, K, V, dO, LSE, D, M, dK, dV,  N, head_dim, causal, has_mask, hq, hkv)
+//   ar_fl_fwd_short, ar_fl_bwd_dq_short, ar_fl_bwd_dkv_short: the same arguments with grid.x = ceil(n/32), for few,
+//   short heads (32 queries / keys per workgroup, the tiles of the other side dealt out between its waves); head_dim 64
 // head_dim must be 64 or 128; any other value makes the kernel return without writing.
 // The *_long entries address K and V with 32-bit byte offsets: (N + 320) * head_dim * 2 < 2^31.
 #include "attn_fwd.h"
@@ -120,6 +123,46 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_fwd(const float *Q, cons
     }
 }
 
+// Short shapes (few workgroups of 128 queries would leave most of the chip idle): 32 queries per
+// workgroup, grid [ceil(N/32), B*hq, 1], the key tiles dealt out between the four waves.  head_dim 64
+// only (the reference's own head size); any other returns without writing.  LSE may be null.
+namespace {
+__device__ __forceinline__ void flash_f32_short(const float *Q, const float *K, const float *V, float *O, float *LSE,
+                                                const float *M, int N, int causal, int has_mask, int hq, int hkv, float *lds)
+{
+    FlashF32Params p = {};
+    p.q = Q; p.k = K; p.v = V; p.o = O; p.lse = LSE;
+    p.mask = has_mask ? M : nullptr;
+    p.Hq = hq; p.Hkv = hkv; p.N = N;
+    p.nq = (int)gridDim.x;
+    dense(p.qs, hq, N, 64);
+    dense(p.ks, hkv, N, 64);
+    dense(p.os, hq, N, 64);
+    p.scale = 0.125f;
+    const int wg = linear_wg();
+    if (causal) flash_f32_body<64, 4, true, true>(p, lds, wg);
+    else flash_f32_body<64, 4, false, true>(p, lds, wg);
+}
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_f32_short(const float *Q, const float *K, const float *V, float *O,
+                                                                         const float *M, int N, int head_dim, int causal,
+                                                                         int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<64, 4, true>()];
+    if (head_dim != 64) return;
+    flash_f32_short(Q, K, V, O, nullptr, M, N, causal, has_mask, hq, hkv, lds);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_fl_fwd_short(const float *Q, const float *K, const float *V, float *O,
+                                                                      float *LSE, const float *M, int N, int head_dim,
+                                                                      int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<64, 4, true>()];
+    if (head_dim != 64) return;
+    flash_f32_short(Q, K, V, O, LSE, M, N, causal, has_mask, hq, hkv, lds);
+}
+
 extern "C" __global__ void __launch_bounds__(256) ar_fl_prep(const float *O, const float *dO, float *D, int N, int head_dim)
 {
     const long row0 = (long)blockIdx.y * N + (long)blockIdx.x * 4, rows = ((long)blockIdx.y + 1) * N;
@@ -176,6 +219,36 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_bwd_dkv(const float *Q, 
         if (causal) bwd_dkv_body<128, 4, true>(p, lds, wg);
         else bwd_dkv_body<128, 4, false>(p, lds, wg);
     }
+}
+
+// The same for short shapes: 32 queries (dQ) / 32 keys (dK, dV) per workgroup, grid [ceil(N/32), B*hq, 1] /
+// [ceil(N/32), B*hkv, 1], the tiles of the other side dealt out between the four waves.  head_dim 64 only.
+extern "C" __global__ void __launch_bounds__(256, 2) ar_fl_bwd_dq_short(const float *Q, const float *K, const float *V,
+                                                                         const float *dO, const float *LSE, const float *D,
+                                                                         const float *M, float *dQ, int N, int head_dim,
+                                                                         int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<64, 4, true>()];
+    if (head_dim != 64) return;
+    FlashBwdParams p = bwd_params(Q, K, V, dO, LSE, D, M, N, head_dim, has_mask, hq, hkv);
+    p.dq = dQ;
+    const int wg = linear_wg();
+    if (causal) bwd_dq_body<64, 4, true, true>(p, lds, wg);
+    else bwd_dq_body<64, 4, false, true>(p, lds, wg);
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_fl_bwd_dkv_short(const float *Q, const float *K, const float *V,
+                                                                       const float *dO, const float *LSE, const float *D,
+                                                                       const float *M, float *dK, float *dV, int N,
+                                                                       int head_dim, int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[bwd_lds_floats<64, 4, true>()];
+    if (head_dim != 64) return;
+    FlashBwdParams p = bwd_params(Q, K, V, dO, LSE, D, M, N, head_dim, has_mask, hq, hkv);
+    p.dk = dK; p.dv = dV;
+    const int wg = linear_wg();
+    if (causal) bwd_dkv_body<64, 4, true, true>(p, lds, wg);
+    else bwd_dkv_body<64, 4, false, true>(p, lds, wg);
 }
 
 extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V,

@@ -376,6 +376,12 @@ bool long_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int6
 
 }  // namespace
 
+// The fp32 kernels: 128 queries (keys) per workgroup when that still fills the chip, else 32
+static bool short_f32(const std::shared_ptr<Device> &dev, int64_t b, int64_t heads, int64_t n)
+{
+    return b * heads * ((n + 127) / 128) < 2 * (int64_t)dev->compute_units();
+}
+
 std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
                                            const Tensor &out, bool is_causal, Kernel kern, const Settings &st)
 {
@@ -389,8 +395,13 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     std::vector<HostCall> calls;
 
     if (kern == Kernel::FlashF32) {
-        calls.push_back(make_call(dev, "ar_flash_f32", {q, k, v, out, mslot}, {F, F, F, F, F}, {(n + 127) / 128, b * h, 1},
-                                  {256, 1, 1}, vals));
+        // few, short heads: 32 queries per workgroup instead of 128 (the rule of arhip_flash_fwd)
+        if (d == 64 && short_f32(dev, b, h, n))
+            calls.push_back(make_call(dev, "ar_flash_f32_short", {q, k, v, out, mslot}, {F, F, F, F, F},
+                                      {(n + 31) / 32, b * h, 1}, {256, 1, 1}, vals));
+        else
+            calls.push_back(make_call(dev, "ar_flash_f32", {q, k, v, out, mslot}, {F, F, F, F, F}, {(n + 127) / 128, b * h, 1},
+                                      {256, 1, 1}, vals));
         return calls;
     }
     if (kern == Kernel::FlashBf16) {
@@ -524,8 +535,10 @@ std::optional<TrainOut> fused_attention_train(const Tensor &q, const Tensor &k, 
     const DType F = DType::Float32;
     Tensor out = Tensor::empty(dev, {b, h, n, d}, F), lse = Tensor::empty(dev, {b * h, n}, F);
     const Tensor mslot = attn_mask ? *attn_mask : out;
-    const HostCall call = make_call(dev, "ar_fl_fwd", {q, k, v, out, lse, mslot}, {F, F, F, F, F, F}, {(n + 127) / 128, b * h, 1},
-                                    {256, 1, 1}, {n, d, (int64_t)is_causal, (int64_t)(attn_mask != nullptr), h, hk});
+    const bool shrt = d == 64 && short_f32(dev, b, h, n);
+    const HostCall call = make_call(dev, shrt ? "ar_fl_fwd_short" : "ar_fl_fwd", {q, k, v, out, lse, mslot}, {F, F, F, F, F, F},
+                                    {(n + (shrt ? 31 : 127)) / (shrt ? 32 : 128), b * h, 1}, {256, 1, 1},
+                                    {n, d, (int64_t)is_causal, (int64_t)(attn_mask != nullptr), h, hk});
     sess.capture_host(call);
     call.exec();
     return TrainOut{out, lse};
@@ -545,12 +558,15 @@ std::optional<Grads> fused_attention_backward(const Tensor &q, const Tensor &k, 
     Grads g{Tensor::empty(dev, {b, h, n, d}, F), Tensor::empty(dev, {b, hk, n, d}, F), Tensor::empty(dev, {b, hk, n, d}, F)};
     const Tensor mslot = attn_mask ? *attn_mask : g.dq;   // the reference's dummy (cuda_flash_train.rs:442-449)
     const std::vector<int64_t> vals = {n, d, (int64_t)is_causal, (int64_t)(attn_mask != nullptr), h, hk};
+    // few, short heads: 32 queries / keys per workgroup (the rule of arhip_flash_bwd)
+    const bool shrt = d == 64 && short_f32(dev, b, hk, n);
+    const int64_t rows = shrt ? 32 : 128;
     const std::vector<HostCall> calls = {
         make_call(dev, "ar_fl_prep", {out, dout, delta}, {F, F, F}, {(n + 3) / 4, b * h, 1}, {256, 1, 1}, {n, d}),
-        make_call(dev, "ar_fl_bwd_dq", {q, k, v, dout, lse, delta, mslot, g.dq}, {F, F, F, F, F, F, F, F},
-                  {(n + 127) / 128, b * h, 1}, {256, 1, 1}, vals),
-        make_call(dev, "ar_fl_bwd_dkv", {q, k, v, dout, lse, delta, mslot, g.dk, g.dv}, {F, F, F, F, F, F, F, F, F},
-                  {(n + 127) / 128, b * hk, 1}, {256, 1, 1}, vals),
+        make_call(dev, shrt ? "ar_fl_bwd_dq_short" : "ar_fl_bwd_dq", {q, k, v, dout, lse, delta, mslot, g.dq},
+                  {F, F, F, F, F, F, F, F}, {(n + rows - 1) / rows, b * h, 1}, {256, 1, 1}, vals),
+        make_call(dev, shrt ? "ar_fl_bwd_dkv_short" : "ar_fl_bwd_dkv", {q, k, v, dout, lse, delta, mslot, g.dk, g.dv},
+                  {F, F, F, F, F, F, F, F, F}, {(n + rows - 1) / rows, b * hk, 1}, {256, 1, 1}, vals),
     };
     for (const HostCall &call : calls) {
         sess.capture_host(call);

@@ -28,6 +28,9 @@
 /* fp32 exact mode: replaces `ar_flash_f32`, src/runtime/cuda_flash.rs:53-141.
  * (const float *Q, *K, *V, float *O, const float *M, 6 ints); general tiling. */
 #define ARHIP_KERNEL_FLASH_F32 "ar_flash_f32"
+/* the variant for few, short heads (B * hq * ceil(N/128) below twice the compute units): same
+ * arguments, head_dim 64 only; 32 queries per workgroup, block [256,1,1], grid [ceil(N/32), B*hq, 1]. */
+#define ARHIP_KERNEL_FLASH_F32_SHORT "ar_flash_f32_short"
 
 /* Training kernels, f32: replace `ar_fl_fwd`, `ar_fl_prep`, `ar_fl_bwd_dq`, `ar_fl_bwd_dkv`,
  * src/runtime/cuda_flash_train.rs:57-309, with the reference's argument order and head_dim
@@ -41,6 +44,12 @@
 #define ARHIP_KERNEL_FL_PREP "ar_fl_prep"
 #define ARHIP_KERNEL_FL_BWD_DQ "ar_fl_bwd_dq"
 #define ARHIP_KERNEL_FL_BWD_DKV "ar_fl_bwd_dkv"
+/* the variants for few, short heads (B * hkv * ceil(N/128) below twice the compute units): the same
+ * arguments, head_dim 64 only; 32 queries (keys for dK/dV) per workgroup, block [256,1,1], grid.x =
+ * ceil(N/32); `ar_fl_prep` is shared. */
+#define ARHIP_KERNEL_FL_FWD_SHORT "ar_fl_fwd_short"
+#define ARHIP_KERNEL_FL_BWD_DQ_SHORT "ar_fl_bwd_dq_short"
+#define ARHIP_KERNEL_FL_BWD_DKV_SHORT "ar_fl_bwd_dkv_short"
 
 /* bf16: replaces `ar_flash_bf16`, src/runtime/cuda_flash_bf16.rs:226-427.
  * (const bf16 *Q, *K, *V, bf16 *O, const float *M, 6 ints); general tiling, any mask. */

@@ -52,7 +52,7 @@ pub fn hip_calls(dev: &str, kernel: HipKernel, bufs: Vec<Buffer>, b: i64, h: i64
     match kernel {
         HipKernel::F32 => {
             hip_flash::note_selected(0);
-            vec![hip_flash::host_call_f32(bufs, b, h, n, d, opts)]
+            vec![hip_flash::host_call_f32(dev, bufs, b, h, n, d, opts)]
         }
         HipKernel::Bf16 => {
             hip_flash::note_selected(1);

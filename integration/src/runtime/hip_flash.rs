@@ -10,6 +10,7 @@
 //! | entry                | block | grid                    | arguments after the buffers                  |
 //! |----------------------|-------|-------------------------|----------------------------------------------|
 //! | `ar_flash_f32`       | 256   | `[ceil(n/128), b*h, 1]` | `n, head_dim, causal, has_mask, hq, hkv`     |
+//! | `ar_flash_f32_short` | 256   | `[ceil(n/32), b*h, 1]`  | same; few, short heads; `head_dim` 64        |
 //! | `ar_flash_bf16`      | 256   | `[ceil(n/128), b*h, 1]` | same                                         |
 //! | `ar_flash_bf16_long` | 512   | `[ceil(n/256), b*h, 1]` | same (`has_mask` must be 0)                  |
 //! | `ar_flash_sage`      | 256   | `[ceil(n/128), b*h, 1]` | same `+ bq, bk`; buffers `+ SQ, SK`; O is f32|
@@ -129,10 +130,20 @@ fn long_variant(dev: &str, b: i64, h: i64, n: i64, d: i64) -> bool {
     (wgs >= 2 * cus || (n >= 512 && 2 * wgs >= cus)) && (n + 320) * d * 2 < 1 << 31
 }
 
+/// The fp32 kernels take 128 queries (keys) per workgroup when that still fills the chip, else 32
+/// with the tiles of the other side dealt out between the waves (`*_short`, `head_dim` 64).
+fn short_f32(dev: &str, b: i64, heads: i64, n: i64, d: i64) -> bool {
+    d == 64 && b * heads * ((n + 127) / 128) < 2 * crate::runtime::ops_hip::compute_units(dev)
+}
+
 /// fp32 exact mode: `bufs = [q, k, v, o, mask-or-o]`, all f32 `[b, h, n, d]`.
-pub fn host_call_f32(bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
+pub fn host_call_f32(dev: &str, bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
     let f = dtype::FLOAT32;
-    call("ar_flash_f32", bufs, &[f, f, f, f, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+    if short_f32(dev, b, h, n, d) {
+        call("ar_flash_f32_short", bufs, &[f, f, f, f, f], [(n + 31) / 32, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+    } else {
+        call("ar_flash_f32", bufs, &[f, f, f, f, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+    }
 }
 
 /// bf16: `bufs = [q, k, v, o, mask-or-o]`, q/k/v/o bf16, mask f32 `[n, n]`.
@@ -247,25 +258,32 @@ pub fn host_calls_sage(
 // src/runtime/cuda_flash_train.rs:336-541): f32 tensors, dense `[b, h, n, d]` ----
 
 /// Forward that also writes `lse [b*h, n]`: `bufs = [q, k, v, o, lse, mask-or-o]`.
-pub fn host_call_train_fwd(bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
+pub fn host_call_train_fwd(dev: &str, bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
     let f = dtype::FLOAT32;
-    call("ar_fl_fwd", bufs, &[f, f, f, f, f, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+    if short_f32(dev, b, h, n, d) {
+        call("ar_fl_fwd_short", bufs, &[f, f, f, f, f, f], [(n + 31) / 32, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+    } else {
+        call("ar_fl_fwd", bufs, &[f, f, f, f, f, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+    }
 }
 
 /// The three launches of the backward, in order.  `delta` is a scratch tensor `[b*h, n]`; `mask` is
 /// the additive mask or `dq` again (the reference's dummy, cuda_flash_train.rs:442-449).
 #[allow(clippy::too_many_arguments)]
 pub fn host_calls_train_bwd(
+    dev: &str,
     q: Buffer, k: Buffer, v: Buffer, o: Buffer, lse: Buffer, dout: Buffer, mask: Buffer, delta: Buffer,
     dq: Buffer, dk: Buffer, dv: Buffer, b: i64, h: i64, n: i64, d: i64, opts: Options,
 ) -> Vec<HostCall> {
     let f = dtype::FLOAT32;
-    let tiles = (n + 127) / 128;
+    let short = short_f32(dev, b, opts.h_kv, n, d);
+    let tiles = if short { (n + 31) / 32 } else { (n + 127) / 128 };
+    let (dq_name, dkv_name) = if short { ("ar_fl_bwd_dq_short", "ar_fl_bwd_dkv_short") } else { ("ar_fl_bwd_dq", "ar_fl_bwd_dkv") };
     vec![
         call("ar_fl_prep", vec![o, dout.clone(), delta.clone()], &[f, f, f], [(n + 3) / 4, b * h, 1], [256, 1, 1], vec![n, d], &[]),
-        call("ar_fl_bwd_dq", vec![q.clone(), k.clone(), v.clone(), dout.clone(), lse.clone(), delta.clone(), mask.clone(), dq],
+        call(dq_name, vec![q.clone(), k.clone(), v.clone(), dout.clone(), lse.clone(), delta.clone(), mask.clone(), dq],
              &[f, f, f, f, f, f, f, f], [tiles, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[]),
-        call("ar_fl_bwd_dkv", vec![q, k, v, dout, lse, delta, mask, dk, dv],
+        call(dkv_name, vec![q, k, v, dout, lse, delta, mask, dk, dv],
              &[f, f, f, f, f, f, f, f, f], [tiles, b * opts.h_kv, 1], [256, 1, 1], vals(n, d, h, opts), &[]),
     ]
 }

@@ -52,6 +52,28 @@ def test_ar_flash_f32_by_name(dev, kernels, case):
     assert np.abs(got - want).max() < 2e-5
 
 
+@pytest.mark.parametrize("case", [c for c in CASES if c[4] == 64] + [(1, 12, 12, 197, 64, False, False)], ids=str)
+def test_ar_flash_f32_short_by_name(dev, kernels, case):
+    """The 32-query variant for few, short heads (head_dim 64): grid [ceil(n/32), b*hq, 1]."""
+    b, hq, hkv, n, d, causal, has_mask = case
+    q, k, v = fill_qkv(b, hq, hkv, n, d)
+    mask = ref_mask(n).reshape(n, n) if has_mask else None
+    with Bufs(dev) as bufs:
+        dq, dk, dv = bufs.put(q), bufs.put(k), bufs.put(v)
+        do = bufs.new(q.nbytes)
+        dm = bufs.put(mask) if has_mask else do
+        dev.launch(kernels, "ar_flash_f32_short", _grid(n, 32, b, hq), (256, 1, 1), [dq, dk, dv, do, dm],
+                   [n, d, int(causal), int(has_mask), hq, hkv])
+        got = do.copyout(np.float32, q.shape)
+        # any other head_dim: the kernel returns without writing
+        do2 = bufs.new(q.nbytes)
+        dev.launch(kernels, "ar_flash_f32_short", _grid(n, 32, b, hq), (256, 1, 1), [dq, dk, dv, do2, do2],
+                   [n, 128, int(causal), 0, hq, hkv])
+        assert not do2.copyout(np.float32, q.shape).any()
+    want = oracle.flash_f32(q, k, v, mask=mask, causal=causal)
+    assert np.abs(got - want).max() < 2e-5
+
+
 @pytest.mark.parametrize("case", CASES, ids=str)
 def test_ar_flash_bf16_by_name(dev, kernels, case):
     b, hq, hkv, n, d, causal, has_mask = case
@@ -165,6 +187,34 @@ def test_ar_flash_sage_long_by_name(dev, kernels, causal, out_f32):
     # the int8 error to wash out, so they are left to the comparison with the emulation above
     lo = 256 if causal else 0
     assert np.abs(got - oracle.sdpa_f64(q, k, v, causal=causal))[:, :, lo:].max() <= 2e-2
+
+
+@pytest.mark.parametrize("case", [(2, 4, 2, 37, 64, True, False), (1, 4, 4, 150, 64, False, True), (1, 12, 12, 197, 64, False, False)],
+                         ids=str)
+def test_short_training_kernels_by_name(dev, kernels, case):
+    """ar_fl_fwd_short / ar_fl_prep / ar_fl_bwd_dq_short / ar_fl_bwd_dkv_short: 32 queries (keys) per
+    workgroup, grid.x = ceil(n/32), head_dim 64; against the float64 oracle."""
+    b, hq, hkv, n, d, causal, has_mask = case
+    q, k, v = fill_qkv(b, hq, hkv, n, d)
+    do = synth.normal(78, q.shape)
+    mask = ref_mask(n).reshape(n, n) if has_mask else None
+    vals = [n, d, int(causal), int(has_mask), hq, hkv]
+    with Bufs(dev) as bufs:
+        dq_, dk_, dv_, ddo = bufs.put(q), bufs.put(k), bufs.put(v), bufs.put(do)
+        o, lse, delta = bufs.new(q.nbytes), bufs.new(b * hq * n * 4), bufs.new(b * hq * n * 4, zero=False)
+        gq, gk, gv = bufs.new(q.nbytes, zero=False), bufs.new(k.nbytes, zero=False), bufs.new(v.nbytes, zero=False)
+        dm = bufs.put(mask) if has_mask else o
+        blk = (256, 1, 1)
+        dev.launch(kernels, "ar_fl_fwd_short", _grid(n, 32, b, hq), blk, [dq_, dk_, dv_, o, lse, dm], vals)
+        dev.launch(kernels, "ar_fl_prep", ((n + 3) // 4, b * hq, 1), blk, [o, ddo, delta], [n, d])
+        dev.launch(kernels, "ar_fl_bwd_dq_short", _grid(n, 32, b, hq), blk, [dq_, dk_, dv_, ddo, lse, delta, dm, gq], vals)
+        dev.launch(kernels, "ar_fl_bwd_dkv_short", _grid(n, 32, b, hkv), blk, [dq_, dk_, dv_, ddo, lse, delta, dm, gk, gv], vals)
+        got = (o.copyout(np.float32, q.shape), lse.copyout(np.float32, (b, hq, n)), gq.copyout(np.float32, q.shape),
+               gk.copyout(np.float32, k.shape), gv.copyout(np.float32, v.shape))
+    want = oracle.attention_backward_f64(q, k, v, do, mask=mask, causal=causal)
+    for name, g, w in zip(("o", "lse", "dq", "dk", "dv"), got, want):
+        assert np.abs(g - w).max() < 2e-3, name
+        assert np.abs(g - w).max() <= 3e-5 * max(1.0, np.abs(w).max()), name
 
 
 @pytest.mark.parametrize("case", [(2, 4, 2, 37, 64, True, False), (1, 4, 4, 150, 128, False, True)], ids=str)

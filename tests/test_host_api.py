@@ -236,7 +236,9 @@ def test_fused_attention_train_and_backward(hdev):
     out, lse = host.fused_attention_train(tq, tk, tv, sess, is_causal=causal)
     dq, dk, dv = host.fused_attention_backward(tq, tk, tv, out, lse, tdo, sess, is_causal=causal)
     assert sess.end_capture() == 4
-    assert [sess.step(i)[0] for i in range(4)] == ["ar_fl_fwd", "ar_fl_prep", "ar_fl_bwd_dq", "ar_fl_bwd_dkv"]
+    # few, short heads: the 32-row entries, grid.x = ceil(n / 32)
+    assert [sess.step(i)[0] for i in range(4)] == ["ar_fl_fwd_short", "ar_fl_prep", "ar_fl_bwd_dq_short", "ar_fl_bwd_dkv_short"]
+    assert sess.step(0)[1] == [2, b * h, 1] and sess.step(2)[1] == [2, b * h, 1] and sess.step(3)[1] == [2, b * hk, 1]
     want = oracle.attention_backward_f64(q, k, v, do, causal=causal, scale=0.125)
     for name, got, w in zip(("out", "lse", "dq", "dk", "dv"), (out, lse, dq, dk, dv), want):
         assert float(np.abs(got.to_list().reshape(w.shape) - w).max()) < 2e-3, name
@@ -245,6 +247,20 @@ def test_fused_attention_train_and_backward(hdev):
     # bf16 tensors keep the graph path: None (flash_attention.rs:802-807)
     tb = Tensor.from_slice(hdev, q, q.shape, BFLOAT16)
     assert host.fused_attention_train(tb, tb, tb, sess) is None
+    # enough 128-row workgroups to fill the chip: the reference's own grid and names
+    b, h, hk = 72, 8, 8
+    q, k, v, do = (data(b * hh * n * d, s).reshape(b, hh, n, d) for hh, s in ((h, 0.0), (hk, 1.3), (hk, 2.7), (h, 4.1)))
+    tq, tk, tv, tdo = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v, do))
+    sess = Session()
+    sess.begin_capture()
+    out, lse = host.fused_attention_train(tq, tk, tv, sess, is_causal=causal)
+    dq, dk, dv = host.fused_attention_backward(tq, tk, tv, out, lse, tdo, sess, is_causal=causal)
+    assert sess.end_capture() == 4
+    assert [sess.step(i)[0] for i in range(4)] == ["ar_fl_fwd", "ar_fl_prep", "ar_fl_bwd_dq", "ar_fl_bwd_dkv"]
+    assert sess.step(0)[1] == [1, b * h, 1]
+    want = oracle.attention_backward_f64(q, k, v, do, causal=causal, scale=0.125)
+    for name, got, w in zip(("out", "lse", "dq", "dk", "dv"), (out, lse, dq, dk, dv), want):
+        assert float(np.abs(got.to_list().reshape(w.shape) - w).max()) < 2e-3, name
 
 
 @gpu
@@ -275,6 +291,23 @@ def test_short_sequences_take_the_short_kernel(hdev):
     name, grid, vals = sess.step(0)
     assert name == "ar_flash_bf16_short" and grid == [2, b * h, 1] and sess.step_detail(0)[1] == [512, 1, 1]
     assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v)).max()) < 2e-2
+
+
+@gpu
+def test_fp32_exact_mode_picks_its_tiling_from_the_shape(hdev):
+    """Float32 tensors take the fp32 exact kernel: the 32-query entry for few, short heads (ViT-B/16 at
+    batch 1), the reference's 128-query grid when that fills the chip."""
+    d = 64
+    for (b, h, n), want_name, per_wg in (((1, 12, 197), "ar_flash_f32_short", 32), ((48, 12, 197), "ar_flash_f32", 128)):
+        q, k, v = (synth.normal(720 + i, (b, h, n, d)) for i in range(3))
+        tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v))
+        sess = Session()
+        sess.begin_capture()
+        out = tq.flash_attention_with(tk, tv, None, 0.0, True, sess)
+        assert sess.end_capture() == 1
+        name, grid, vals = sess.step(0)
+        assert name == want_name and grid == [(n + per_wg - 1) // per_wg, b * h, 1] and vals == [n, d, 1, 0, h, h]
+        assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v, causal=True)).max()) < 2e-5
 
 
 @gpu
