@@ -86,10 +86,9 @@ __device__ __forceinline__ void pipe_work_item(const AttnParams &p, int wg, int 
 }
 
 // The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
-// aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below;
-// m_grid: the power of two the exponent reference is kept a multiple of (BIAS only).
+// aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below.
 template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS>
-__device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear, float m_grid)
+__device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
     constexpr int NW = 8;
@@ -229,7 +228,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // fma((float)sum, c, -m_run) does PROVIDED m_bias is exact.  Two things make it exact: c is
     // rounded to 21 significant bits (so that 12582912 c = 3 c 2^22 has at most 23), and m_run only
     // ever takes multiples of m_grid, a power of two that no unit in the last place of any
-    // 12582912 c + m_run this workgroup can meet exceeds (attn_pipe_body derives it from the largest
+    // 12582912 c + m_run this workgroup can meet exceeds (the prologue derives it from the largest
     // scales).  Where m_run outweighs 12582912 c (tiny scales) the sum may still round, by at most
     // half a unit in the last place of m_run: 2^-16 for references below 256.
     constexpr float BIAS_F = 12582912.0f;
@@ -243,7 +242,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     }
     float m_bias = NEG_SENTINEL;  // what the pipelined softmax subtracts for the block it works on
     auto set_bias = [&](float c) __attribute__((always_inline)) { m_bias = BIAS ? __builtin_fmaf(BIAS_F, c, m_run) : m_run; };
-    const float m_grid_inv = BIAS ? 1.0f / m_grid : 1.0f;
+    float m_grid = 1.0f, m_grid_inv = 1.0f;  // set in the prologue (BIAS only)
     // a logit accumulator as a float (before the factor c)
     auto as_logit = [&](const acc_t &a, int r) __attribute__((always_inline)) -> float {
         if constexpr (BIAS) return __builtin_bit_cast(float, (int)a[r]);
@@ -557,8 +556,37 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         skv_cur = load_sk_group(0);
         skv_nxt = load_sk_group(1);
     }
+    // BIAS: the largest Q scale of the workgroup's queries and the largest K scale of the head, read
+    // behind the transfers issued above so that their latency is spent under them
+    float mq = 0.f, mk = 0.f;
+    if constexpr (BIAS) {
+        const int nqb = (N + p.bq - 1) / p.bq, nkb = (N + p.bk - 1) / p.bk;
+        const int qb0 = qblk / p.bq, qb1 = min(qblk + BQ - 1, N - 1) / p.bq;
+        for (int i = qb0 + lane; i <= qb1; i += 64) mq = fmaxf(mq, fabsf(p.sq[(size_t)bh * nqb + i]));
+        for (int i = lane; i < nkb; i += 64) mk = fmaxf(mk, fabsf(p.sk[(size_t)kv_bh * nkb + i]));
+    }
     wait_vmem_le<0>();
     __syncthreads();
+    if constexpr (BIAS) {
+        // The exponent reference stays on a grid no finer than the unit in the last place of
+        // 12582912 c for the largest c = sq sk scale log2(e) the workgroup can meet; every wave reduces
+        // the same scales, so the grid is uniform over the workgroup.
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) {
+            mq = fmaxf(mq, __shfl_xor(mq, o));
+            mk = fmaxf(mk, __shfl_xor(mk, o));
+        }
+        // 12582912 c_max < 2^(E+1): the sums stay below 2^(E+2) wherever the bias outweighs the
+        // reference, so their unit in the last place is at most 2^(E-22); the grid is twice that.
+        // (Scales that are not finite, or zero, give a grid of 1: the results are garbage or
+        // trivial either way.)
+        const float x = 12582912.0f * (((mq * mk) * fabsf(p.scale)) * LOG2E);
+        const int e = (int)((__float_as_uint(x) >> 23) & 0xff) - 127;  // floor(log2 x)
+        float grid = 1.0f;
+        if (x > 0x1p-60f && x < 0x1p100f) grid = __uint_as_float((uint32_t)(e - 21 + 127) << 23);
+        m_grid = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(grid)));
+        m_grid_inv = 1.0f / m_grid;
+    }
     float c_carry = tile_c(0, 0);  // exponent factor of the tile the next tile_iter works on
     acc_t s_a, s_b;  // logits of the even / odd block of a tile
 #pragma unroll
@@ -666,42 +694,11 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     }
 }
 
-// int8: the biased accumulators (see s_init) need the exponent reference on a grid no finer than the
-// unit in the last place of 12582912 c for the largest c = sq sk scale log2(e) the workgroup can
-// meet: every wave reduces the same scales, so the grid is uniform over the workgroup.
+// int8 uses the biased accumulators (see s_init); bf16 and FP8 the plain ones.
 template <int D, bool CAUSAL, int MODE, bool OUT_F32>
 __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
-    if constexpr (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS) {
-        int bh, qt;
-        pipe_work_item<CAUSAL>(p, wg_linear, bh, qt);
-        const int lane = threadIdx.x & 63;
-        const int N = p.N;
-        const int nqb = (N + p.bq - 1) / p.bq, nkb = (N + p.bk - 1) / p.bk;
-        const int b = bh / p.Hq;
-        const int kv_bh = b * p.Hkv + (bh - b * p.Hq) / (p.Hq / p.Hkv);
-        const int qb0 = (qt * 256) / p.bq, qb1 = min(qt * 256 + 255, N - 1) / p.bq;
-        float mq = 0.f, mk = 0.f;
-        for (int i = qb0 + lane; i <= qb1; i += 64) mq = fmaxf(mq, fabsf(p.sq[(size_t)bh * nqb + i]));
-        for (int i = lane; i < nkb; i += 64) mk = fmaxf(mk, fabsf(p.sk[(size_t)kv_bh * nkb + i]));
-#pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) {
-            mq = fmaxf(mq, __shfl_xor(mq, o));
-            mk = fmaxf(mk, __shfl_xor(mk, o));
-        }
-        // 12582912 c_max < 2^(E+1): the sums stay below 2^(E+2) wherever the bias outweighs the
-        // reference, so their unit in the last place is at most 2^(E-22); the grid is twice that.
-        // (Scales that are not finite, or zero, give a grid of 1: the results are garbage or
-        // trivial either way.)
-        const float x = 12582912.0f * (((mq * mk) * fabsf(p.scale)) * LOG2E);
-        const int e = (int)((__float_as_uint(x) >> 23) & 0xff) - 127;  // floor(log2 x)
-        float grid = 1.0f;
-        if (x > 0x1p-60f && x < 0x1p100f) grid = __uint_as_float((uint32_t)(e - 21 + 127) << 23);
-        grid = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(grid)));
-        attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, true>(p, lds, wg_linear, grid);
-    } else {
-        attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, false>(p, lds, wg_linear, 1.0f);
-    }
+    attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS)>(p, lds, wg_linear);
 }
 
 template <int D, bool CAUSAL, int MODE, bool OUT_F32>
