@@ -136,7 +136,7 @@ def _wave(qw, kk, vb, scale, rows, causal=False, kvl=None, sq_rows=None, sk_tile
 
 
 def _grid(sq_h, sk_h, wg, bq, scale):
-    """attn_pipe_body: the grid of workgroup wg (256 queries) of a head with scales sq_h, sk_h."""
+    """the prologue of attn_pipe_impl: the grid of workgroup wg (256 queries) of a head with scales sq_h, sk_h."""
     qb = np.arange((wg * 256) // bq, min((wg * 256 + 255) // bq, len(sq_h) - 1) + 1)
     x = F(BIAS) * F(F(F(np.abs(sq_h[qb]).max() * np.abs(sk_h).max()) * scale) * LOG2E)
     e = int((np.asarray(x, F).view(np.uint32) >> 23) & 0xFF) - 127

@@ -1,5 +1,5 @@
 """CPU check of the arithmetic the pipelined int8 kernel relies on when it reads its int32 logit
-accumulators as biased floats (autorust_amd/csrc/attn_pipe.h, s_init / set_bias / attn_pipe_body):
+accumulators as biased floats (autorust_amd/csrc/attn_pipe.h, s_init / set_bias / the grid set in the prologue):
 
     accumulators start at 0x4B400000, so their bits read as the float B + acc, B = 12582912;
     c' = c cut to 21 significant bits (round to nearest);
