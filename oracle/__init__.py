@@ -310,7 +310,9 @@ def sage_fp8(qc, kc, sq, sk, v, bq, bk, mask=None, causal=False, kv_len=None, sc
                 s = (s + np.broadcast_to(_f32(mask), (N, N))).astype(np.float32)
             s = np.where(dead, np.float32(-1e30), s)
             m = s.max(axis=1, keepdims=True)
-            p = np.exp((s - m).astype(np.float32)).astype(np.float32)
+            # the fp32 exponential, correctly rounded (float64 evaluation of the fp32 argument, one rounding):
+            # numpy's own fp32 exp is a vector routine that may be 1 ulp off, which moves bf16 roundings of P
+            p = np.exp((s - m).astype(np.float32).astype(np.float64)).astype(np.float32)
             p = np.where(dead, np.float32(0), p) if (causal or kv_len is not None) else p
             l = p.sum(axis=1, keepdims=True, dtype=np.float32)
             o = (bf16_round(p).astype(np.float64) @ vb[b, kh].astype(np.float64)).astype(np.float32)

@@ -454,3 +454,109 @@ def test_fp8_e4m3_against_torch_and_closed_forms():
     c, sc = oracle.quant_blocks_fp8(x, 32)
     assert np.abs(oracle.fp8_e4m3_value(c[0, 0, :32])).max() == 448 and sc[0, 1].tolist() == [1.0, 1.0]
     assert np.abs(oracle.fp8_e4m3_value(c[0, 0]) * np.repeat(sc[0, 0], 32)[:, None] - x[0, 0]).max() <= np.abs(x[0, 0]).max() / 16
+
+
+def _sage_fp8_inputs(seed, B, Hq, Hkv, N, D, bq, bk):
+    q = synth.normal(seed, (B, Hq, N, D))
+    k = synth.normal(seed + 1, (B, Hkv, N, D)) + 3 * synth.normal(seed + 3, (1, Hkv, 1, D))
+    v = synth.normal(seed + 2, (B, Hkv, N, D))
+    qc, sq = oracle.quant_blocks_fp8(q, bq)
+    kc, sk = oracle.quant_blocks_fp8(k, bk, sub=oracle.k_mean(k))
+    return qc, kc, sq, sk, v
+
+
+@pytest.mark.parametrize("bq,bk", [(1, 1), (128, 64), (32, 16)])
+@pytest.mark.parametrize("causal,use_mask,kv_len,hkv", [
+    (False, False, None, 2), (True, False, None, 2), (False, True, None, 2), (False, False, 100, 2),
+    (True, True, 77, 1), (True, False, 131, 4)])
+def test_sage_fp8_reference_against_torch_ops(bq, bk, causal, use_mask, kv_len, hkv):
+    """Every branch and rounding point of the FP8 attention emulation (the AR_FP8 branch of
+    src/runtime/cuda_flash_sage.rs:92-147,280-412), re-derived with torch tensor ops: operands are
+    torch's own float8_e4m3fn view of the codes (exact in float64, as are their products and sums),
+    the dequantisation factor in the kernel's order, additive mask, causal triangle, key length,
+    fp32 softmax numerator, bf16 P and V, division by the sum of the unrounded probabilities."""
+    torch = pytest.importorskip("torch")
+    B, Hq, N, D = 1, 4, 150, 64
+    qc, kc, sq, sk, v = _sage_fp8_inputs(191, B, Hq, hkv, N, D, bq, bk)
+    mask = synth.normal(195, (N, N)).astype(np.float32) if use_mask else None
+    scale = np.float32(1.0) / np.sqrt(np.float32(D))
+    rep = Hq // hkv
+    bf = lambda t: t.to(torch.bfloat16).to(torch.float32)
+    tq = torch.from_numpy(qc).view(torch.float8_e4m3fn).double()
+    tk = torch.from_numpy(np.repeat(kc, rep, 1)).view(torch.float8_e4m3fn).double()
+    acc = (tq @ tk.transpose(-1, -2)).float()                         # exact in float64, one rounding
+    fq = torch.from_numpy(np.repeat(sq, bq, -1)[..., :N])             # scale of row i: sq[i // bq]
+    fk = torch.from_numpy(np.repeat(np.repeat(sk, rep, 1), bk, -1)[..., :N])
+    a = (fq[..., :, None] * fk[..., None, :]) * torch.tensor(scale)   # (sq * sk) * scale, fp32
+    s = acc * a
+    if mask is not None:
+        s = s + torch.from_numpy(mask)
+    dead = torch.zeros(N, N, dtype=torch.bool)
+    if causal:
+        dead |= torch.ones(N, N, dtype=torch.bool).triu(1)
+    if kv_len is not None:
+        dead[:, kv_len:] = True
+    s = s.masked_fill(dead, float("-inf"))
+    # the fp32 exponential correctly rounded (float64 exp of the fp32 argument, rounded once): a last-place
+    # difference between two exp routines would flip bf16 roundings of P (2^-9 of a probability each)
+    p = torch.exp((s - s.max(-1, keepdim=True).values).double()).float()
+    tv = bf(torch.from_numpy(np.repeat(v, rep, 1)))
+    want = ((bf(p).double() @ tv.double()).float() / p.sum(-1, keepdim=True)).numpy()
+    kl = None if kv_len is None else np.array([kv_len], np.int32)
+    got = oracle.sage_fp8(qc, kc, sq, sk, v, bq, bk, mask=mask, causal=causal, kv_len=kl)
+    # only summation order and libm-vs-torch exp differ (a dropped bf16 rounding of P or V moves the
+    # result by ~1e-3, a wrong mask edge or scale index by O(0.1))
+    assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+    got_b = oracle.sage_fp8(qc, kc, sq, sk, v, bq, bk, mask=mask, causal=causal, kv_len=kl, round_out=True)
+    assert np.array_equal(got_b, oracle.bf16_round(got))
+
+
+def test_sage_fp8_reference_closed_forms():
+    B, Hq, Hkv, N, D, bq, bk = 1, 2, 2, 96, 64, 32, 16
+    qc, kc, sq, sk, v = _sage_fp8_inputs(201, B, Hq, Hkv, N, D, bq, bk)
+    full = oracle.sage_fp8(qc, kc, sq, sk, v, bq, bk, causal=True)
+    # a key length is the truncated problem (L a multiple of both block sizes keeps the scale
+    # indices aligned); rows at or past L still attend to keys < L only
+    L = 64
+    cut = oracle.sage_fp8(qc[:, :, :L], kc[:, :, :L], sq[:, :, :L // bq], sk[:, :, :L // bk], v[:, :, :L], bq, bk)
+    got = oracle.sage_fp8(qc, kc, sq, sk, v, bq, bk, kv_len=np.array([L], np.int32))
+    assert np.array_equal(got[:, :, :L], cut)
+    # causal row 0 sees key 0 only: the output is bf16(v[0]) whatever the logits are
+    assert np.array_equal(full[:, :, 0], oracle.bf16_round(v[:, :, 0]))
+    # a mask of -inf above the diagonal is the causal flag
+    tri = np.where(np.triu(np.ones((N, N), bool), 1), -np.inf, 0).astype(np.float32)
+    assert np.array_equal(oracle.sage_fp8(qc, kc, sq, sk, v, bq, bk, mask=tri), full)
+    # a constant added to every logit of a row cancels (up to fp32 rounding of s + c)
+    shifted = oracle.sage_fp8(qc, kc, sq, sk, v, bq, bk, causal=True, mask=np.full((N, N), 0.5, np.float32))
+    assert np.abs(shifted - full).max() < 1e-4
+    # codes that are small integers: the FP8 emulation must agree with the (pinned) int8 emulation
+    # on the same integers, scales and values
+    ints = np.clip(np.rint(synth.normal(205, (B, Hq, N, D)) * 3), -8, 8).astype(np.int8)
+    ints_k = np.clip(np.rint(synth.normal(206, (B, Hkv, N, D)) * 3), -8, 8).astype(np.int8)
+    as_fp8 = lambda t: oracle.fp8_e4m3_bits(t.astype(np.float32))
+    for kw in (dict(causal=True), dict(kv_len=np.array([50], np.int32)), dict(mask=synth.normal(207, (N, N)))):
+        a = oracle.sage_fp8(as_fp8(ints), as_fp8(ints_k), sq, sk, v, bq, bk, **kw)
+        b = oracle.sage(ints, ints_k, sq, sk, v, bq, bk, **kw)
+        assert np.abs(a - b).max() <= 2e-6 * max(1.0, np.abs(b).max())
+
+
+def test_quant_blocks_fp8_subtracts_the_mean_first():
+    """quant_blocks_fp8(x, sub=mu) is quant_blocks_fp8(x - mu) with the subtraction done once in
+    fp32 (K smoothing before the FP8 quantiser), and its scale is absmax / 448 of the shifted block
+    (src/runtime/cuda_flash_sage.rs:9,209-222), checked with torch's cast."""
+    torch = pytest.importorskip("torch")
+    B, H, N, D, blk = 2, 3, 100, 64, 32
+    x = synth.normal(211, (B, H, N, D)) + 3 * synth.normal(212, (1, H, 1, D))
+    mu = oracle.k_mean(x)
+    c1, s1 = oracle.quant_blocks_fp8(x, blk, sub=mu)
+    shifted = (x - mu[:, :, None, :]).astype(np.float32)
+    c2, s2 = oracle.quant_blocks_fp8(shifted, blk)
+    assert np.array_equal(c1, c2) and np.array_equal(s1, s2)
+    # the mean matters: without it the codes differ
+    c3, _ = oracle.quant_blocks_fp8(x, blk)
+    assert not np.array_equal(c1, c3)
+    # independent evaluation of one ragged block (the last: rows 96..99) with torch
+    seg = torch.from_numpy(shifted[1, 2, 96:])
+    sc = seg.abs().max() / torch.tensor(np.float32(448.0))
+    want = (seg * (torch.tensor(np.float32(1.0)) / sc)).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(c1[1, 2, 96:], want) and s1[1, 2, 3] == sc.numpy()
