@@ -31,6 +31,14 @@
 //   ar_fl_bwd_dkv  [256,1,1]  [ceil(n/128), B*hkv, 1]  (Q, K, V, dO, LSE, D, M, dK, dV,  N, head_dim, causal, has_mask, hq, hkv)
 //   ar_fl_fwd_short, ar_fl_bwd_dq_short, ar_fl_bwd_dkv_short: the same arguments with grid.x = ceil(n/32), for few,
 //   short heads (32 queries / keys per workgroup, the tiles of the other side dealt out between its waves); head_dim 64
+// Key-padding masks: every forward entry `X` of the first table has a twin `X_lens` that takes one more
+// pointer after M, `const int *L` ([B] int32: batch b attends to keys [0, L[b]) only, clamped to [0, N];
+// a batch with L[b] = 0 yields zeros), with the same scalars, grid and block:
+//     ar_flash_f32_lens, ar_flash_bf16_lens, ar_flash_bf16_long_lens          (Q, K, V, O, M, L,  6 ints)
+//     ar_flash_sage_lens, ar_flash_sage_long_lens, ar_flash_sage_fp8_lens,
+//     ar_flash_sage_fp8_long_lens                                             (Q8, K8, V, O, M, L, SQ, SK,  ints as above)
+// (The reference's fused kernels take a dense [n, n] mask only, src/models/flash_attention.rs:389-396; its
+// Tensor API reaches key-padding masks through the general path, src/tensor/mod.rs:2405-2447.)
 // head_dim must be 64 or 128; any other value makes the kernel return without writing.
 // The *_long entries address K and V with 32-bit byte offsets: (N + 320) * head_dim * 2 < 2^31.
 #include "attn_fwd.h"
@@ -55,11 +63,12 @@ __device__ __forceinline__ void dense(long s[3], int H, int N, int D)
 
 // AttnParams of a dense launch whose grid is [query tiles, B * hq, 1]
 __device__ __forceinline__ AttnParams dense_params(const void *q, const void *k, const void *v, void *o, const float *m,
-                                                   int N, int D, int has_mask, int hq, int hkv)
+                                                   int N, int D, int has_mask, int hq, int hkv, const int *lens = nullptr)
 {
     AttnParams p = {};
     p.q = q; p.k = k; p.v = (const uint16_t *)v; p.o = o;
     p.mask = has_mask ? m : nullptr;
+    p.kv_len = lens;
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     dense(p.qs, hq, N, D);
     dense(p.ks, hkv, N, D);
@@ -75,14 +84,15 @@ __device__ __forceinline__ AttnParams dense_params(const void *q, const void *k,
 
 }  // namespace
 
-extern "C" __global__ void __launch_bounds__(256) ar_flash_f32(const float *Q, const float *K, const float *V, float *O,
-                                                                const float *M, int N, int head_dim, int causal,
-                                                                int has_mask, int hq, int hkv)
+namespace {
+__device__ __forceinline__ void flash_f32_entry(float *lds, const float *Q, const float *K, const float *V, float *O,
+                                                const float *M, const int *L, int N, int head_dim, int causal, int has_mask,
+                                                int hq, int hkv)
 {
-    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<128>()];
     FlashF32Params p = {};
     p.q = Q; p.k = K; p.v = V; p.o = O;
     p.mask = has_mask ? M : nullptr;
+    p.kv_len = L;
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nq = (int)gridDim.x;
     dense(p.qs, hq, N, head_dim);
@@ -97,6 +107,23 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_f32(const float *Q, c
         if (causal) flash_f32_body<128, 4, true>(p, lds, wg);
         else flash_f32_body<128, 4, false>(p, lds, wg);
     }
+}
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_f32(const float *Q, const float *K, const float *V, float *O,
+                                                                const float *M, int N, int head_dim, int causal,
+                                                                int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<128>()];
+    flash_f32_entry(lds, Q, K, V, O, M, nullptr, N, head_dim, causal, has_mask, hq, hkv);
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_f32_lens(const float *Q, const float *K, const float *V, float *O,
+                                                                     const float *M, const int *L, int N, int head_dim,
+                                                                     int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) float lds[flash_f32_lds_floats<128>()];
+    flash_f32_entry(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
 }
 
 extern "C" __global__ void __launch_bounds__(256) ar_fl_fwd(const float *Q, const float *K, const float *V, float *O,
@@ -251,12 +278,12 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_bwd_dkv_short(const floa
     else bwd_dkv_body<64, 4, false, true>(p, lds, wg);
 }
 
-extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
-                                                                 uint16_t *O, const float *M, int N, int head_dim, int causal,
-                                                                 int has_mask, int hq, int hkv)
+namespace {
+__device__ __forceinline__ void flash_bf16_entry(unsigned char *lds, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                 uint16_t *O, const float *M, const int *L, int N, int head_dim, int causal,
+                                                 int has_mask, int hq, int hkv)
 {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_BF16, false>()];
-    AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, has_mask, hq, hkv);
+    AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, has_mask, hq, hkv, L);
     const int wg = linear_wg();
 #define AR_BF16(DD)                                                                                       \
     do {                                                                                                  \
@@ -271,6 +298,23 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16(const uint16_t *
     if (head_dim == 64) AR_BF16(64);
     else if (head_dim == 128) AR_BF16(128);
 #undef AR_BF16
+}
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                 uint16_t *O, const float *M, int N, int head_dim, int causal,
+                                                                 int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_BF16, false>()];
+    flash_bf16_entry(lds, Q, K, V, O, M, nullptr, N, head_dim, causal, has_mask, hq, hkv);
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16_lens(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                      uint16_t *O, const float *M, const int *L, int N,
+                                                                      int head_dim, int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_BF16, false>()];
+    flash_bf16_entry(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
 }
 
 // sequences of at most 256 keys: all of K/V of the head in LDS at once, 8 waves (two per 32 queries on
@@ -292,13 +336,13 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_short(const uint
     }
 }
 
-extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
-                                                                      uint16_t *O, const float *M, int N, int head_dim,
-                                                                      int causal, int has_mask, int hq, int hkv)
+namespace {
+__device__ __forceinline__ void flash_bf16_long_entry(unsigned char *lds, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                      uint16_t *O, const float *M, const int *L, int N, int head_dim, int causal,
+                                                      int has_mask, int hq, int hkv)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_BF16>()];
     if (has_mask) return;  // this entry has no additive mask: the host picks ar_flash_bf16 for those
-    AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, 0, hq, hkv);
+    AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, 0, hq, hkv, L);
     const int wg = linear_wg();
     if (head_dim == 64) {
         if (causal) attn_pipe_body<64, true, MODE_BF16, false>(p, lds, wg);
@@ -308,15 +352,32 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long(const uint1
         else attn_pipe_body<128, false, MODE_BF16, false>(p, lds, wg);
     }
 }
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                      uint16_t *O, const float *M, int N, int head_dim,
+                                                                      int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_BF16>()];
+    flash_bf16_long_entry(lds, Q, K, V, O, M, nullptr, N, head_dim, causal, has_mask, hq, hkv);
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long_lens(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                           uint16_t *O, const float *M, const int *L, int N,
+                                                                           int head_dim, int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_BF16>()];
+    flash_bf16_long_entry(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
+}
 
 namespace {
 // ar_flash_sage / ar_flash_sage_fp8: the general kernel on pre-quantised operands, QMODE = MODE_I8 or MODE_FP8
 template <int QMODE>
 __device__ __forceinline__ void flash_sage_entry(unsigned char *lds, const void *Q8, const void *K8, const uint16_t *V, float *O,
-                                                 const float *M, const float *SQ, const float *SK, int N, int head_dim, int causal,
-                                                 int has_mask, int hq, int hkv, int bq, int bk)
+                                                 const float *M, const int *L, const float *SQ, const float *SK, int N, int head_dim,
+                                                 int causal, int has_mask, int hq, int hkv, int bq, int bk)
 {
-    AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, has_mask, hq, hkv);
+    AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, has_mask, hq, hkv, L);
     p.sq = SQ; p.sk = SK;
     p.bq = bq; p.bk = bk;
     // K scales that are uniform over a 64-key tile (bk = 64 * 2^n) are a scalar per tile; any other
@@ -353,7 +414,16 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_sage(const int8_t *Q8
                                                                  int bq, int bk)
 {
     __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_I8, true>()];
-    flash_sage_entry<MODE_I8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
+    flash_sage_entry<MODE_I8>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_lens(const int8_t *Q8, const int8_t *K8, const uint16_t *V, float *O,
+                                                                      const float *M, const int *L, const float *SQ, const float *SK,
+                                                                      int N, int head_dim, int causal, int has_mask, int hq, int hkv,
+                                                                      int bq, int bk)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_I8, true>()];
+    flash_sage_entry<MODE_I8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
 }
 
 // the FP8 E4M3 variant (the reference's AR_FP8 = 1 source, src/runtime/cuda_flash_sage.rs:82-84): same
@@ -364,19 +434,29 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_fp8(const uint8_
                                                                      int hkv, int bq, int bk)
 {
     __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_FP8, true>()];
-    flash_sage_entry<MODE_FP8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
+    flash_sage_entry<MODE_FP8>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
+}
+
+extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_fp8_lens(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
+                                                                          float *O, const float *M, const int *L, const float *SQ,
+                                                                          const float *SK, int N, int head_dim, int causal,
+                                                                          int has_mask, int hq, int hkv, int bq, int bk)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 4, MODE_FP8, true>()];
+    flash_sage_entry<MODE_FP8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
 }
 
 // ar_flash_sage_long / ar_flash_sage_fp8_long: the pipelined kernel on pre-quantised operands
 template <int QMODE>
 __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const void *Q8, const void *K8, const uint16_t *V, void *O,
-                                                      const float *M, const float *SQ, const float *SK, int N, int head_dim,
-                                                      int causal, int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
+                                                      const float *M, const int *L, const float *SQ, const float *SK, int N,
+                                                      int head_dim, int causal, int has_mask, int hq, int hkv, int bq, int bk,
+                                                      int out_f32)
 {
     int shift = 0;
     while ((64 << shift) < bk) ++shift;
     if (has_mask || (64 << shift) != bk) return;  // the general kernels cover those
-    AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, 0, hq, hkv);
+    AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, 0, hq, hkv, L);
     p.sq = SQ; p.sk = SK;
     p.bq = bq; p.bk = bk;
     p.bk_tile_shift = shift;
@@ -402,7 +482,16 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_
                                                                       int hkv, int bq, int bk, int out_f32)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8>()];
-    flash_sage_long_entry<MODE_I8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+    flash_sage_long_entry<MODE_I8>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long_lens(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
+                                                                           void *O, const float *M, const int *L, const float *SQ,
+                                                                           const float *SK, int N, int head_dim, int causal,
+                                                                           int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8>()];
+    flash_sage_long_entry<MODE_I8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
 extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
@@ -411,7 +500,17 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long(const u
                                                                           int hkv, int bq, int bk, int out_f32)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8>()];
-    flash_sage_long_entry<MODE_FP8>(lds, Q8, K8, V, O, M, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+    flash_sage_long_entry<MODE_FP8>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long_lens(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
+                                                                               void *O, const float *M, const int *L, const float *SQ,
+                                                                               const float *SK, int N, int head_dim, int causal,
+                                                                               int has_mask, int hq, int hkv, int bq, int bk,
+                                                                               int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8>()];
+    flash_sage_long_entry<MODE_FP8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
 // ---- Sage pre-pass (the quantiser the reference runs inside its attention kernel,

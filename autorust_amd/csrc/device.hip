@@ -410,6 +410,86 @@ extern "C" int arhip_module_load(arhip_device *dev, const void *image, size_t le
     return ARHIP_OK;
 }
 
+// What the attention entry points of attn_kernels.hsaco (include/arhip_kernels.h) require of a launch.
+// Given anything else they return without writing (or, with a wrong workgroup shape, compute on
+// partly loaded tiles), and the caller's output is uninitialised memory with rc 0: a launch by one of
+// these names is therefore checked here first.  Other names (probes, a host's own kernels) are not.
+namespace {
+struct named_entry {
+    const char *name;
+    int nbufs;        // device pointers
+    int nvals;        // 32-bit scalars: n, head_dim, causal, has_mask, hq, hkv [, bq, bk [, out_f32]]
+    unsigned block;   // workgroup size
+    int rows;         // queries (keys for dK/dV) per workgroup: grid.x = ceil(n / rows)
+    bool d64_only;    // head_dim must be 64
+    bool no_mask;     // has_mask must be 0
+    bool pipelined;   // 32-bit K/V offsets, bk = 64 * 2^j
+    int max_n;        // 0 = any
+    bool kv_grid;     // grid.y counts kv heads (dK/dV)
+};
+const named_entry NAMED[] = {
+    {"ar_flash_f32", 5, 6, 256, 128, false, false, false, 0, false},
+    {"ar_flash_f32_lens", 6, 6, 256, 128, false, false, false, 0, false},
+    {"ar_flash_f32_short", 5, 6, 256, 32, true, false, false, 0, false},
+    {"ar_flash_bf16", 5, 6, 256, 128, false, false, false, 0, false},
+    {"ar_flash_bf16_lens", 6, 6, 256, 128, false, false, false, 0, false},
+    {"ar_flash_bf16_long", 5, 6, 512, 256, false, true, true, 0, false},
+    {"ar_flash_bf16_long_lens", 6, 6, 512, 256, false, true, true, 0, false},
+    {"ar_flash_bf16_short", 5, 6, 512, 128, false, true, false, 256, false},
+    {"ar_flash_sage", 7, 8, 256, 128, false, false, false, 0, false},
+    {"ar_flash_sage_lens", 8, 8, 256, 128, false, false, false, 0, false},
+    {"ar_flash_sage_fp8", 7, 8, 256, 128, false, false, false, 0, false},
+    {"ar_flash_sage_fp8_lens", 8, 8, 256, 128, false, false, false, 0, false},
+    {"ar_flash_sage_long", 7, 9, 512, 256, false, true, true, 0, false},
+    {"ar_flash_sage_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
+    {"ar_flash_sage_fp8_long", 7, 9, 512, 256, false, true, true, 0, false},
+    {"ar_flash_sage_fp8_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
+    {"ar_fl_fwd", 6, 6, 256, 128, false, false, false, 0, false},
+    {"ar_fl_fwd_short", 6, 6, 256, 32, true, false, false, 0, false},
+    {"ar_fl_bwd_dq", 8, 6, 256, 128, false, false, false, 0, false},
+    {"ar_fl_bwd_dq_short", 8, 6, 256, 32, true, false, false, 0, false},
+    {"ar_fl_bwd_dkv", 9, 6, 256, 128, false, false, false, 0, true},
+    {"ar_fl_bwd_dkv_short", 9, 6, 256, 32, true, false, false, 0, true},
+};
+
+int check_named_entry(const char *name, const unsigned grid[3], const unsigned block[3], int nbufs, const int64_t *vals,
+                      int nvals)
+{
+    const named_entry *e = nullptr;
+    for (const named_entry &c : NAMED)
+        if (std::strcmp(c.name, name) == 0) e = &c;
+    if (!e) return ARHIP_OK;
+    ARHIP_REQUIRE(nbufs == e->nbufs && nvals == e->nvals, "arhip_launch: %s takes %d buffers and %d scalars, got %d and %d", name,
+                  e->nbufs, e->nvals, nbufs, nvals);
+    ARHIP_REQUIRE(block[0] == e->block && block[1] == 1 && block[2] == 1, "arhip_launch: %s runs with block [%u,1,1], got [%u,%u,%u]",
+                  name, e->block, block[0], block[1], block[2]);
+    const int64_t n = vals[0], d = vals[1], has_mask = vals[3], hq = vals[4], hkv = vals[5];
+    ARHIP_REQUIRE(n > 0 && n <= ((int64_t)1 << 24), "arhip_launch: %s: n = %lld", name, (long long)n);
+    ARHIP_REQUIRE(d == 64 || (d == 128 && !e->d64_only), "arhip_launch: %s: head_dim %lld (%s)", name, (long long)d,
+                  e->d64_only ? "64 only" : "64 or 128");
+    ARHIP_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0, "arhip_launch: %s: hq = %lld, hkv = %lld", name, (long long)hq, (long long)hkv);
+    ARHIP_REQUIRE(!(e->no_mask && has_mask), "arhip_launch: %s takes no additive mask (has_mask must be 0)", name);
+    ARHIP_REQUIRE(e->max_n == 0 || n <= e->max_n, "arhip_launch: %s: n = %lld exceeds %d", name, (long long)n, e->max_n);
+    ARHIP_REQUIRE((int64_t)grid[0] == (n + e->rows - 1) / e->rows && grid[2] == 1,
+                  "arhip_launch: %s: grid [%u,%u,%u], expected [ceil(n/%d) = %lld, B*h, 1]", name, grid[0], grid[1], grid[2], e->rows,
+                  (long long)((n + e->rows - 1) / e->rows));
+    ARHIP_REQUIRE(grid[1] % (unsigned)(e->kv_grid ? hkv : hq) == 0, "arhip_launch: %s: grid.y = %u is not a multiple of %s = %lld", name,
+                  grid[1], e->kv_grid ? "hkv" : "hq", (long long)(e->kv_grid ? hkv : hq));
+    if (e->nvals >= 8) ARHIP_REQUIRE(vals[6] >= 1 && vals[7] >= 1, "arhip_launch: %s: block sizes bq = %lld, bk = %lld", name,
+                                     (long long)vals[6], (long long)vals[7]);
+    if (e->pipelined) {
+        ARHIP_REQUIRE((n + 320) * d * 2 < ((int64_t)1 << 31), "arhip_launch: %s addresses K/V with 32-bit offsets: (n + 320) * head_dim * 2 "
+                      "must stay below 2^31", name);
+        if (e->nvals >= 8) {
+            const int64_t bk = vals[7];
+            ARHIP_REQUIRE(bk >= 64 && (bk & (bk - 1)) == 0, "arhip_launch: %s needs K scales uniform over 64-key tiles (bk = 64 * 2^j), got bk = %lld",
+                          name, (long long)bk);
+        }
+    }
+    return ARHIP_OK;
+}
+}  // namespace
+
 extern "C" int arhip_launch(arhip_device *dev, void *module, const char *name,
                             const unsigned grid[3], const unsigned block[3],
                             void *const *bufs, int nbufs,
@@ -436,6 +516,7 @@ extern "C" int arhip_launch(arhip_device *dev, void *module, const char *name,
     }
     ARHIP_REQUIRE(block[0] * block[1] * block[2] >= 1 && block[0] * block[1] * block[2] <= 1024,
                   "arhip_launch: block of %u threads", block[0] * block[1] * block[2]);
+    if (int rc = check_named_entry(name, grid, block, nbufs, vals, nvals)) return rc;
     void *ptrs[64];
     int32_t v32[64];
     int64_t v64[64];

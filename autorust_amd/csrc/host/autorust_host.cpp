@@ -103,6 +103,9 @@ std::optional<double> Device::run_host_kernel(const std::string &src, const std:
         void *mod = nullptr;
         check(arhip_module_load(dev_, image.data(), image.size(), &mod));
         it = modules_.emplace(src, mod).first;
+        uint64_t key = 1469598103934665603ull;  // content hash of the compiled artifact (FNV-1a), printed by KPROF
+        for (char c : image) key = (key ^ (unsigned char)c) * 1099511628211ull;
+        module_keys_[src] = key;
         if (getenv("AUTORUST_KERNEL_INFO"))  // ops_cuda.rs:902-918 prints per-kernel resources at load
             std::fprintf(stderr, "[hip] loaded %s (%zu bytes) for %s\n", src.c_str(), image.size(), this->name().c_str());
     }
@@ -129,9 +132,17 @@ std::optional<double> Device::run_host_kernel(const std::string &src, const std:
         g[i] = (unsigned)std::max<int64_t>(global[i], 0);       // negatives clamp to 0 (session.rs:241-251)
         l[i] = (unsigned)std::max<int64_t>((*local)[i], 0);
     }
+    // AUTORUST_KPROF (src/runtime/ops_cuda.rs:879-885, 1004-1012): a launch that would not wait is
+    // synchronised and reported as `KPROF <name> <secs> <content key>` on stderr; it serialises the
+    // stream, so it is a profiling aid, not a benchmark mode.
+    const bool kprof = !wait && getenv("AUTORUST_KPROF") != nullptr;
     double secs = 0.0;
     check(arhip_launch(dev_, it->second, name.c_str(), g, l, ptrs.data(), (int)nb, sv.data(), bits.data(), (int)sv.size(),
-                       wait ? 1 : 0, &secs));
+                       (wait || kprof) ? 1 : 0, &secs));
+    if (kprof) {
+        std::fprintf(stderr, "KPROF\t%s\t%.6f\t%016llx\n", name.c_str(), secs, (unsigned long long)module_keys_[src]);
+        return secs;
+    }
     if (wait) return secs;
     return std::nullopt;
 }
@@ -215,6 +226,13 @@ Tensor Tensor::from_slice(const std::shared_ptr<Device> &dev, const float *data,
         dev->check(arhip_cast_bf16(dev->handle(), (const float *)tmp, (uint16_t *)t.ptr(), n, 1, nullptr));
         dev->release(tmp, (size_t)n * 4);
     }
+    return t;
+}
+
+Tensor Tensor::from_i32(const std::shared_ptr<Device> &dev, const int32_t *data, const std::vector<int64_t> &shape)
+{
+    Tensor t = empty(dev, shape, DType::Int32);
+    if (t.numel() > 0) dev->check(arhip_copyin(dev->handle(), t.ptr(), data, (size_t)t.numel() * 4));
     return t;
 }
 
@@ -383,7 +401,8 @@ static bool short_f32(const std::shared_ptr<Device> &dev, int64_t b, int64_t hea
 }
 
 std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
-                                           const Tensor &out, bool is_causal, Kernel kern, const Settings &st)
+                                           const Tensor &out, bool is_causal, Kernel kern, const Settings &st,
+                                           const Tensor *key_lengths)
 {
     const int64_t b = q.shape()[0], h = q.shape()[1], n = q.shape()[2], d = q.shape()[3], hk = k.shape()[1];
     const auto dev = q.device();
@@ -393,26 +412,35 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     const Tensor mslot = has_mask ? *attn_mask : out;
     const std::vector<int64_t> vals = {n, d, (int64_t)is_causal, (int64_t)has_mask, h, hk};  // cuda_flash_bf16.rs:550-561
     std::vector<HostCall> calls;
+    // the attention kernel itself: with key lengths it is the `_lens` twin, whose argument list has the
+    // lengths ([b] int32) right after the mask slot (slot 4 in every forward entry)
+    auto attn_call = [&](const std::string &name, std::vector<Tensor> bufs, std::vector<DType> types, std::array<int64_t, 3> global,
+                         std::array<int64_t, 3> local, const std::vector<int64_t> &scalars) {
+        if (!key_lengths) return make_call(dev, name.c_str(), bufs, types, global, local, scalars);
+        bufs.insert(bufs.begin() + 5, *key_lengths);
+        types.insert(types.begin() + 5, DType::Int32);
+        return make_call(dev, (name + "_lens").c_str(), bufs, types, global, local, scalars);
+    };
 
     if (kern == Kernel::FlashF32) {
         // few, short heads: 32 queries per workgroup instead of 128 (the rule of arhip_flash_fwd)
-        if (d == 64 && short_f32(dev, b, h, n))
+        if (d == 64 && short_f32(dev, b, h, n) && !key_lengths)
             calls.push_back(make_call(dev, "ar_flash_f32_short", {q, k, v, out, mslot}, {F, F, F, F, F},
                                       {(n + 31) / 32, b * h, 1}, {256, 1, 1}, vals));
         else
-            calls.push_back(make_call(dev, "ar_flash_f32", {q, k, v, out, mslot}, {F, F, F, F, F}, {(n + 127) / 128, b * h, 1},
+            calls.push_back(attn_call("ar_flash_f32", {q, k, v, out, mslot}, {F, F, F, F, F}, {(n + 127) / 128, b * h, 1},
                                       {256, 1, 1}, vals));
         return calls;
     }
     if (kern == Kernel::FlashBf16) {
-        if (!has_mask && n <= 256 && b * h * ((n + 127) / 128) <= 4 * (int64_t)dev->compute_units())
+        if (!has_mask && !key_lengths && n <= 256 && b * h * ((n + 127) / 128) <= 4 * (int64_t)dev->compute_units())
             calls.push_back(make_call(dev, "ar_flash_bf16_short", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 127) / 128, b * h, 1}, {512, 1, 1}, vals));
         else if (!has_mask && long_variant(dev, b, h, n, d))
-            calls.push_back(make_call(dev, "ar_flash_bf16_long", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
+            calls.push_back(attn_call("ar_flash_bf16_long", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 255) / 256, b * h, 1}, {512, 1, 1}, vals));
         else
-            calls.push_back(make_call(dev, "ar_flash_bf16", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
+            calls.push_back(attn_call("ar_flash_bf16", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 127) / 128, b * h, 1}, {256, 1, 1}, vals));
         return calls;
     }
@@ -465,17 +493,17 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     const bool tile_uniform = ((int64_t)64 << shift) == bk;
     if (!has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
         svals.push_back(bf16_in ? 0 : 1);  // out_f32
-        calls.push_back(make_call(dev, st.sage_fp8 ? "ar_flash_sage_fp8_long" : "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
+        calls.push_back(attn_call(st.sage_fp8 ? "ar_flash_sage_fp8_long" : "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
                                   {(n + 255) / 256, b * h, 1}, {512, 1, 1}, svals));
     } else if (!bf16_in) {
-        calls.push_back(make_call(dev, general, {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, F, F, F, F},
+        calls.push_back(attn_call(general, {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, F, F, F, F},
                                   {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
     } else {
         // ar_flash_sage stores f32 (the reference's convention); bf16 tensors get their bf16 result
         // through one more cast
         Tensor o32 = Tensor::empty(dev, {b, h, n, d}, F);
         const Tensor m2 = has_mask ? *attn_mask : o32;
-        calls.push_back(make_call(dev, general, {q8, k8, vb, o32, m2, sq, sk}, {I8, I8, BF, F, F, F, F},
+        calls.push_back(attn_call(general, {q8, k8, vb, o32, m2, sq, sk}, {I8, I8, BF, F, F, F, F},
                                   {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
         const int64_t no = b * h * n * d;
         calls.push_back(make_call(dev, "ar_cast_bf16", {o32, out}, {F, BF}, {std::min<int64_t>((no + 255) / 256, 16384), 1, 1},
@@ -485,7 +513,8 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
 }
 
 std::optional<Tensor> fused_attention_ex(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
-                                         bool is_causal, bool enable_gqa, bool quantized, Session &sess, const Settings &st)
+                                         bool is_causal, bool enable_gqa, bool quantized, Session &sess, const Settings &st,
+                                         const Tensor *key_lengths)
 {
     static std::once_flag sage_note;
     bool sage_declined = false;
@@ -497,13 +526,17 @@ std::optional<Tensor> fused_attention_ex(const Tensor &q, const Tensor &k, const
     if (sage_declined)
         note_once(sage_note, "[attention] sage: quantized attention is not available for this shape/settings: using the exact kernel");
     if (kern == Kernel::None) return std::nullopt;
+    // key lengths: one int32 per batch entry on the same device; anything else is the caller's general path
+    if (key_lengths && (key_lengths->dtype() != DType::Int32 || key_lengths->shape() != std::vector<int64_t>{q.shape()[0]} ||
+                        key_lengths->device() != q.device()))
+        return std::nullopt;
 
     const int64_t b = q.shape()[0], h = q.shape()[1], n = q.shape()[2], d = q.shape()[3];
     // out: bf16 for bf16 tensors, f32 otherwise (:514-530); no host-side zero fill is needed, the
     // kernels write every element
     Tensor out = Tensor::empty(q.device(), {b, h, n, d}, q.dtype());
     // Record the launches for replay and run them now (flash_attention.rs:696-701).
-    for (const HostCall &call : attention_host_calls(q, k, v, attn_mask, out, is_causal, kern, st)) {
+    for (const HostCall &call : attention_host_calls(q, k, v, attn_mask, out, is_causal, kern, st, key_lengths)) {
         sess.capture_host(call);
         call.exec();
     }
@@ -578,14 +611,15 @@ std::optional<Grads> fused_attention_backward(const Tensor &q, const Tensor &k, 
 // ---- Tensor API -----------------------------------------------------------------------
 
 Tensor Tensor::attention_kind(const Tensor &key, const Tensor &value, const Tensor *mask, double dropout_p, bool is_causal,
-                              std::optional<AttentionKind> force, Session *sess, const Settings &st) const
+                              std::optional<AttentionKind> force, Session *sess, const Settings &st,
+                              const Tensor *key_lengths) const
 {
     bool quantized = false;
     const bool fused = wants_fused(force, st, dropout_p, sess != nullptr, &quantized);
     // fewer K/V heads than Q heads means GQA (tensor/mod.rs:2185-2195)
     const bool gqa = shape_.size() == 4 && key.shape().size() == 4 && key.shape()[1] != shape_[1];
     if (fused) {
-        auto t = fused_attention_ex(*this, key, value, mask, is_causal, gqa, quantized, *sess, st);
+        auto t = fused_attention_ex(*this, key, value, mask, is_causal, gqa, quantized, *sess, st, key_lengths);
         if (t) return *t;
     }
     // tensor/mod.rs:2207: the general scaled_dot_product_attention (generated kernels) runs here in the
@@ -596,22 +630,22 @@ Tensor Tensor::attention_kind(const Tensor &key, const Tensor &value, const Tens
 
 Tensor Tensor::attention(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal) const
 {
-    return attention_kind(k, v, mask, dropout_p, is_causal, std::nullopt, nullptr, Settings());
+    return attention_kind(k, v, mask, dropout_p, is_causal, std::nullopt, nullptr, Settings(), nullptr);
 }
 Tensor Tensor::attention_with(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal,
-                              Session &sess, const Settings &st) const
+                              Session &sess, const Settings &st, const Tensor *key_lengths) const
 {
-    return attention_kind(k, v, mask, dropout_p, is_causal, std::nullopt, &sess, st);
+    return attention_kind(k, v, mask, dropout_p, is_causal, std::nullopt, &sess, st, key_lengths);
 }
 Tensor Tensor::flash_attention_with(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal,
-                                    Session &sess, const Settings &st) const
+                                    Session &sess, const Settings &st, const Tensor *key_lengths) const
 {
-    return attention_kind(k, v, mask, dropout_p, is_causal, AttentionKind::Flash, &sess, st);
+    return attention_kind(k, v, mask, dropout_p, is_causal, AttentionKind::Flash, &sess, st, key_lengths);
 }
 Tensor Tensor::sage_attention_with(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal,
-                                   Session &sess, const Settings &st) const
+                                   Session &sess, const Settings &st, const Tensor *key_lengths) const
 {
-    return attention_kind(k, v, mask, dropout_p, is_causal, AttentionKind::Sage, &sess, st);
+    return attention_kind(k, v, mask, dropout_p, is_causal, AttentionKind::Sage, &sess, st, key_lengths);
 }
 
 }  // namespace autorust

@@ -83,6 +83,7 @@ private:
     int ordinal_;
     std::map<size_t, std::vector<void *>> free_;
     std::map<std::string, void *> modules_;  // code object path -> loaded module
+    std::map<std::string, uint64_t> module_keys_;  // code object path -> content hash (the key KPROF prints)
     uint64_t raw_allocs_ = 0;
 };
 
@@ -105,6 +106,8 @@ public:
     static Tensor from_slice(const std::shared_ptr<Device> &dev, const float *data, const std::vector<int64_t> &shape,
                              DType dtype);                       // tensor/mod.rs:1088
     static Tensor empty(const std::shared_ptr<Device> &dev, const std::vector<int64_t> &shape, DType dtype);
+    // an Int32 tensor (the only integer tensors of this path: per-batch key lengths)
+    static Tensor from_i32(const std::shared_ptr<Device> &dev, const int32_t *data, const std::vector<int64_t> &shape);
     size_t nbytes() const;
     Tensor reshape(const std::vector<int64_t> &shape) const;     // view: shares storage
     std::vector<float> to_list() const;                          // tensor/mod.rs:695 (bf16 widened to f32)
@@ -115,24 +118,27 @@ public:
     const std::shared_ptr<Device> &device() const { return st_->dev; }
     bool defined() const { return (bool)st_; }
 
-    // The public attention entry points (tensor/mod.rs:2045-2161).  `used` (optional) receives
-    // the kind that actually ran.  When the policy or the kernels decline, the call throws
-    // "TGERR: ... general SDPA path ..." because that path is outside this build.
+    // The public attention entry points (tensor/mod.rs:2045-2161).  When the policy or the kernels
+    // decline, the call throws "TGERR: ... general SDPA path ..." because that path is outside this build.
+    // `key_lengths` (optional, Int32 [b]) is a key-padding mask: batch i attends to keys [0, key_lengths[i])
+    // only.  The reference reaches such masks through its general path (a broadcast bool mask,
+    // tensor/mod.rs:2405-2447); here they stay on the fused kernels (the `*_lens` entry points).
     Tensor attention(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal) const;
     Tensor attention_with(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal,
-                          Session &sess, const Settings &st) const;
+                          Session &sess, const Settings &st, const Tensor *key_lengths = nullptr) const;
     Tensor flash_attention_with(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal,
-                                Session &sess, const Settings &st) const;
+                                Session &sess, const Settings &st, const Tensor *key_lengths = nullptr) const;
     Tensor sage_attention_with(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal,
-                               Session &sess, const Settings &st) const;
+                               Session &sess, const Settings &st, const Tensor *key_lengths = nullptr) const;
 private:
     Tensor attention_kind(const Tensor &k, const Tensor &v, const Tensor *mask, double dropout_p, bool is_causal,
-                          std::optional<AttentionKind> force, Session *sess, const Settings &st) const;
+                          std::optional<AttentionKind> force, Session *sess, const Settings &st,
+                          const Tensor *key_lengths) const;
     std::shared_ptr<Storage> st_;
     std::vector<int64_t> shape_;
     DType dtype_ = DType::Float32;
     friend std::optional<Tensor> fused_attention_ex(const Tensor &, const Tensor &, const Tensor &, const Tensor *, bool,
-                                                    bool, bool, Session &, const Settings &);
+                                                    bool, bool, Session &, const Settings &, const Tensor *);
 };
 
 // ---- captured launches ----------------------------------------------------------------
@@ -165,8 +171,11 @@ enum class Kernel { None = -1, FlashF32 = ARHIP_K_FLASH_F32, FlashBf16 = ARHIP_K
 // The launches one fused attention call consists of, in order (the pre-pass of the quantised
 // path first, the attention kernel last), without running them: the `host_call` builders of
 // src/runtime/cuda_flash{,_bf16,_sage}.rs (cuda_flash_bf16.rs:580-599).
+// With `key_lengths` (Int32 [b]) the attention kernel is the `*_lens` twin and the lengths ride as one more
+// buffer after the mask slot.
 std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
-                                           const Tensor &out, bool is_causal, Kernel kern, const Settings &st);
+                                           const Tensor &out, bool is_causal, Kernel kern, const Settings &st,
+                                           const Tensor *key_lengths = nullptr);
 
 // The gates of fused_attention_ex without touching a device (flash_attention.rs:358-472):
 // which kernel would run, or Kernel::None (=> the caller's SDPA).
@@ -185,7 +194,7 @@ std::optional<Tensor> fused_attention_kind(const Tensor &q, const Tensor &k, con
                                            Session &sess, const Settings &st);               // :303-320
 std::optional<Tensor> fused_attention_ex(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *attn_mask,
                                          bool is_causal, bool enable_gqa, bool quantized, Session &sess,
-                                         const Settings &st);                                // :348-702
+                                         const Settings &st, const Tensor *key_lengths = nullptr);  // :348-702
 uint64_t selections(Kernel k);   // cuda_flash_bf16.rs:458-461
 
 // ---- training: forward with the saved log-sum-exp, and the backward ------------------------

@@ -84,6 +84,13 @@ void *arh_tensor_from_slice(void *d, const float *data, const int64_t *shape, in
         return new Tensor(Tensor::from_slice(*(std::shared_ptr<Device> *)d, data, shp, (DType)dtype));
     }, nullptr);
 }
+void *arh_tensor_from_i32(void *d, const int32_t *data, const int64_t *shape, int ndim)
+{
+    return guard([&]() -> void * {
+        std::vector<int64_t> shp(shape, shape + ndim);
+        return new Tensor(Tensor::from_i32(*(std::shared_ptr<Device> *)d, data, shp));
+    }, nullptr);
+}
 void arh_tensor_free(void *t) { delete (Tensor *)t; }
 int64_t arh_tensor_numel(void *t) { return ((Tensor *)t)->numel(); }
 int arh_tensor_dtype(void *t) { return (int)((Tensor *)t)->dtype(); }
@@ -148,20 +155,22 @@ int arh_session_replay(void *s)
 }
 
 // api: 0 attention (no session), 1 attention_with, 2 flash_attention_with, 3 sage_attention_with
+// key_lengths: an Int32 [b] tensor or NULL (the *_with entry points only)
 void *arh_attention(void *q, void *k, void *v, void *mask, double dropout_p, int is_causal, int api, void *sess,
-                    const arh_settings *st)
+                    const arh_settings *st, void *key_lengths)
 {
     return guard([&]() -> void * {
         const Tensor &tq = *(Tensor *)q, &tk = *(Tensor *)k, &tv = *(Tensor *)v;
-        const Tensor *tm = (const Tensor *)mask;
+        const Tensor *tm = (const Tensor *)mask, *tl = (const Tensor *)key_lengths;
+        if (api == 0 && tl) throw std::runtime_error("TGERR: key lengths need a session (the *_with entry points)");
         const Settings s = to_settings(st);
         Session *ss = sess ? &((SessionBox *)sess)->sess : nullptr;
         if (api != 0 && !ss) throw std::runtime_error("TGERR: a session is required for the *_with entry points");
         switch (api) {
         case 0: return new Tensor(tq.attention(tk, tv, tm, dropout_p, is_causal != 0));
-        case 1: return new Tensor(tq.attention_with(tk, tv, tm, dropout_p, is_causal != 0, *ss, s));
-        case 2: return new Tensor(tq.flash_attention_with(tk, tv, tm, dropout_p, is_causal != 0, *ss, s));
-        default: return new Tensor(tq.sage_attention_with(tk, tv, tm, dropout_p, is_causal != 0, *ss, s));
+        case 1: return new Tensor(tq.attention_with(tk, tv, tm, dropout_p, is_causal != 0, *ss, s, tl));
+        case 2: return new Tensor(tq.flash_attention_with(tk, tv, tm, dropout_p, is_causal != 0, *ss, s, tl));
+        default: return new Tensor(tq.sage_attention_with(tk, tv, tm, dropout_p, is_causal != 0, *ss, s, tl));
         }
     }, nullptr);
 }
@@ -234,6 +243,25 @@ int arh_wants_fused(int force, const arh_settings *st, double dropout_p, int has
     if (quantized) *quantized = qz;
     return w;
 }
+
+// Device::run_host_kernel with device pointers and 32-bit scalars (the generic seam, for tests of
+// its own behaviour: argument marshalling, the KPROF line).  Returns 0, or -1 with arh_last_error().
+int arh_run_host_kernel(void *d, const char *src, const char *name, void **bufs, int nbufs, const int64_t *vals, int nvals,
+                        const int64_t *global3, const int64_t *local3, int wait, double *secs)
+{
+    return guard([&]() -> int {
+        std::vector<std::pair<int64_t, DType>> sig;
+        for (int i = 0; i < nbufs; ++i) sig.emplace_back(i, DType::Float32);
+        for (int i = 0; i < nvals; ++i) sig.emplace_back(nbufs + i, DType::Int32);
+        const std::vector<void *> b(bufs, bufs + nbufs);
+        const std::vector<int64_t> v(vals, vals + nvals);
+        const std::array<int64_t, 3> loc = {local3[0], local3[1], local3[2]};
+        const auto r = (*(std::shared_ptr<Device> *)d)->run_host_kernel(src, name, sig, b, global3, loc, v, wait != 0);
+        if (secs) *secs = r ? *r : -1.0;
+        return 0;
+    }, -1);
+}
+void *arh_tensor_ptr(void *t) { return ((Tensor *)t)->ptr(); }
 
 uint64_t arh_selections(int kernel) { return selections((Kernel)kernel); }
 

@@ -67,6 +67,12 @@ def host():
         h.arh_device_raw_allocs.argtypes = [vp]
         h.arh_tensor_from_slice.restype = vp
         h.arh_tensor_from_slice.argtypes = [vp, ctypes.c_void_p, i64p, ci, ci]
+        h.arh_tensor_from_i32.restype = vp
+        h.arh_tensor_from_i32.argtypes = [vp, ctypes.c_void_p, i64p, ci]
+        h.arh_tensor_ptr.restype = vp
+        h.arh_tensor_ptr.argtypes = [vp]
+        h.arh_run_host_kernel.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(vp), ci, i64p, ci, i64p, i64p, ci,
+                                          ctypes.POINTER(ctypes.c_double)]
         h.arh_tensor_free.argtypes = [vp]
         h.arh_tensor_numel.restype = ctypes.c_int64
         h.arh_tensor_numel.argtypes = [vp]
@@ -85,7 +91,7 @@ def host():
         h.arh_fused_attention_train.argtypes = [vp, vp, vp, vp, ci, vp, pvp, pvp]
         h.arh_fused_attention_backward.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, vp, pvp, pvp, pvp]
         h.arh_attention.restype = vp
-        h.arh_attention.argtypes = [vp, vp, vp, vp, ctypes.c_double, ci, ci, vp, ctypes.POINTER(Settings)]
+        h.arh_attention.argtypes = [vp, vp, vp, vp, ctypes.c_double, ci, ci, vp, ctypes.POINTER(Settings), vp]
         h.arh_plan_fused.argtypes = [i64p, ci, i64p, ci, i64p, ci, ci, ci, ci, i64p, ci, ci, ci, ci,
                                      ctypes.POINTER(Settings), ctypes.POINTER(ci)]
         h.arh_wants_fused.argtypes = [ci, ctypes.POINTER(Settings), ctypes.c_double, ci, ctypes.POINTER(ci)]
@@ -123,6 +129,16 @@ class HipDevice:
     @property
     def raw_allocs(self):
         return int(host().arh_device_raw_allocs(self.h))
+
+    def run_host_kernel(self, src, name, bufs, vals, global_, local, wait=True):
+        """`Compiled::run_host_kernel` (src/runtime/device.rs:383-402) on Tensor buffers and 32-bit
+        scalars; returns the elapsed device seconds, or None for a launch that did not wait."""
+        ptrs = (ctypes.c_void_p * max(len(bufs), 1))(*[host().arh_tensor_ptr(b.h) for b in bufs])
+        secs = ctypes.c_double(-1.0)
+        if host().arh_run_host_kernel(self.h, src.encode(), name.encode(), ptrs, len(bufs), _i64(list(vals)), len(vals),
+                                      _i64(list(global_)), _i64(list(local)), int(wait), ctypes.byref(secs)) != 0:
+            raise _err()
+        return None if secs.value < 0 else secs.value
 
 
 class Session:
@@ -180,6 +196,16 @@ class Tensor:
             raise _err()
         return Tensor(h)
 
+    @staticmethod
+    def from_i32(dev, data, shape=None):
+        """An Int32 tensor (per-batch key lengths)."""
+        data = np.ascontiguousarray(data, dtype=np.int32)
+        shape = data.shape if shape is None else shape
+        h = host().arh_tensor_from_i32(dev.h, data.ctypes.data, _i64(list(shape)), len(shape))
+        if not h:
+            raise _err()
+        return Tensor(h)
+
     @property
     def shape(self):
         out = (ctypes.c_int64 * 8)()
@@ -196,10 +222,11 @@ class Tensor:
             raise _err()
         return out.reshape(self.shape)
 
-    def _call(self, api, k, v, mask, dropout_p, is_causal, sess, settings):
+    def _call(self, api, k, v, mask, dropout_p, is_causal, sess, settings, key_lengths=None):
         st = settings if settings is not None else Settings.default()
         h = host().arh_attention(self.h, k.h, v.h, mask.h if mask is not None else None, float(dropout_p),
-                                 int(is_causal), api, sess.h if sess is not None else None, ctypes.byref(st))
+                                 int(is_causal), api, sess.h if sess is not None else None, ctypes.byref(st),
+                                 key_lengths.h if key_lengths is not None else None)
         if not h:
             raise _err()
         return Tensor(h)
@@ -207,14 +234,14 @@ class Tensor:
     def attention(self, k, v, mask=None, dropout_p=0.0, is_causal=False):
         return self._call(0, k, v, mask, dropout_p, is_causal, None, None)
 
-    def attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None):
-        return self._call(1, k, v, mask, dropout_p, is_causal, sess, settings)
+    def attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None, key_lengths=None):
+        return self._call(1, k, v, mask, dropout_p, is_causal, sess, settings, key_lengths)
 
-    def flash_attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None):
-        return self._call(2, k, v, mask, dropout_p, is_causal, sess, settings)
+    def flash_attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None, key_lengths=None):
+        return self._call(2, k, v, mask, dropout_p, is_causal, sess, settings, key_lengths)
 
-    def sage_attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None):
-        return self._call(3, k, v, mask, dropout_p, is_causal, sess, settings)
+    def sage_attention_with(self, k, v, mask, dropout_p, is_causal, sess, settings=None, key_lengths=None):
+        return self._call(3, k, v, mask, dropout_p, is_causal, sess, settings, key_lengths)
 
 
 def fused_attention(q, k, v, sess, kind=None, settings=None):

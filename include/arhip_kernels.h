@@ -95,6 +95,23 @@
 #define ARHIP_KERNEL_SAGE_QUANT_ROWS_BF16 "ar_sage_quant_rows_bf16"
 #define ARHIP_KERNEL_CAST_BF16 "ar_cast_bf16"
 
+/* Key-padding masks on the named-kernel seam.  The reference's fused kernels admit a dense [n, n] mask
+ * only (src/models/flash_attention.rs:389-396) and leave per-batch key lengths to its general path
+ * (src/tensor/mod.rs:2405-2447); these twins keep padded batches on the fused path.  Each takes the
+ * arguments of the entry it is named after with one more pointer directly after M:
+ *     const int *L   [B] int32; batch b attends to keys [0, L[b]) only (clamped to [0, N]; 0 => zeros)
+ * and the same scalars, grid and block.
+ *   ar_flash_f32_lens, ar_flash_bf16_lens, ar_flash_bf16_long_lens      (Q, K, V, O, M, L, 6 ints)
+ *   ar_flash_sage_lens, ar_flash_sage_fp8_lens                           (Q8, K8, V, O, M, L, SQ, SK, 6 ints, bq, bk)
+ *   ar_flash_sage_long_lens, ar_flash_sage_fp8_long_lens                 (..., bq, bk, out_f32) */
+#define ARHIP_KERNEL_FLASH_F32_LENS "ar_flash_f32_lens"
+#define ARHIP_KERNEL_FLASH_BF16_LENS "ar_flash_bf16_lens"
+#define ARHIP_KERNEL_FLASH_BF16_LONG_LENS "ar_flash_bf16_long_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_LENS "ar_flash_sage_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_LONG_LENS "ar_flash_sage_long_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_LENS "ar_flash_sage_fp8_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_LONG_LENS "ar_flash_sage_fp8_long_lens"
+
 /* FP8 E4M3 variant (the reference's `src(fp8 = true)`, src/runtime/cuda_flash_sage.rs:82-84, 92-147):
  * the same argument lists as ar_flash_sage / ar_sage_quant_{blocks,rows}_*, with E4M3 codes
  * (scale = absmax / 448) in place of int8 values. */

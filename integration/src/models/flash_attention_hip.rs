@@ -47,21 +47,25 @@ pub enum HipKernel {
 
 /// The launches of one fused attention call on a HIP device.  `bufs` is
 /// `[q, k, v, out, mask-or-out]` exactly as for the CUDA arms (`flash_attention.rs:531-540`).
+/// `lens` is the realised int32 `[b]` buffer of per-batch key lengths, if the caller has a
+/// key-padding mask in that form (the CUDA arms send such masks to the general path,
+/// `flash_attention.rs:389-396`); it selects the `_lens` entry points.
 #[allow(clippy::too_many_arguments)]
-pub fn hip_calls(dev: &str, kernel: HipKernel, bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> Vec<HostCall> {
+pub fn hip_calls(dev: &str, kernel: HipKernel, bufs: Vec<Buffer>, lens: Option<Buffer>, b: i64, h: i64, n: i64, d: i64,
+                 opts: Options) -> Vec<HostCall> {
     match kernel {
         HipKernel::F32 => {
             hip_flash::note_selected(0);
-            vec![hip_flash::host_call_f32(dev, bufs, b, h, n, d, opts)]
+            vec![hip_flash::host_call_f32(dev, bufs, lens, b, h, n, d, opts)]
         }
         HipKernel::Bf16 => {
             hip_flash::note_selected(1);
-            vec![hip_flash::host_call_bf16(dev, bufs, b, h, n, d, opts)]
+            vec![hip_flash::host_call_bf16(dev, bufs, lens, b, h, n, d, opts)]
         }
         HipKernel::Sage { bf16_in, scratch, opts: sage } => {
             hip_flash::note_selected(2);
             let [q, k, v, o, m]: [Buffer; 5] = bufs.try_into().unwrap_or_else(|_| panic!("TGERR: sage expects 5 buffers"));
-            hip_flash::host_calls_sage(dev, q, k, v, o, m, scratch, bf16_in, b, h, n, d, opts, sage)
+            hip_flash::host_calls_sage(dev, q, k, v, o, m, lens, scratch, bf16_in, b, h, n, d, opts, sage)
         }
     }
 }

@@ -16,6 +16,13 @@
 //! | `ar_flash_sage`      | 256   | `[ceil(n/128), b*h, 1]` | same `+ bq, bk`; buffers `+ SQ, SK`; O is f32|
 //! | `ar_flash_sage_long` | 512   | `[ceil(n/256), b*h, 1]` | same `+ bq, bk, out_f32`                     |
 //! | `ar_flash_sage_fp8`, `ar_flash_sage_fp8_long` | as the int8 pair, on E4M3 codes (`SageOptions::fp8`)        |
+//! | `<entry>_lens`       | as `<entry>` | as `<entry>`     | one more buffer after the mask slot: `L`, int32 `[b]` key lengths |
+//!
+//! Key-padding masks: the CUDA fused kernels admit a dense `[n, n]` mask only
+//! (`src/models/flash_attention.rs:389-396`); here a per-batch key length keeps a padded batch on the
+//! fused kernels.  Every builder takes `lens: Option<Buffer>`; with `Some`, the `_lens` twin of the
+//! entry is named and the buffer is inserted after the mask slot.  `ar_flash_f32_short` and
+//! `ar_flash_bf16_short` have no twin: the builders fall through to the general entries then.
 //!
 //! Unlike the CUDA Sage kernel, which quantises inside the attention kernel (K once per query
 //! block, `cuda_flash_sage.rs:248-278`), the quantiser is a pre-pass of its own here, with K
@@ -117,6 +124,22 @@ fn call(name: &str, bufs: Vec<Buffer>, buf_types: &[DTypeId], global: [i64; 3], 
     }
 }
 
+/// The attention launch itself: with key lengths, the `_lens` twin with `L` (int32 `[b]`) after the
+/// mask slot (index 4 in every forward entry).
+#[allow(clippy::too_many_arguments)]
+fn attn_call(name: &str, mut bufs: Vec<Buffer>, buf_types: &[DTypeId], lens: Option<Buffer>, global: [i64; 3], local: [i64; 3],
+             vals: Vec<i64>) -> HostCall {
+    match lens {
+        None => call(name, bufs, buf_types, global, local, vals, &[]),
+        Some(l) => {
+            let mut types = buf_types.to_vec();
+            bufs.insert(5, l);
+            types.insert(5, dtype::INT32);
+            call(&format!("{name}_lens"), bufs, &types, global, local, vals, &[])
+        }
+    }
+}
+
 fn vals(n: i64, d: i64, h: i64, opts: Options) -> Vec<i64> {
     // `cuda_flash_bf16.rs:550-561`, with the head size as a real parameter
     vec![n, d, opts.causal as i64, opts.has_mask as i64, h, opts.h_kv]
@@ -136,26 +159,28 @@ fn short_f32(dev: &str, b: i64, heads: i64, n: i64, d: i64) -> bool {
     d == 64 && b * heads * ((n + 127) / 128) < 2 * crate::runtime::ops_hip::compute_units(dev)
 }
 
-/// fp32 exact mode: `bufs = [q, k, v, o, mask-or-o]`, all f32 `[b, h, n, d]`.
-pub fn host_call_f32(dev: &str, bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
+/// fp32 exact mode: `bufs = [q, k, v, o, mask-or-o]`, all f32 `[b, h, n, d]`; `lens`: int32 `[b]` key lengths.
+#[allow(clippy::too_many_arguments)]
+pub fn host_call_f32(dev: &str, bufs: Vec<Buffer>, lens: Option<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
     let f = dtype::FLOAT32;
-    if short_f32(dev, b, h, n, d) {
+    if lens.is_none() && short_f32(dev, b, h, n, d) {
         call("ar_flash_f32_short", bufs, &[f, f, f, f, f], [(n + 31) / 32, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
     } else {
-        call("ar_flash_f32", bufs, &[f, f, f, f, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+        attn_call("ar_flash_f32", bufs, &[f, f, f, f, f], lens, [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts))
     }
 }
 
-/// bf16: `bufs = [q, k, v, o, mask-or-o]`, q/k/v/o bf16, mask f32 `[n, n]`.
-pub fn host_call_bf16(dev: &str, bufs: Vec<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
+/// bf16: `bufs = [q, k, v, o, mask-or-o]`, q/k/v/o bf16, mask f32 `[n, n]`; `lens`: int32 `[b]` key lengths.
+#[allow(clippy::too_many_arguments)]
+pub fn host_call_bf16(dev: &str, bufs: Vec<Buffer>, lens: Option<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
     let (bf, f) = (dtype::BFLOAT16, dtype::FLOAT32);
-    if !opts.has_mask && n <= 256 && b * h * ((n + 127) / 128) <= 4 * crate::runtime::ops_hip::compute_units(dev) {
+    if !opts.has_mask && lens.is_none() && n <= 256 && b * h * ((n + 127) / 128) <= 4 * crate::runtime::ops_hip::compute_units(dev) {
         // all of K/V of a head in LDS at once: the ViT sequence lengths
         call("ar_flash_bf16_short", bufs, &[bf, bf, bf, bf, f], [(n + 127) / 128, b * h, 1], [512, 1, 1], vals(n, d, h, opts), &[])
     } else if !opts.has_mask && long_variant(dev, b, h, n, d) {
-        call("ar_flash_bf16_long", bufs, &[bf, bf, bf, bf, f], [(n + 255) / 256, b * h, 1], [512, 1, 1], vals(n, d, h, opts), &[])
+        attn_call("ar_flash_bf16_long", bufs, &[bf, bf, bf, bf, f], lens, [(n + 255) / 256, b * h, 1], [512, 1, 1], vals(n, d, h, opts))
     } else {
-        call("ar_flash_bf16", bufs, &[bf, bf, bf, bf, f], [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts), &[])
+        attn_call("ar_flash_bf16", bufs, &[bf, bf, bf, bf, f], lens, [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts))
     }
 }
 
@@ -172,8 +197,26 @@ pub struct SageScratch {
     pub o32: Option<Buffer>, // f32 result when the tensors are bf16 and the general kernel runs
 }
 
+/// One quantiser launch: per-row scales (`blk == 1`) or per-block scales.  A free function (it returns
+/// the launch instead of pushing it) so that the caller's vector is never borrowed across calls.
+#[allow(clippy::too_many_arguments)]
+fn quant_call(fmt: &str, sfx: &str, x: DTypeId, src: &Buffer, dst: &Buffer, scales: &Buffer, mean: &Buffer, b: i64, heads: i64,
+              n: i64, d: i64, blk: i64, nblk: i64, smooth: bool) -> HostCall {
+    let (f, i8t) = (dtype::FLOAT32, dtype::INT8);
+    let bufs = vec![src.clone(), dst.clone(), scales.clone(), mean.clone()];
+    if blk == 1 {
+        let rows = b * heads * n;
+        let rpb = 256 / (d / 8);
+        call(&format!("ar_sage_quant_rows_{fmt}{sfx}"), bufs, &[x, i8t, f, f], [(rows + rpb - 1) / rpb, 1, 1], [256, 1, 1],
+             vec![n, d, rows, smooth as i64], &[2])
+    } else {
+        call(&format!("ar_sage_quant_blocks_{fmt}{sfx}"), bufs, &[x, i8t, f, f], [nblk, b * heads, 1], [256, 1, 1],
+             vec![n, d, blk, nblk, smooth as i64], &[])
+    }
+}
+
 /// Sage int8: the launches of one call, in order.  `q, k, v, o` are f32 or bf16 (`bf16_in`),
-/// `mask` is the f32 `[n, n]` additive mask or `o` again.
+/// `mask` is the f32 `[n, n]` additive mask or `o` again; `lens`: int32 `[b]` key lengths.
 #[allow(clippy::too_many_arguments)]
 pub fn host_calls_sage(
     dev: &str,
@@ -182,6 +225,7 @@ pub fn host_calls_sage(
     v: Buffer,
     o: Buffer,
     mask: Buffer,
+    lens: Option<Buffer>,
     s: SageScratch,
     bf16_in: bool,
     b: i64,
@@ -200,19 +244,7 @@ pub fn host_calls_sage(
     let (bq, bk) = (sage.block_q, sage.block_k);
     let (nqb, nkb, nchunk) = ((n + bq - 1) / bq, (n + bk - 1) / bk, (n + 63) / 64);
     let mut calls = Vec::new();
-    let mut quant = |src: &Buffer, dst: &Buffer, scales: &Buffer, heads: i64, blk: i64, nblk: i64, smooth: bool| {
-        let bufs = vec![src.clone(), dst.clone(), scales.clone(), s.mean.clone()];
-        if blk == 1 {
-            let rows = b * heads * n;
-            let rpb = 256 / (d / 8);
-            calls.push(call(&format!("ar_sage_quant_rows_{q8fmt}{sfx}"), bufs, &[x, i8t, f, f], [(rows + rpb - 1) / rpb, 1, 1], [256, 1, 1],
-                            vec![n, d, rows, smooth as i64], &[2]));
-        } else {
-            calls.push(call(&format!("ar_sage_quant_blocks_{q8fmt}{sfx}"), bufs, &[x, i8t, f, f], [nblk, b * heads, 1], [256, 1, 1],
-                            vec![n, d, blk, nblk, smooth as i64], &[]));
-        }
-    };
-    quant(&q, &s.q8, &s.sq, h, bq, nqb, false);
+    calls.push(quant_call(q8fmt, sfx, x, &q, &s.q8, &s.sq, &s.mean, b, h, n, d, bq, nqb, false));
     if sage.smooth_k {
         let cpb = 256 / (d / 8);
         calls.push(call(&format!("ar_sage_kmean_partial_{sfx}"), vec![k.clone(), s.part.clone()], &[x, f],
@@ -220,7 +252,7 @@ pub fn host_calls_sage(
         calls.push(call("ar_sage_kmean_final", vec![s.part.clone(), s.mean.clone()], &[f, f], [b * hk, 1, 1], [d, 1, 1],
                         vec![n, d, nchunk], &[]));
     }
-    quant(&k, &s.k8, &s.sk, hk, bk, nkb, sage.smooth_k);
+    calls.push(quant_call(q8fmt, sfx, x, &k, &s.k8, &s.sk, &s.mean, b, hk, n, d, bk, nkb, sage.smooth_k));
     let vb = match &s.vb {
         Some(vb) => {
             let nv = b * hk * n * d;
@@ -236,18 +268,18 @@ pub fn host_calls_sage(
     let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
     if !opts.has_mask && tile_uniform && long_variant(dev, b, h, n, d) {
         sv.push(!bf16_in as i64); // out_f32
-        calls.push(call(long, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f],
-                        [(n + 255) / 256, b * h, 1], [512, 1, 1], sv, &[]));
+        calls.push(attn_call(long, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
+                             [(n + 255) / 256, b * h, 1], [512, 1, 1], sv));
     } else if !bf16_in {
-        calls.push(call(general, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f],
-                        [(n + 127) / 128, b * h, 1], [256, 1, 1], sv, &[]));
+        calls.push(attn_call(general, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f], lens,
+                             [(n + 127) / 128, b * h, 1], [256, 1, 1], sv));
     } else {
         // the general kernel stores f32 (the CUDA kernel's convention); bf16 tensors get their
         // bf16 result through one more cast
         let o32 = s.o32.expect("o32 scratch for bf16 tensors");
         let m2 = if opts.has_mask { mask } else { o32.clone() };
-        calls.push(call(general, vec![s.q8, s.k8, vb, o32.clone(), m2, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f],
-                        [(n + 127) / 128, b * h, 1], [256, 1, 1], sv, &[]));
+        calls.push(attn_call(general, vec![s.q8, s.k8, vb, o32.clone(), m2, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f], lens,
+                             [(n + 127) / 128, b * h, 1], [256, 1, 1], sv));
         let no = b * h * n * d;
         calls.push(call("ar_cast_bf16", vec![o32, o], &[f, bf], [((no + 255) / 256).min(16384), 1, 1], [256, 1, 1], vec![no], &[0]));
     }

@@ -229,6 +229,15 @@ pub struct HipProgram {
     module: *mut c_void,
     name: CString,
     signature: Vec<(i64, crate::dtype::DTypeId)>,
+    /// Content hash of the code object (FNV-1a), printed by KPROF so that two kernels that share a
+    /// name can be told apart (`ops_cuda.rs:873-876`).
+    key: u64,
+}
+
+/// `AUTORUST_KPROF=1` synchronises after each kernel and prints its name/time (`ops_cuda.rs:879-885`).
+fn kprof_enabled() -> bool {
+    static ON: std::sync::OnceLock<bool> = std::sync::OnceLock::new();
+    *ON.get_or_init(|| crate::helpers::env::get("AUTORUST_KPROF").is_some())
 }
 
 impl HipProgram {
@@ -240,7 +249,8 @@ impl HipProgram {
         if crate::helpers::env::get_os("AUTORUST_KERNEL_INFO").is_some() {
             eprintln!("[hip] {}: code object of {} bytes loaded for {}", elf.name, elf.lib.len(), inner.arch);
         }
-        HipProgram { inner, module, name: CString::new(elf.name.clone()).unwrap(), signature: elf.signature.clone() }
+        let key = elf.lib.iter().fold(0xcbf29ce484222325u64, |h, b| (h ^ *b as u64).wrapping_mul(0x100000001b3));
+        HipProgram { inner, module, name: CString::new(elf.name.clone()).unwrap(), signature: elf.signature.clone(), key }
     }
 }
 
@@ -277,6 +287,8 @@ impl Prog for HipProgram {
         let ls = local_size.unwrap_or([1, 1, 1]);
         let grid = [global_size[0] as c_uint, global_size[1] as c_uint, global_size[2] as c_uint];
         let block = [ls[0] as c_uint, ls[1] as c_uint, ls[2] as c_uint];
+        // KPROF (`ops_cuda.rs:1004-1012`): a launch that would not wait is synchronised and reported
+        let kprof = kprof_enabled() && !wait;
         let mut secs = 0f64;
         let rc = unsafe {
             self.inner.sym::<FnLaunch>(b"arhip_launch")(
@@ -290,11 +302,15 @@ impl Prog for HipProgram {
                 scalars.as_ptr(),
                 bits.as_ptr(),
                 scalars.len() as c_int,
-                wait as c_int,
+                (wait || kprof) as c_int,
                 &mut secs,
             )
         };
         self.inner.check(rc);
+        if kprof {
+            eprintln!("KPROF\t{}\t{secs:.6}\t{:016x}", self.name.to_string_lossy(), self.key);
+            return Some(secs);
+        }
         wait.then_some(secs)
     }
 

@@ -70,7 +70,7 @@ def run_flash(dev, q, k, v, dtype, mask=None, kv_len=None, causal=False, scale=N
 
 
 def run_sage(dev, q, k, v, bq, bk, smooth=True, in_dtype=F32, out_dtype=F32, mask=None, kv_len=None, causal=False,
-             dbg_sel=None):
+             dbg_sel=None, scale=None):
     """Quantise Q and K, cast V, run the int8 kernel; returns everything the checks need."""
     B, Hq, N, D = q.shape
     Hkv = k.shape[1]
@@ -94,7 +94,7 @@ def run_sage(dev, q, k, v, bq, bk, smooth=True, in_dtype=F32, out_dtype=F32, mas
         dl = bufs.put(np.ascontiguousarray(kv_len, np.int32)) if kv_len is not None else None
         dbg = bufs.new(32 * 64 * 4) if dbg_sel is not None else None
         dev.sage_fwd(q8, k8, sq, sk, dv, do, B, Hq, Hkv, N, D, bq, bk, out_dtype=out_dtype, mask=dm, kv_len=dl,
-                     causal=causal, dbg_logits=dbg, dbg_sel=dbg_sel)
+                     causal=causal, dbg_logits=dbg, dbg_sel=dbg_sel, scale=scale)
         res = {
             "q8": q8.copyout(np.int8, q.shape), "k8": k8.copyout(np.int8, k.shape),
             "sq": sq.copyout(np.float32, (B, Hq, nqb)), "sk": sk.copyout(np.float32, (B, Hkv, nkb)),

@@ -65,11 +65,10 @@ def test_ar_flash_f32_short_by_name(dev, kernels, case):
         dev.launch(kernels, "ar_flash_f32_short", _grid(n, 32, b, hq), (256, 1, 1), [dq, dk, dv, do, dm],
                    [n, d, int(causal), int(has_mask), hq, hkv])
         got = do.copyout(np.float32, q.shape)
-        # any other head_dim: the kernel returns without writing
-        do2 = bufs.new(q.nbytes)
-        dev.launch(kernels, "ar_flash_f32_short", _grid(n, 32, b, hq), (256, 1, 1), [dq, dk, dv, do2, do2],
-                   [n, 128, int(causal), 0, hq, hkv])
-        assert not do2.copyout(np.float32, q.shape).any()
+        # any other head_dim is refused on the host (the kernel itself would return without writing)
+        with pytest.raises(_lib.ArhipError, match="head_dim 128"):
+            dev.launch(kernels, "ar_flash_f32_short", _grid(n, 32, b, hq), (256, 1, 1), [dq, dk, dv, do, do],
+                       [n, 128, int(causal), 0, hq, hkv])
     want = oracle.flash_f32(q, k, v, mask=mask, causal=causal)
     assert np.abs(got - want).max() < 2e-5
 
@@ -319,3 +318,116 @@ def test_ar_flash_bf16_short_by_name(dev, kernels, n, d, causal, hkv):
         got = synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
     want = oracle.attn_bf16(q, k, v, causal=causal)
     assert np.abs(got - want).max() < 5e-3
+
+
+# ---- key lengths on the named-kernel seam (the `_lens` twins) --------------------------------------
+
+def _lens_for(b, n):
+    """Per-batch key lengths: the first batch entry short, the last full, 0 < L <= n."""
+    return np.array([max(1, (n * (3 + 2 * i)) // (3 + 2 * b)) if i < b - 1 else n for i in range(b)], np.int32)
+
+
+@pytest.mark.parametrize("case", [(2, 4, 2, 100, 128, True, False), (2, 4, 1, 64, 64, False, True), (3, 2, 2, 300, 64, True, True)],
+                         ids=str)
+def test_flash_lens_entries_by_name(dev, kernels, case):
+    """ar_flash_f32_lens and ar_flash_bf16_lens: (Q, K, V, O, M, L, 6 ints), L int32 [b]."""
+    b, hq, hkv, n, d, causal, has_mask = case
+    q, k, v = fill_qkv(b, hq, hkv, n, d)
+    mask = ref_mask(n).reshape(n, n) if has_mask else None
+    lens = _lens_for(b, n)
+    vals = [n, d, int(causal), int(has_mask), hq, hkv]
+    with Bufs(dev) as bufs:
+        dl = bufs.put(lens)
+        dq, dk, dv = bufs.put(q), bufs.put(k), bufs.put(v)
+        do = bufs.new(q.nbytes)
+        dm = bufs.put(mask) if has_mask else do
+        dev.launch(kernels, "ar_flash_f32_lens", _grid(n, 128, b, hq), (256, 1, 1), [dq, dk, dv, do, dm, dl], vals)
+        got32 = do.copyout(np.float32, q.shape)
+        bq_, bk_, bv_ = (bufs.put(synth.to_bf16_bits(t)) for t in (q, k, v))
+        bo = bufs.new(q.size * 2)
+        bm = dm if has_mask else bo
+        dev.launch(kernels, "ar_flash_bf16_lens", _grid(n, 128, b, hq), (256, 1, 1), [bq_, bk_, bv_, bo, bm, dl], vals)
+        got16 = synth.from_bf16_bits(bo.copyout(np.uint16, q.shape))
+    assert np.abs(got32 - oracle.flash_f32(q, k, v, mask=mask, causal=causal, kv_len=lens)).max() < 2e-5
+    assert np.abs(got16 - oracle.attn_bf16(q, k, v, mask=mask, causal=causal, kv_len=lens)).max() < 5e-3
+
+
+@pytest.mark.parametrize("bq,bk", [(1, 1), (128, 64)])
+def test_sage_lens_entries_by_name(dev, kernels, bq, bk):
+    """ar_flash_sage_lens / ar_flash_sage_long_lens: (Q8, K8, V, O, M, L, SQ, SK, ints)."""
+    b, hq, hkv, n, d = 2, 4, 2, 700, 128
+    q = synth.normal(31, (b, hq, n, d))
+    k = synth.normal(32, (b, hkv, n, d)) + np.float32(3.0) * synth.normal(34, (1, hkv, 1, d))
+    v = synth.normal(33, (b, hkv, n, d))
+    lens = np.array([333, 700], np.int32)
+    with Bufs(dev) as bufs:
+        dl = bufs.put(lens)
+        q8, sq, _, h_q8, h_sq, _ = _quantise_by_name(dev, kernels, bufs, q, bq, False, F32)
+        k8, sk, _, h_k8, h_sk, _ = _quantise_by_name(dev, kernels, bufs, k, bk, True, F32)
+        dv = bufs.put(synth.to_bf16_bits(v))
+        do = bufs.new(q.size * 4)
+        dev.launch(kernels, "ar_flash_sage_lens", _grid(n, 128, b, hq), (256, 1, 1), [q8, k8, dv, do, do, dl, sq, sk],
+                   [n, d, 1, 0, hq, hkv, bq, bk])
+        got = do.copyout(np.float32, q.shape)
+        want = oracle.sage(h_q8, h_k8, h_sq, h_sk, v, bq, bk, causal=True, kv_len=lens)
+        assert np.abs(got - want).max() < 4e-3
+        if bk == 64:
+            dp = bufs.new(q.size * 4)
+            dev.launch(kernels, "ar_flash_sage_long_lens", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, dp, dp, dl, sq, sk],
+                       [n, d, 1, 0, hq, hkv, bq, bk, 1])
+            assert np.abs(dp.copyout(np.float32, q.shape) - want).max() < 4e-3
+        else:
+            # per-key scales are the general kernel's: the pipelined entry refuses them on the host
+            with pytest.raises(_lib.ArhipError, match="bk = 64"):
+                dev.launch(kernels, "ar_flash_sage_long_lens", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, do, do, dl, sq, sk],
+                           [n, d, 1, 0, hq, hkv, bq, bk, 1])
+
+
+def test_decoder_shape_with_key_lengths_by_name(dev, kernels):
+    """The causal decoder configuration (B4 H32 S2048 D128, per-batch key lengths uniform in [S/2, S]) launched by
+    name: `ar_flash_bf16_long_lens` through arhip_launch, sampled rows against the bf16 emulation with
+    the same lengths, within three bf16 steps."""
+    from gpu_util import bf16_ulps
+    b, h, n, d = 4, 32, 2048, 128
+    q, k, v = (synth.normal(3001 + i, (b, h, n, d)) for i in range(3))
+    lens = synth.randint(3005, b, n // 2, n)
+    with Bufs(dev) as bufs:
+        dq, dk, dv = (bufs.put(synth.to_bf16_bits(t)) for t in (q, k, v))
+        dl = bufs.put(lens)
+        do = bufs.new(q.size * 2, zero=False)
+        dev.launch(kernels, "ar_flash_bf16_long_lens", _grid(n, 256, b, h), (512, 1, 1), [dq, dk, dv, do, do, dl],
+                   [n, d, 1, 0, h, h])
+        got = synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+    assert np.isfinite(got).all()
+    rows = np.array([0, 1, 63, 64, 255, 256, 1023, 1024, 1500, 2047], np.int32)
+    for bi, hi in ((0, 0), (1, 17), (3, 31)):
+        rr = np.unique(np.concatenate([rows, [lens[bi] - 1, min(lens[bi], n - 1)]])).astype(np.int32)
+        want = oracle.attn_bf16(q[bi:bi + 1, hi:hi + 1], k[bi:bi + 1, hi:hi + 1], v[bi:bi + 1, hi:hi + 1], causal=True,
+                                kv_len=lens[bi:bi + 1], rows=rr)
+        assert bf16_ulps(got[bi:bi + 1, hi:hi + 1][:, :, rr], want) <= 3.0
+
+
+def test_named_entries_refuse_launches_they_cannot_run(dev, kernels):
+    """A launch that a named attention entry cannot serve is an error on the host (EINVAL), never a
+    kernel that returns without writing its output."""
+    b, hq, n, d = 1, 2, 300, 64
+    with Bufs(dev) as bufs:
+        x = bufs.new(b * hq * n * d * 4)
+        m = bufs.new(n * n * 4)
+        ok = [n, d, 0, 0, hq, hq]
+        bad = [
+            ("ar_flash_bf16_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, m], [n, d, 0, 1, hq, hq], "no additive mask"),
+            ("ar_flash_bf16_long", _grid(n, 256, b, hq), (256, 1, 1), [x, x, x, x, x], ok, r"block \[512,1,1\]"),
+            ("ar_flash_bf16_long", _grid(n, 128, b, hq), (512, 1, 1), [x, x, x, x, x], ok, "grid"),
+            ("ar_flash_bf16_short", _grid(n, 128, b, hq), (512, 1, 1), [x, x, x, x, x], ok, "exceeds 256"),
+            ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x, x], [n, 96, 0, 0, hq, hq], "head_dim 96"),
+            ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x], ok, "takes 5 buffers"),
+            ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x, x], [n, d, 0, 0, hq, 3], "hkv"),
+            ("ar_flash_sage_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x, x, x], [n, d, 0, 0, hq, hq, 128, 48, 0], "bk = 64"),
+            ("ar_fl_bwd_dkv_short", _grid(n, 32, b, hq), (256, 1, 1), [x] * 9, [n, 128, 0, 0, hq, hq], "64 only"),
+        ]
+        for name, grid, block, bufs_, vals, msg in bad:
+            with pytest.raises(_lib.ArhipError, match=msg):
+                dev.launch(kernels, name, grid, block, bufs_, vals)
+        # and the same entry with a launch it can serve still runs
+        dev.launch(kernels, "ar_flash_bf16_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x], ok)

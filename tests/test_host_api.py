@@ -345,3 +345,90 @@ def test_capture_and_replay(hdev):
     assert np.array_equal(out.to_list(), first) and np.array_equal(o2.to_list(), first2)
     err = float(np.abs(first - oracle.attn_bf16(q, k, v, causal=True)).max())
     assert err < 1.6e-2
+
+
+@gpu
+@pytest.mark.parametrize("api,dtype", [("attention_with", BFLOAT16), ("flash_attention_with", FLOAT32),
+                                       ("sage_attention_with", FLOAT32), ("sage_attention_with", BFLOAT16)])
+def test_key_lengths_through_the_tensor_api(hdev, api, dtype):
+    """A key-padding mask as per-batch key lengths through Tensor::*_with: the captured HostCall
+    names the `_lens` entry point, carries the lengths after the mask slot, and the result matches
+    the oracle with the same lengths (the reference sends such masks to its general path,
+    src/tensor/mod.rs:2405-2447, src/models/flash_attention.rs:389-396)."""
+    b, h, hk, n, d = 2, 4, 2, 300, 64
+    q, k, v = synth.normal(801, (b, h, n, d)), synth.normal(802, (b, hk, n, d)), synth.normal(803, (b, hk, n, d))
+    lens = np.array([123, 300], np.int32)
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape, dtype) for a in (q, k, v))
+    tl = Tensor.from_i32(hdev, lens)
+    sess = Session()
+    sess.begin_capture()
+    out = getattr(tq, api)(tk, tv, None, 0.0, True, sess, None, tl)
+    nsteps = sess.end_capture()
+    name, grid, vals = sess.step(nsteps - 1)
+    if api == "sage_attention_with" and dtype == BFLOAT16:
+        name, grid, vals = sess.step(nsteps - 2)      # the general int8 kernel stores f32; a cast follows
+    assert name.endswith("_lens"), name
+    src, local, nbufs, nvals, sig = sess.step_detail(nsteps - (2 if (api == "sage_attention_with" and dtype == BFLOAT16) else 1))
+    assert sig[5][1] == 4                                # DType::Int32 in the slot after the mask
+    got = out.to_list()
+    if api == "sage_attention_with":
+        qr, kr = (oracle.bf16_round(q), oracle.bf16_round(k)) if dtype == BFLOAT16 else (q, k)
+        q8, sq = oracle.quant_blocks(qr, 128)
+        k8, sk = oracle.quant_blocks(kr, 64, sub=oracle.k_mean(kr))
+        want = oracle.sage(q8, k8, sq, sk, v, 128, 64, causal=True, kv_len=lens, round_out=dtype == BFLOAT16)
+        assert np.abs(got - want).max() <= (2.0 ** -6 if dtype == BFLOAT16 else 4e-3)
+    elif dtype == BFLOAT16:
+        assert np.abs(got - oracle.attn_bf16(q, k, v, causal=True, kv_len=lens)).max() <= 2.0 ** -6
+    else:
+        assert np.abs(got - oracle.flash_f32(q, k, v, causal=True, kv_len=lens)).max() < 2e-5
+    # replay finds the lengths again
+    sess.replay()
+    assert np.array_equal(out.to_list(), got)
+    # lengths of the wrong shape: the fused kernels decline (the reference's None -> general path)
+    with pytest.raises(host.HostError, match="general SDPA path"):
+        getattr(tq, api)(tk, tv, None, 0.0, True, sess, None, Tensor.from_i32(hdev, np.array([1, 2, 3], np.int32)))
+
+
+@gpu
+def test_decoder_configuration_through_the_tensor_api(hdev):
+    """Causal decoder attention, B4 H32 S2048 D128 bf16 with key lengths uniform in [S/2, S], from
+    Tensor::attention_with: the pipelined `_lens` entry, sampled rows within three bf16 steps of the
+    bf16 emulation."""
+    from gpu_util import bf16_ulps
+    b, h, n, d = 4, 32, 2048, 128
+    q, k, v = (synth.normal(3001 + i, (b, h, n, d)) for i in range(3))
+    lens = synth.randint(3005, b, n // 2, n)
+    tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape, BFLOAT16) for a in (q, k, v))
+    sess = Session()
+    sess.begin_capture()
+    out = tq.attention_with(tk, tv, None, 0.0, True, sess, None, Tensor.from_i32(hdev, lens))
+    assert sess.end_capture() == 1 and sess.step(0)[0] == "ar_flash_bf16_long_lens"
+    got = out.to_list()
+    rows = np.array([0, 63, 64, 255, 256, 1023, 1024, 1500, 2047], np.int32)
+    for bi, hi in ((0, 3), (2, 30)):
+        rr = np.unique(np.concatenate([rows, [lens[bi] - 1, min(lens[bi], n - 1)]])).astype(np.int32)
+        want = oracle.attn_bf16(q[bi:bi + 1, hi:hi + 1], k[bi:bi + 1, hi:hi + 1], v[bi:bi + 1, hi:hi + 1], causal=True,
+                                kv_len=lens[bi:bi + 1], rows=rr)
+        assert bf16_ulps(got[bi:bi + 1, hi:hi + 1][:, :, rr], want) <= 3.0
+
+
+@gpu
+def test_kprof_line_of_run_host_kernel(hdev, capfd, monkeypatch):
+    """AUTORUST_KPROF: a launch that would not wait is synchronised and reported as
+    `KPROF\\t<name>\\t<secs>\\t<content key>` (src/runtime/ops_cuda.rs:879-885, 1004-1012)."""
+    import re
+    from autorust_amd import _lib
+    x = synth.normal(5, (1000,))
+    tx, ty = Tensor.from_slice(hdev, x, x.shape), Tensor.from_slice(hdev, np.zeros_like(x), x.shape)
+    capfd.readouterr()
+    assert hdev.run_host_kernel(_lib.PROBES_PATH, "probe_axpb", [tx, ty], [1000], [4, 1, 1], [256, 1, 1], wait=False) is None
+    assert "KPROF" not in capfd.readouterr().err
+    monkeypatch.setenv("AUTORUST_KPROF", "1")
+    secs = hdev.run_host_kernel(_lib.PROBES_PATH, "probe_axpb", [tx, ty], [1000], [4, 1, 1], [256, 1, 1], wait=False)
+    err = capfd.readouterr().err
+    m = re.search(r"^KPROF\tprobe_axpb\t(\d+\.\d{6})\t([0-9a-f]{16})$", err, re.M)
+    assert m and secs is not None and abs(float(m.group(1)) - secs) < 1e-6
+    assert np.array_equal(ty.to_list(), x * np.float32(3.0) + np.float32(1.0))
+    # a launch that waits anyway prints nothing (the reference's `kprof_enabled() && !wait`)
+    assert hdev.run_host_kernel(_lib.PROBES_PATH, "probe_axpb", [tx, ty], [1000], [4, 1, 1], [256, 1, 1], wait=True) is not None
+    assert "KPROF" not in capfd.readouterr().err
