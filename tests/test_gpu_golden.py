@@ -6,8 +6,9 @@ sizes are 4 and 8; the kernels take 64 or 128, so q, k and v are zero-padded alo
 (zero channels add nothing to q.k and give zero output channels) and the scale is passed as
 1/sqrt(original head size).  Additive and boolean masks become the kernels' dense [n, n] mask
 (boolean: 0 where allowed, -inf where not), the causal case uses the flag, GQA the kv-head count.
-Tolerance: the reference's own, 1e-5 * max(|want|, 1) (tests/nn_attention.rs:11-24), for fp32;
-2e-2 for bf16 and int8 against these fp32 results.
+Tolerance: the reference's own measure, |got - want| <= tol * max(|want|, 1) (tests/nn_attention.rs:11-24),
+with its tol = 1e-5 for fp32 and tol = 2e-2 for bf16 and int8 against these fp32 results (the vectors
+reach 19, where a bf16-stored output alone is off by up to 2^-9 * 19 = 0.04).
 """
 import json
 import os
@@ -60,7 +61,7 @@ def test_reference_vectors_bf16_kernel(dev, case, D):
     q, k, v, mask, want, d0 = _load(case, D)
     got = run_flash(dev, q, k, v, BF16, mask=mask, causal=case["is_causal"], scale=1.0 / np.sqrt(np.float32(d0)))
     assert not got[..., d0:].any()
-    assert np.abs(got[..., :d0] - want).max() <= 2e-2
+    assert np.all(np.abs(got[..., :d0] - want) <= 2e-2 * np.maximum(np.abs(want), 1.0))
 
 
 @pytest.mark.parametrize("case", _cases(), ids=lambda c: c["name"])
@@ -70,4 +71,4 @@ def test_reference_vectors_int8_kernel(dev, case):
     q, k, v, mask, want, d0 = _load(case, 64)
     res = run_sage(dev, q, k, v, 1, 1, smooth=False, mask=mask, causal=case["is_causal"],
                    scale=1.0 / np.sqrt(np.float32(d0)))
-    assert np.abs(res["out"][..., :d0] - want).max() <= 2e-2
+    assert np.all(np.abs(res["out"][..., :d0] - want) <= 2e-2 * np.maximum(np.abs(want), 1.0))

@@ -370,12 +370,15 @@ def test_sage_lens_entries_by_name(dev, kernels, bq, bk):
                    [n, d, 1, 0, hq, hkv, bq, bk])
         got = do.copyout(np.float32, q.shape)
         want = oracle.sage(h_q8, h_k8, h_sq, h_sk, v, bq, bk, causal=True, kv_len=lens)
-        assert np.abs(got - want).max() < 4e-3
+        # N(0,1) data: the kernel rounds P to bf16 relative to its running reference, the emulation
+        # relative to the final maximum; rows that few keys carry differ by up to 2 * 2^-9 * max|v|
+        tol = 2.0 ** -8 * float(np.abs(v).max())
+        assert np.abs(got - want).max() < tol
         if bk == 64:
             dp = bufs.new(q.size * 4)
             dev.launch(kernels, "ar_flash_sage_long_lens", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, dp, dp, dl, sq, sk],
                        [n, d, 1, 0, hq, hkv, bq, bk, 1])
-            assert np.abs(dp.copyout(np.float32, q.shape) - want).max() < 4e-3
+            assert np.abs(dp.copyout(np.float32, q.shape) - want).max() < tol
         else:
             # per-key scales are the general kernel's: the pipelined entry refuses them on the host
             with pytest.raises(_lib.ArhipError, match="bk = 64"):

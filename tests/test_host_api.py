@@ -428,7 +428,7 @@ def test_kprof_line_of_run_host_kernel(hdev, capfd, monkeypatch):
     err = capfd.readouterr().err
     m = re.search(r"^KPROF\tprobe_axpb\t(\d+\.\d{6})\t([0-9a-f]{16})$", err, re.M)
     assert m and secs is not None and abs(float(m.group(1)) - secs) < 1e-6
-    assert np.array_equal(ty.to_list(), x * np.float32(3.0) + np.float32(1.0))
+    assert np.abs(ty.to_list() - (x * np.float32(3.0) + np.float32(1.0))).max() < 1e-5   # the kernel may contract x * 3 + 1
     # a launch that waits anyway prints nothing (the reference's `kprof_enabled() && !wait`)
     assert hdev.run_host_kernel(_lib.PROBES_PATH, "probe_axpb", [tx, ty], [1000], [4, 1, 1], [256, 1, 1], wait=True) is not None
     assert "KPROF" not in capfd.readouterr().err
