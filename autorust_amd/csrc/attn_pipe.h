@@ -625,8 +625,19 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     };
     // the last unmasked tile hands a masked block to the look-ahead: it is peeled off
     const int nplain = (nfull < ntiles) ? max(nfull - 1, 0) : nfull;
+    // 8-bit operands: four tiles per trip, so that the stage of a tile (it % 4) and with it every LDS
+    // offset and transfer destination is a constant (15 vector and 23 scalar instructions fewer per
+    // tile: Sage B4 H32 S8192 3.05 -> 2.96 ms).  The bf16 loop body is larger and gains nothing from it.
+    const int nplain4 = (MODE != MODE_BF16) ? (nplain & ~3) : 0;
 #pragma clang loop unroll(disable)
-    for (int it = 0; it < nplain; ++it) tile_iter(PLAIN, PLAIN, PLAIN, it);
+    for (int it = 0; it < nplain4; it += 4) {
+        tile_iter(PLAIN, PLAIN, PLAIN, it);
+        tile_iter(PLAIN, PLAIN, PLAIN, it + 1);
+        tile_iter(PLAIN, PLAIN, PLAIN, it + 2);
+        tile_iter(PLAIN, PLAIN, PLAIN, it + 3);
+    }
+#pragma clang loop unroll(disable)
+    for (int it = nplain4; it < nplain; ++it) tile_iter(PLAIN, PLAIN, PLAIN, it);
     if (nplain < nfull) tile_iter(PLAIN, PLAIN, MASKED, nplain);
     // under the causal mask a wave is done once the tiles start past its last query; it keeps
     // feeding the transfers and the barriers the other waves rely on
