@@ -15,10 +15,12 @@
 //   ar_flash_f32_short  [256,1,1]  [ceil(n/32), B*hq, 1]     fp32 exact for few, short heads; head_dim 64
 //   ar_flash_bf16       [256,1,1]  [ceil(n/128), B*hq, 1]    bf16 (cuda_flash_bf16.rs), any mask
 //   ar_flash_bf16_long  [512,1,1]  [ceil(n/256), B*hq, 1]    bf16 pipelined, has_mask must be 0
+//   ar_flash_bf16_mid   [256,1,1]  [ceil(n/128), B*hq, 1]    the same with 4 waves (two workgroups per CU): short / causal
 //   ar_flash_bf16_short [512,1,1]  [ceil(n/128), B*hq, 1]    bf16, n <= 256, has_mask must be 0
 //   ar_flash_sage       [256,1,1]  [ceil(n/128), B*hq, 1]    int8 (cuda_flash_sage.rs), any mask, any
 //                                                            block sizes incl. per-row scales; O f32
 //   ar_flash_sage_long  [512,1,1]  [ceil(n/256), B*hq, 1]    int8 pipelined: has_mask 0, bk = 64 * 2^n
+//   ar_flash_sage_mid   [256,1,1]  [ceil(n/128), B*hq, 1]    the same with 4 waves
 //   ar_flash_sage_fp8_long  the same on E4M3 codes
 // The Sage entries take pre-quantised operands (the quantiser is the pre-pass below, not part of
 // the attention kernel as in the reference):
@@ -34,8 +36,8 @@
 // Key-padding masks: every forward entry `X` of the first table has a twin `X_lens` that takes one more
 // pointer after M, `const int *L` ([B] int32: batch b attends to keys [0, L[b]) only, clamped to [0, N];
 // a batch with L[b] = 0 yields zeros), with the same scalars, grid and block:
-//     ar_flash_f32_lens, ar_flash_bf16_lens, ar_flash_bf16_long_lens          (Q, K, V, O, M, L,  6 ints)
-//     ar_flash_sage_lens, ar_flash_sage_long_lens, ar_flash_sage_fp8_lens,
+//     ar_flash_f32_lens, ar_flash_bf16_lens, ar_flash_bf16_long_lens, ar_flash_bf16_mid_lens   (Q, K, V, O, M, L,  6 ints)
+//     ar_flash_sage_lens, ar_flash_sage_long_lens, ar_flash_sage_mid_lens, ar_flash_sage_fp8_lens,
 //     ar_flash_sage_fp8_long_lens                                             (Q8, K8, V, O, M, L, SQ, SK,  ints as above)
 // (The reference's fused kernels take a dense [n, n] mask only, src/models/flash_attention.rs:389-396; its
 // Tensor API reaches key-padding masks through the general path, src/tensor/mod.rs:2405-2447.)
@@ -337,6 +339,7 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_short(const uint
 }
 
 namespace {
+template <int NW>
 __device__ __forceinline__ void flash_bf16_long_entry(unsigned char *lds, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                                                       uint16_t *O, const float *M, const int *L, int N, int head_dim, int causal,
                                                       int has_mask, int hq, int hkv)
@@ -345,11 +348,11 @@ __device__ __forceinline__ void flash_bf16_long_entry(unsigned char *lds, const 
     AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, 0, hq, hkv, L);
     const int wg = linear_wg();
     if (head_dim == 64) {
-        if (causal) attn_pipe_body<64, true, MODE_BF16, false>(p, lds, wg);
-        else attn_pipe_body<64, false, MODE_BF16, false>(p, lds, wg);
+        if (causal) attn_pipe_body<64, true, MODE_BF16, false, NW>(p, lds, wg);
+        else attn_pipe_body<64, false, MODE_BF16, false, NW>(p, lds, wg);
     } else if (head_dim == 128) {
-        if (causal) attn_pipe_body<128, true, MODE_BF16, false>(p, lds, wg);
-        else attn_pipe_body<128, false, MODE_BF16, false>(p, lds, wg);
+        if (causal) attn_pipe_body<128, true, MODE_BF16, false, NW>(p, lds, wg);
+        else attn_pipe_body<128, false, MODE_BF16, false, NW>(p, lds, wg);
     }
 }
 }  // namespace
@@ -359,7 +362,7 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long(const uint1
                                                                       int causal, int has_mask, int hq, int hkv)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_BF16>()];
-    flash_bf16_long_entry(lds, Q, K, V, O, M, nullptr, N, head_dim, causal, has_mask, hq, hkv);
+    flash_bf16_long_entry<8>(lds, Q, K, V, O, M, nullptr, N, head_dim, causal, has_mask, hq, hkv);
 }
 
 extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long_lens(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
@@ -367,7 +370,24 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long_lens(const 
                                                                            int head_dim, int causal, int has_mask, int hq, int hkv)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_BF16>()];
-    flash_bf16_long_entry(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
+    flash_bf16_long_entry<8>(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
+}
+
+// the 4-wave form of the pipelined kernel: 128 queries per workgroup, two workgroups per compute unit
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_bf16_mid(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                        uint16_t *O, const float *M, int N, int head_dim,
+                                                                        int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_BF16, 4>()];
+    flash_bf16_long_entry<4>(lds, Q, K, V, O, M, nullptr, N, head_dim, causal, has_mask, hq, hkv);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_bf16_mid_lens(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
+                                                                             uint16_t *O, const float *M, const int *L, int N,
+                                                                             int head_dim, int causal, int has_mask, int hq, int hkv)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_BF16, 4>()];
+    flash_bf16_long_entry<4>(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
 }
 
 namespace {
@@ -447,7 +467,7 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_fp8_lens(const u
 }
 
 // ar_flash_sage_long / ar_flash_sage_fp8_long: the pipelined kernel on pre-quantised operands
-template <int QMODE>
+template <int QMODE, int NW = 8>
 __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const void *Q8, const void *K8, const uint16_t *V, void *O,
                                                       const float *M, const int *L, const float *SQ, const float *SK, int N,
                                                       int head_dim, int causal, int has_mask, int hq, int hkv, int bq, int bk,
@@ -464,11 +484,11 @@ __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const 
 #define AR_SAGE_LONG(DD)                                                                  \
     do {                                                                                  \
         if (out_f32) {                                                                    \
-            if (causal) attn_pipe_body<DD, true, QMODE, true>(p, lds, wg);                \
-            else attn_pipe_body<DD, false, QMODE, true>(p, lds, wg);                      \
+            if (causal) attn_pipe_body<DD, true, QMODE, true, NW>(p, lds, wg);            \
+            else attn_pipe_body<DD, false, QMODE, true, NW>(p, lds, wg);                  \
         } else {                                                                          \
-            if (causal) attn_pipe_body<DD, true, QMODE, false>(p, lds, wg);               \
-            else attn_pipe_body<DD, false, QMODE, false>(p, lds, wg);                     \
+            if (causal) attn_pipe_body<DD, true, QMODE, false, NW>(p, lds, wg);           \
+            else attn_pipe_body<DD, false, QMODE, false, NW>(p, lds, wg);                 \
         }                                                                                 \
     } while (0)
     if (head_dim == 64) AR_SAGE_LONG(64);
@@ -492,6 +512,25 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long_lens(const 
 {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8>()];
     flash_sage_long_entry<MODE_I8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+// the 4-wave form: 128 queries per workgroup, two workgroups per compute unit
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_mid(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
+                                                                        void *O, const float *M, const float *SQ, const float *SK,
+                                                                        int N, int head_dim, int causal, int has_mask, int hq,
+                                                                        int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4>()];
+    flash_sage_long_entry<MODE_I8, 4>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_mid_lens(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
+                                                                             void *O, const float *M, const int *L, const float *SQ,
+                                                                             const float *SK, int N, int head_dim, int causal,
+                                                                             int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4>()];
+    flash_sage_long_entry<MODE_I8, 4>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
 extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,

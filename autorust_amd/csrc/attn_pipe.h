@@ -32,6 +32,14 @@
 //                transfers and barriers.
 //
 // 8 waves of 32 queries per workgroup, two waves per SIMD.
+//
+// NW = 4 is the variant for launches whose workgroups see few tiles (short or causal sequences): 128
+// queries per workgroup and at most 80 KB of LDS, so that a compute unit holds two workgroups and one's
+// prologue and epilogue (first transfers, output store, the gap to the next workgroup) run under the
+// other's tiles.  K and V then live in rings of their own, K two tiles deep and V three: while tile t is
+// computed the wave reads K(t+1), V(t) and V(t+1) from LDS (K(t) went into registers during tile t-1),
+// and tile t+2 is on its way.  The rare reference move takes the block's logits from their registers
+// instead of recomputing them from K(t), which this ring no longer holds.
 #pragma once
 
 #include "attn_fwd.h"
@@ -62,11 +70,12 @@ __device__ __forceinline__ void static_for(F &&f)
     }
 }
 
-// LDS bytes attn_pipe_body needs: four stages of [piece][64 rows][64 B] K and V tiles
-template <int D, int MODE>
+// LDS bytes attn_pipe_body needs: [piece][64 rows][64 B] K and V tiles, four stages of both (NW = 8), or a
+// ring of two K tiles and one of three V tiles (NW = 4)
+template <int D, int MODE, int NW = 8>
 constexpr int attn_pipe_lds_bytes()
 {
-    return 4 * 4096 * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64 + D * 2 / 64);
+    return 4096 * ((NW == 8 ? 4 : 2) * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64) + (NW == 8 ? 4 : 3) * (D * 2 / 64));
 }
 
 // workgroup index -> (batch * heads + head, query tile of 256), as in attn_fwd_kernel
@@ -87,11 +96,12 @@ __device__ __forceinline__ void pipe_work_item(const AttnParams &p, int wg, int 
 
 // The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
 // aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below.
-template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS>
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS, int NW = 8>
 __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
-    constexpr int NW = 8;
+    static_assert(NW == 8 || NW == 4, "8 waves (one workgroup per CU) or 4 (two)");
+    constexpr bool RINGS = NW == 4;  // K and V in rings of their own, two and three tiles deep
     constexpr int BQ = NW * 32;
     constexpr int QK_BYTES = (MODE != MODE_BF16) ? 1 : 2;
     constexpr int KP = D * QK_BYTES / 64;  // 64-byte pieces per K row
@@ -100,6 +110,8 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     constexpr int V_TILE = VP * 4096;
     constexpr int STAGE = K_TILE + V_TILE;
     constexpr int NSTAGE = 4;
+    constexpr int AHEAD = RINGS ? 2 : 3;          // a tile is requested this many iterations before the one that computes on it
+    constexpr int LDS_BYTES = attn_pipe_lds_bytes<D, MODE, NW>();
     constexpr int XFERS = (KP + VP) * 4;          // 1 KB transfers per tile
     constexpr int XPW = (XFERS + NW - 1) / NW;    // at most this many per wave
     constexpr int XPW_MIN = XFERS / NW;           // at least this many per wave
@@ -107,7 +119,12 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     constexpr int DB = D / 32;
     static_assert(KP >= 1 && XFERS >= NW, "tile too small for 8 waves");
 
-    static_assert(NSTAGE * STAGE == attn_pipe_lds_bytes<D, MODE>(), "LDS size bookkeeping");
+    static_assert(RINGS ? (2 * K_TILE + 3 * V_TILE == LDS_BYTES) : (NSTAGE * STAGE == LDS_BYTES), "LDS size bookkeeping");
+    // where the K and the V part of tile t live (byte offsets into lds)
+    auto k_base = [](int t) __attribute__((always_inline)) -> int { return RINGS ? (t & 1) * K_TILE : (t & 3) * STAGE; };
+    auto v_base = [](int t) __attribute__((always_inline)) -> int {
+        return RINGS ? 2 * K_TILE + (t % 3) * V_TILE : (t & 3) * STAGE + K_TILE;
+    };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -177,8 +194,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // instruction writing a scalar register (v_readfirstlane of the descriptors, a scalar register
     // reloaded from a spill lane) and a memory instruction reading it: the compiler pads neither
     // for inline assembly, so the assembly carries the wait states itself (s_mov + s_nop 3).
-    auto issue_tile = [&](int tile, int stage) __attribute__((always_inline)) {
-        const uint32_t dst = (uint32_t)(uintptr_t)(lds_ptr_t)lds + stage * STAGE;
+    auto issue_tile = [&](int tile) __attribute__((always_inline)) {
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+        const uint32_t dst_k = lds0 + k_base(tile), dst_v = lds0 + v_base(tile);
 #pragma unroll
         for (int j = 0; j < XPW; ++j) {
             const int x = wave + NW * j;
@@ -190,7 +208,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
                 const i32x4 rsrc = is_k ? k_rsrc : v_rsrc;
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                              :
-                             : "s"(dst + x * 1024), "v"(off), "s"(rsrc)
+                             : "s"(is_k ? dst_k + x * 1024 : dst_v + (x - KP * 4) * 1024), "v"(off), "s"(rsrc)
                              : "memory", "m0");
             }
         }
@@ -209,8 +227,8 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // block, i.e. chunk 2 ((lane / 16) % 2) + (lane % 4) / 2, byte 8 (lane % 2) inside it
     const int v_r0 = 4 * h + ((lane & 15) >> 2);
     const int v_c = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
-    const int v_addr[2] = {K_TILE + v_r0 * 64 + (v_c ^ h) * 16 + (lane & 1) * 8,
-                           K_TILE + (v_r0 + 8) * 64 + (v_c ^ (h + 2)) * 16 + (lane & 1) * 8};
+    const int v_addr[2] = {v_r0 * 64 + (v_c ^ h) * 16 + (lane & 1) * 8,
+                           (v_r0 + 8) * 64 + (v_c ^ (h + 2)) * 16 + (lane & 1) * 8};
 
     typedef typename std::conditional<MODE == MODE_I8, i32x16, f32x16>::type acc_t;
     f32x16 oacc[DB];
@@ -374,20 +392,30 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // not finite (the first block, or a jump of the maximum), moves the reference and redoes the
     // block.  Rare, so the raw logits are not kept for it: they are recomputed from the K block,
     // which is still in LDS (block blk of stage st).
-    auto fix_reference = [&](auto masked, const unsigned char *st, int blk, float c, int rel, uint4 (&pb)[2], float &rs)
-                             __attribute__((always_inline)) {
+    // (RINGS: K of the block is gone from LDS by now; its logits are still in their registers, s_blk, as
+    // the matrix instructions left them, i.e. with the bias in the int8 case.)
+    auto fix_reference = [&](auto masked, const unsigned char *st, int blk, const acc_t &s_blk, float c, int rel, uint4 (&pb)[2],
+                             float &rs) __attribute__((always_inline)) {
         constexpr bool M = decltype(masked)::value;
         acc_t s;
+        if constexpr (RINGS) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0;
-        uint4 kt[KSTEPS];
+            for (int r = 0; r < 16; ++r) {
+                if constexpr (BIAS) s[r] = s_blk[r] - 0x4B400000;  // integer subtraction: exactly the sum
+                else s[r] = s_blk[r];
+            }
+        } else {
 #pragma unroll
-        for (int q = 0; q < KSTEPS; ++q) kt[q] = *(const uint4 *)(st + k_addr[q & 1] + (q >> 1) * 4096 + blk * 2048);
-        static_for<0, KSTEPS>([&](auto qi) __attribute__((always_inline)) {
-            constexpr int q = decltype(qi)::value;
-            constexpr int pv = q > 0 ? q - 1 : 0;
-            qk_step(qi, s, kt[pv], kt[q], qreg[pv], qreg[q]);
-        });
+            for (int r = 0; r < 16; ++r) s[r] = 0;
+            uint4 kt[KSTEPS];
+#pragma unroll
+            for (int q = 0; q < KSTEPS; ++q) kt[q] = *(const uint4 *)(st + k_addr[q & 1] + (q >> 1) * 4096 + blk * 2048);
+            static_for<0, KSTEPS>([&](auto qi) __attribute__((always_inline)) {
+                constexpr int q = decltype(qi)::value;
+                constexpr int pv = q > 0 ? q - 1 : 0;
+                qk_step(qi, s, kt[pv], kt[q], qreg[pv], qreg[q]);
+            });
+        }
         // max3 is inline assembly, which the compiler leaves out when it pads the distance between a
         // matrix instruction and the first vector read of its result: the scaled copies below are
         // ordinary vector instructions, so the result has landed by the time max3 runs
@@ -480,7 +508,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     constexpr int R2_SLOTS = DB * 2 - 2;  // S is not ready under the first two O^T MFMAs
     constexpr int SM_SPLIT = (MODE != MODE_BF16) ? (SM_OPS * R2_SLOTS) / (R2_SLOTS + KSTEPS) : SM_HALF;
     // mc / mn: block j / block j+1 has masked keys (causal diagonal, key-length edge); rel_cur /
-    // rel_next are their mask offsets (see lim4h).
+    // rel_next are their mask offsets (see lim4h).  sc and sk point at K tiles, sv at a V tile.
     auto pipe_block = [&](auto mc, auto mn, acc_t &s_old, acc_t &s_new, uint4 (&p_cur)[2], uint4 (&p_nxt)[2],
                           const unsigned char *sc, int cb,
                           const unsigned char *sv, int vb, const unsigned char *sk, int kb, float c_cur, float c_next,
@@ -507,7 +535,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             ARHIP_FENCE();
         });
         rs = sm_half[0] + sm_half[1];
-        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(mc, sc, cb, c_cur, rel_cur, p_cur, rs);
+        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(mc, sc, cb, s_old, c_cur, rel_cur, p_cur, rs);
         l_run += rs;
         set_bias(c_next);  // the reference is final for block j+1 from here to the end of its softmax
         ARHIP_FENCE();
@@ -540,9 +568,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // causal diagonal, or the last partial one) run the same pipeline with the mask applied inside
     // the softmax.  Every wave runs every tile, so all waves execute the same code between barriers.
     const int nfull = CAUSAL ? min(kend / BK, qblk / BK) : kend / BK;
-    issue_tile(0, 0);
-    issue_tile(1, 1);
-    issue_tile(2, 2);
+    static_for<0, AHEAD>([&](auto ti) __attribute__((always_inline)) { issue_tile(decltype(ti)::value); });
     // Q operand, resident in registers.  Everything in flight is awaited here once, Q included, so
     // that no wait for a global load is left inside the loops.
     {
@@ -594,10 +620,10 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     constexpr std::false_type PLAIN{};
     constexpr std::true_type MASKED{};
     if (ntiles > 0) {
-        load_kf(lds, 0);
+        load_kf(lds + k_base(0), 0);
         s_a = mfma_qk();
-        load_kf(lds, 1);
-        load_vf(lds, 0);
+        load_kf(lds + k_base(0), 1);
+        load_vf(lds + v_base(0), 0);
         const float c0 = tile_c(0, 0);
         set_bias(c0);
         if (nfull > 0)
@@ -609,26 +635,30 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // one tile: its two blocks; m0 / m1 / m2 say whether the first block, the second block and the
     // first block of the next tile have masked keys
     auto tile_iter = [&](auto m0, auto m1, auto m2, int it) __attribute__((always_inline)) {
-        const unsigned char *st_cur = lds + (it & 3) * STAGE;
-        const unsigned char *st_nxt = lds + ((it + 1) & 3) * STAGE;
-        // tile it + 3 goes to the stage tile it - 1 vacated at the last barrier
-        issue_tile(it + 3, (it + 3) & 3);
+        const unsigned char *k_cur = lds + k_base(it), *k_nxt = lds + k_base(it + 1);
+        const unsigned char *v_cur = lds + v_base(it), *v_nxt = lds + v_base(it + 1);
+        // tile it + 3 goes to the stage tile it - 1 vacated at the last barrier (RINGS: K(it + 2) to where
+        // K(it) was, read for the last time before that barrier, V(it + 2) to where V(it - 1) was)
+        issue_tile(it + AHEAD);
         advance_sk_group(it);
         // (tile_iter runs on consecutive tiles from 0 on: this tile's factor is last iteration's c_nxt)
         const float c_cur = c_carry, c_nxt = tile_c(it + 1, it);
         c_carry = c_nxt;
         const int rel0 = lim4h - it * BK;
-        pipe_block(m0, m1, s_a, s_b, p_a, p_b, st_cur, 0, st_cur, 1, st_nxt, 0, c_cur, c_cur, rel0, rel0 - 32);
-        pipe_block(m1, m2, s_b, s_a, p_b, p_a, st_cur, 1, st_nxt, 0, st_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64);
-        wait_vmem_le<XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
+        pipe_block(m0, m1, s_a, s_b, p_a, p_b, k_cur, 0, v_cur, 1, k_nxt, 0, c_cur, c_cur, rel0, rel0 - 32);
+        pipe_block(m1, m2, s_b, s_a, p_b, p_a, k_cur, 1, v_nxt, 0, k_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64);
+        wait_vmem_le<RINGS ? 0 : XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
         __syncthreads();
     };
+    // RINGS: the first iteration requests K(2) into the place of K(0), which the lines above have just
+    // read: every wave's reads must have returned first
+    if constexpr (RINGS) __syncthreads();
     // the last unmasked tile hands a masked block to the look-ahead: it is peeled off
     const int nplain = (nfull < ntiles) ? max(nfull - 1, 0) : nfull;
     // 8-bit operands: four tiles per trip, so that the stage of a tile (it % 4) and with it every LDS
     // offset and transfer destination is a constant (15 vector and 23 scalar instructions fewer per
     // tile: Sage B4 H32 S8192 3.05 -> 2.96 ms).  The bf16 loop body is larger and gains nothing from it.
-    const int nplain4 = (MODE != MODE_BF16) ? (nplain & ~3) : 0;
+    const int nplain4 = (MODE != MODE_BF16 && !RINGS) ? (nplain & ~3) : 0;
 #pragma clang loop unroll(disable)
     for (int it = 0; it < nplain4; it += 4) {
         tile_iter(PLAIN, PLAIN, PLAIN, it);
@@ -647,8 +677,8 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     for (int it = nfull; it < my_tiles; ++it) tile_iter(MASKED, MASKED, MASKED, it);
 #pragma clang loop unroll(disable)
     for (int it = max(nfull, my_tiles); it < ntiles; ++it) {
-        issue_tile(it + 3, (it + 3) & 3);
-        wait_vmem_le<XPW_MIN>();
+        issue_tile(it + AHEAD);
+        wait_vmem_le<RINGS ? 0 : XPW_MIN>();
         __syncthreads();
     }
 
@@ -678,7 +708,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         // are free once every wave is past the last tile and the transfers requested beyond it have
         // landed) and leaves as whole rows, 16 bytes per lane, 4 rows per instruction.
         constexpr int OROW = D * 2 + 16;  // bytes; 16-byte aligned rows
-        static_assert(NW * 32 * OROW <= NSTAGE * STAGE, "output staging fits the tile stages");
+        static_assert(NW * 32 * OROW <= LDS_BYTES, "output staging fits the tile stages");
         wait_vmem_le<0>();
         __syncthreads();
         unsigned char *ob = lds + wave * 32 * OROW;
@@ -706,17 +736,17 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
 }
 
 // int8 uses the biased accumulators (see s_init); bf16 and FP8 the plain ones.
-template <int D, bool CAUSAL, int MODE, bool OUT_F32>
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8>
 __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
-    attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS)>(p, lds, wg_linear);
+    attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS), NW>(p, lds, wg_linear);
 }
 
-template <int D, bool CAUSAL, int MODE, bool OUT_F32>
-__global__ void __launch_bounds__(512) attn_pipe_kernel(const AttnParams p)
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8>
+__global__ void __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) attn_pipe_kernel(const AttnParams p)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<D, MODE>()];
-    attn_pipe_body<D, CAUSAL, MODE, OUT_F32>(p, lds, (int)blockIdx.x);
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<D, MODE, NW>()];
+    attn_pipe_body<D, CAUSAL, MODE, OUT_F32, NW>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

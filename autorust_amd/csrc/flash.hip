@@ -64,13 +64,25 @@ static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bo
         hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
 }
 
-// The software-pipelined long-sequence kernel (8 waves, no additive mask, tile-uniform K scales).
-template <int D, int MODE, bool OUT_F32>
+// The software-pipelined kernel (no additive mask, tile-uniform K scales): 8 waves per workgroup, or 4
+// (two workgroups per compute unit) where a workgroup sees few tiles.
+template <int D, int MODE, bool OUT_F32, int NW = 8>
 static void launch_pipe(hipStream_t stream, const AttnParams &p, bool causal)
 {
-    const dim3 grid((unsigned)p.total), block(512);
-    if (causal) hipLaunchKernelGGL((attn_pipe_kernel<D, true, MODE, OUT_F32>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((attn_pipe_kernel<D, false, MODE, OUT_F32>), grid, block, 0, stream, p);
+    const dim3 grid((unsigned)p.total), block(NW * 64);
+    if (causal) hipLaunchKernelGGL((attn_pipe_kernel<D, true, MODE, OUT_F32, NW>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_pipe_kernel<D, false, MODE, OUT_F32, NW>), grid, block, 0, stream, p);
+}
+
+// Which of the two: 128 queries per workgroup hide a workgroup's prologue and epilogue under its
+// neighbour's tiles and fill the chip with fewer heads, but request every K/V tile twice as often and
+// keep only one tile in flight.  Measured at D = 128 (B4 H32): causal N = 512 / 1024 / 2048 -15 / -7 / -5 %,
+// B1 H16 N = 2048 causal -25 %, B2 H16 N = 1024 -22 %; non-causal N = 2048 equal, N = 8192 +3 %, causal
+// N = 32768 +4.5 %.
+static bool pipe_wants_4_waves(arhip_device *dev, int64_t heads, int64_t N)
+{
+    if (dev->attn_waves == 8 || dev->attn_waves == 40) return dev->attn_waves == 40;
+    return N <= 2048 || heads * ((N + 255) / 256) < 2 * (int64_t)dev->cus;
 }
 
 // The pipelined kernel addresses K and V through 32-bit buffer offsets (rows of one head, plus the
@@ -96,8 +108,10 @@ static int pick_waves(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bo
     else if (D == 64 && wg128 < 2 * cus && (special || N < 512)) nw = 1;
     else nw = 4;
     // ARHIP_ATTN_WAVES (read once when the device is opened) is a tuning aid; results do not depend on it
+    // (1, 4: the general kernel with that many waves; 8, 40: the pipelined kernel with 8 / 4 waves)
     const int w = dev->attn_waves;
     if ((w == 1 || w == 4 || w == 8) && !special && (w != 1 || D == 64)) nw = w;
+    if (w == 40 && !special) nw = 8;
     return nw;
 }
 
@@ -207,6 +221,8 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
     const bool c = causal != 0, hm = mask != nullptr;
     int nw = pick_waves(dev, B * Hq, N, D, hm);
     if (nw == 8 && !pipe_addressable(N, kv_strides[2], 2)) nw = 4;
+    const bool pipe = nw == 8;  // the software-pipelined kernel; how many waves it runs with is its own choice
+    if (pipe && pipe_wants_4_waves(dev, B * Hq, N)) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;  // few workgroups per CU: balance them globally
@@ -225,12 +241,14 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
             else hipLaunchKernelGGL((attn_fwd_kernel<128, 8, false, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
         }
     } else if (D == 64) {
-        if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
-        else if (nw == 4) launch_attn<64, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
-        else launch_pipe<64, MODE_BF16, false>(dev->stream, p, c);
+        if (pipe && nw == 4) launch_pipe<64, MODE_BF16, false, 4>(dev->stream, p, c);
+        else if (pipe) launch_pipe<64, MODE_BF16, false>(dev->stream, p, c);
+        else if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
+        else launch_attn<64, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
     } else {
-        if (nw == 4) launch_attn<128, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
-        else launch_pipe<128, MODE_BF16, false>(dev->stream, p, c);
+        if (pipe && nw == 4) launch_pipe<128, MODE_BF16, false, 4>(dev->stream, p, c);
+        else if (pipe) launch_pipe<128, MODE_BF16, false>(dev->stream, p, c);
+        else launch_attn<128, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
     }
     arhip_note_selected(ARHIP_K_FLASH_BF16);
     return t.end();
@@ -299,6 +317,9 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
     int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg);
     if (nw == 1) nw = 4;
     if (nw == 8 && !pipe_addressable(N, std::max<int64_t>(D, v_strides ? v_strides[2] : D), 2)) nw = 4;
+    const bool pipe = nw == 8 && !per_key && !dbg;
+    const bool pipe4 = pipe && !fp8 && pipe_wants_4_waves(dev, B * Hq, N);  // (the FP8 variant keeps to 8 waves)
+    if (pipe4) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;
@@ -323,6 +344,8 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
             if (per_key) SAGE_V(DD, 4, true, true, false);                                             \
             else SAGE_V(DD, 4, false, true, false);                                                    \
         } else if (per_key) SAGE_V(DD, 4, true, false, true);                                          \
+        else if (pipe4 && f32o) launch_pipe<DD, MODE_I8, true, 4>(dev->stream, p, c);                  \
+        else if (pipe4) launch_pipe<DD, MODE_I8, false, 4>(dev->stream, p, c);                         \
         else if (nw == 4) SAGE_V(DD, 4, false, false, true);                                           \
         else if (f32o) launch_pipe<DD, MODE_I8, true>(dev->stream, p, c);                              \
         else launch_pipe<DD, MODE_I8, false>(dev->stream, p, c);                                       \

@@ -392,6 +392,13 @@ bool long_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int6
     return (wgs >= 2 * cus || (n >= 512 && 2 * wgs >= cus)) && (n + 320) * d * 2 < ((int64_t)1 << 31);
 }
 
+// ... and run with 4 waves / 128 queries per workgroup (the `_mid` entry points, two workgroups per compute
+// unit) where a workgroup sees few tiles: the rule of arhip_flash_fwd / arhip_sage_fwd
+bool mid_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int64_t n)
+{
+    return n <= 2048 || b * h * ((n + 255) / 256) < 2 * (int64_t)dev->compute_units();
+}
+
 }  // namespace
 
 // The fp32 kernels: 128 queries (keys) per workgroup when that still fills the chip, else 32
@@ -436,6 +443,9 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
         if (!has_mask && !key_lengths && n <= 256 && b * h * ((n + 127) / 128) <= 4 * (int64_t)dev->compute_units())
             calls.push_back(make_call(dev, "ar_flash_bf16_short", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 127) / 128, b * h, 1}, {512, 1, 1}, vals));
+        else if (!has_mask && long_variant(dev, b, h, n, d) && mid_variant(dev, b, h, n))
+            calls.push_back(attn_call("ar_flash_bf16_mid", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
+                                      {(n + 127) / 128, b * h, 1}, {256, 1, 1}, vals));
         else if (!has_mask && long_variant(dev, b, h, n, d))
             calls.push_back(attn_call("ar_flash_bf16_long", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 255) / 256, b * h, 1}, {512, 1, 1}, vals));
@@ -493,8 +503,12 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     const bool tile_uniform = ((int64_t)64 << shift) == bk;
     if (!has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
         svals.push_back(bf16_in ? 0 : 1);  // out_f32
-        calls.push_back(attn_call(st.sage_fp8 ? "ar_flash_sage_fp8_long" : "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
-                                  {(n + 255) / 256, b * h, 1}, {512, 1, 1}, svals));
+        if (!st.sage_fp8 && mid_variant(dev, b, h, n))
+            calls.push_back(attn_call("ar_flash_sage_mid", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
+                                      {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
+        else
+            calls.push_back(attn_call(st.sage_fp8 ? "ar_flash_sage_fp8_long" : "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk},
+                                      {I8, I8, BF, X, F, F, F}, {(n + 255) / 256, b * h, 1}, {512, 1, 1}, svals));
     } else if (!bf16_in) {
         calls.push_back(attn_call(general, {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, F, F, F, F},
                                   {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));

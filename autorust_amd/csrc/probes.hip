@@ -138,10 +138,13 @@ extern "C" __global__ void probe_clock_sampler(long long *ticks, int samples, in
 
 // What the vector ALU can still issue beside the matrix pipe: every wave runs `iters` times
 // { 1 matrix instruction (bf16 32x32x16 or int8 32x32x32, four accumulators in turn); K independent
-// vector instructions (v_fma_f32 or v_exp_f32) }, two waves per SIMD like the attention kernels, and
-// every wave records the real-time (100 MHz) ticks of its loop.  With K = 0 the loop runs at the
-// matrix rate; the growth with K is what the softmax instructions between the matrix instructions
-// of an attention block cost.  One kernel per (matrix type, vector instruction, K).
+// vector instructions (v_fma_f32 or v_exp_f32) } and records the shader-clock ticks (s_memtime) and
+// the real-time (100 MHz) ticks of its loop: ticks[2 w] and ticks[2 w + 1] for wave w of the grid.
+// The workgroup size sets the waves per SIMD (256 threads: one, 512: two like the attention kernels,
+// 768: three).  With K = 0 the loop runs at the matrix rate; the growth with K is what the softmax
+// instructions between the matrix instructions of an attention block cost, and the shader-clock
+// figures separate an issue limit from a clock (power) limit.  One kernel per (matrix type, vector
+// instruction, K).
 template <int K, bool EXP, bool I8>
 __device__ __forceinline__ void probe_issue_mix_body(const uint4 *src, float *out, long long *ticks, int iters)
 {
@@ -159,7 +162,7 @@ __device__ __forceinline__ void probe_issue_mix_body(const uint4 *src, float *ou
             o[n][r] = 0.f;
             oi[n][r] = 0;
         }
-    const long long r0 = __builtin_amdgcn_s_memrealtime();
+    const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -176,16 +179,20 @@ __device__ __forceinline__ void probe_issue_mix_body(const uint4 *src, float *ou
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    const long long r1 = __builtin_amdgcn_s_memrealtime();
+    const long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
     float r = 0.f;
     for (int i = 0; i < 8; ++i) r += d[i];
     for (int n = 0; n < 4; ++n)
         for (int i = 0; i < 16; ++i) r += o[n][i] + (float)oi[n][i];
     out[blockIdx.x * blockDim.x + threadIdx.x] = r;
-    if ((threadIdx.x & 63) == 0) ticks[blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64] = r1 - r0;
+    if ((threadIdx.x & 63) == 0) {
+        const int w = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
+        ticks[2 * w] = c1 - c0;
+        ticks[2 * w + 1] = r1 - r0;
+    }
 }
 #define PROBE_ISSUE_MIX(NAME, K, EXP, I8)                                                                              \
-    extern "C" __global__ void __launch_bounds__(512) NAME(const uint4 *src, float *out, long long *ticks, int iters)  \
+    extern "C" __global__ void __launch_bounds__(768) NAME(const uint4 *src, float *out, long long *ticks, int iters)  \
     {                                                                                                                  \
         probe_issue_mix_body<K, EXP, I8>(src, out, ticks, iters);                                                      \
     }
@@ -196,7 +203,8 @@ __device__ __forceinline__ void probe_issue_mix_body(const uint4 *src, float *ou
     PROBE_ISSUE_MIX(PREFIX##_k6, 6, EXP, I8)    \
     PROBE_ISSUE_MIX(PREFIX##_k8, 8, EXP, I8)    \
     PROBE_ISSUE_MIX(PREFIX##_k10, 10, EXP, I8)  \
-    PROBE_ISSUE_MIX(PREFIX##_k14, 14, EXP, I8)
+    PROBE_ISSUE_MIX(PREFIX##_k14, 14, EXP, I8)  \
+    PROBE_ISSUE_MIX(PREFIX##_k18, 18, EXP, I8)
 PROBE_ISSUE_MIX_KS(probe_mix_bf16_fma, false, false)
 PROBE_ISSUE_MIX_KS(probe_mix_bf16_exp, true, false)
 PROBE_ISSUE_MIX_KS(probe_mix_i8_fma, false, true)

@@ -287,27 +287,31 @@ def sustained_mfma(dev):
 
 
 def issue_mix(dev):
-    """Time per matrix instruction of a loop of { 1 MFMA ; K vector instructions } for K = 0..14
-    (probe_mix_* in csrc/probes.hip), two waves per SIMD, operands with random mantissas: how much
-    vector work fits beside the matrix pipe before the loop slows down."""
+    """Cost per matrix instruction of a loop of { 1 MFMA ; K vector instructions } for K = 0..18
+    (probe_mix_* in csrc/probes.hip) with one, two (the attention kernels) and three waves per SIMD,
+    operands with random mantissas: how much vector work fits beside the matrix pipe before the loop
+    slows down.  Every entry is [shader-clock cycles, nanoseconds, shader clock in MHz] per matrix
+    instruction per SIMD: the cycles tell an issue limit from a clock (power) limit."""
     mod = _probes(dev)
     rng = np.random.default_rng(5)
     bits = (rng.integers(0, 1 << 16, 8192 * 8, dtype=np.uint32) & 0x007F) | 0x3C00     # bf16 values in [0.0078, 0.0156)
     src = dev.from_numpy(bits.astype(np.uint16))
-    out, ticks = dev.alloc(256 * 512 * 4), dev.alloc(256 * 8 * 8)
+    out, ticks = dev.alloc(256 * 768 * 4), dev.alloc(256 * 12 * 16)
     iters = 2000
     res = {}
-    for mat in ("bf16", "i8"):
-        for op in ("fma", "exp"):
-            row = {}
-            for k in (0, 2, 4, 6, 8, 10, 14):
-                name = "probe_mix_%s_%s_k%d" % (mat, op, k)
-                dev.launch(mod, name, (256, 1, 1), (512, 1, 1), [src, out, ticks], [iters])
-                dev.launch(mod, name, (256, 1, 1), (512, 1, 1), [src, out, ticks], [iters])
-                t = ticks.copyout(np.int64, (256 * 8,)).astype(np.float64)
-                # real-time ticks are 10 ns; 4 matrix instructions per iteration; two waves share a SIMD
-                row["K=%d" % k] = round(float(t.mean()) * 10.0 / (iters * 4) / 2.0, 2)
-            res["%s_mfma+%s" % (mat, op)] = row
+    for waves in (2, 1, 3):
+        for mat in ("bf16", "i8"):
+            for op in ("fma", "exp"):
+                row = {}
+                for k in (0, 2, 4, 6, 8, 10, 14, 18):
+                    name = "probe_mix_%s_%s_k%d" % (mat, op, k)
+                    for _ in range(2):
+                        dev.launch(mod, name, (256, 1, 1), (256 * waves, 1, 1), [src, out, ticks], [iters])
+                    t = ticks.copyout(np.int64, (256 * 4 * waves, 2)).astype(np.float64).mean(axis=0)
+                    # 4 matrix instructions per iteration; `waves` waves share a SIMD; real-time ticks are 10 ns
+                    cyc, ns = t[0] / (iters * 4) / waves, t[1] * 10.0 / (iters * 4) / waves
+                    row["K=%d" % k] = [round(float(cyc), 1), round(float(ns), 2), round(float(t[0] / t[1] * 100.0))]
+                res["%s_mfma+%s_%dwaves" % (mat, op, waves)] = row
     src.free()
     out.free()
     ticks.free()
@@ -415,9 +419,10 @@ def main():
 
     if args.issue_probe:
         dev = Device(0)
-        print(json.dumps({"issue_mix_ns_per_mfma_per_simd": issue_mix(dev),
-                          "note": "loop of {1 MFMA (32x32x16 bf16 or 32x32x32 int8); K v_fma_f32 or v_exp_f32}, "
-                                  "two waves per SIMD, 256 workgroups of 512 threads"}))
+        print(json.dumps({"issue_mix_per_mfma_per_simd": issue_mix(dev),
+                          "note": "loop of {1 MFMA (32x32x16 bf16 or 32x32x32 int8); K v_fma_f32 or v_exp_f32}; entries are "
+                                  "[shader-clock cycles, ns, MHz] per matrix instruction per SIMD; 256 workgroups of "
+                                  "256 / 512 / 768 threads = 1 / 2 / 3 waves per SIMD"}))
         dev.close()
         return
     dev = Device(0)

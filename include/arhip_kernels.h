@@ -21,9 +21,10 @@
 #ifndef ARHIP_KERNELS_H
 #define ARHIP_KERNELS_H
 
-/* queries per workgroup and workgroup size of the two tilings */
+/* queries per workgroup and workgroup size of the tilings */
 #define ARHIP_KQ_GENERAL 128 /* block [256,1,1] */
 #define ARHIP_KQ_LONG 256    /* block [512,1,1] */
+#define ARHIP_KQ_MID 128     /* block [256,1,1]: the pipelined kernel with 4 waves, two workgroups per compute unit */
 
 /* fp32 exact mode: replaces `ar_flash_f32`, src/runtime/cuda_flash.rs:53-141.
  * (const float *Q, *K, *V, float *O, const float *M, 6 ints); general tiling. */
@@ -57,6 +58,10 @@
 /* the software-pipelined variant for long sequences: same arguments, has_mask must be 0,
  * (N + 320) * head_dim * 2 < 2^31; long tiling. */
 #define ARHIP_KERNEL_FLASH_BF16_LONG "ar_flash_bf16_long"
+/* the same kernel with 4 waves and 128 queries per workgroup (mid tiling), for launches whose workgroups
+ * see few tiles (n <= 2048, or fewer than two 256-query workgroups per compute unit): same arguments and
+ * limits as ar_flash_bf16_long. */
+#define ARHIP_KERNEL_FLASH_BF16_MID "ar_flash_bf16_mid"
 /* the variant for sequences of at most 256 keys (all of K/V of a head in LDS at once): same
  * arguments, has_mask must be 0, N <= 256; block [512,1,1], grid [ceil(N/128), B*hq, 1]. */
 #define ARHIP_KERNEL_FLASH_BF16_SHORT "ar_flash_bf16_short"
@@ -70,6 +75,8 @@
 /* pipelined variant: has_mask 0, bk = 64 * 2^n; one more int `out_f32` (O is f32 when set,
  * bf16 otherwise); long tiling. */
 #define ARHIP_KERNEL_FLASH_SAGE_LONG "ar_flash_sage_long"
+/* its 4-wave form (mid tiling), chosen like ar_flash_bf16_mid: same arguments as ar_flash_sage_long. */
+#define ARHIP_KERNEL_FLASH_SAGE_MID "ar_flash_sage_mid"
 
 /* Sage pre-pass (src/runtime/cuda_flash_sage.rs:124-137, 201-223 hoisted out of the attention
  * kernel; K smoothing is an extension).  x is [B*H, N, D]; block [256,1,1] unless noted.
@@ -101,14 +108,16 @@
  * arguments of the entry it is named after with one more pointer directly after M:
  *     const int *L   [B] int32; batch b attends to keys [0, L[b]) only (clamped to [0, N]; 0 => zeros)
  * and the same scalars, grid and block.
- *   ar_flash_f32_lens, ar_flash_bf16_lens, ar_flash_bf16_long_lens      (Q, K, V, O, M, L, 6 ints)
+ *   ar_flash_f32_lens, ar_flash_bf16_lens, ar_flash_bf16_long_lens, ar_flash_bf16_mid_lens   (Q, K, V, O, M, L, 6 ints)
  *   ar_flash_sage_lens, ar_flash_sage_fp8_lens                           (Q8, K8, V, O, M, L, SQ, SK, 6 ints, bq, bk)
- *   ar_flash_sage_long_lens, ar_flash_sage_fp8_long_lens                 (..., bq, bk, out_f32) */
+ *   ar_flash_sage_long_lens, ar_flash_sage_mid_lens, ar_flash_sage_fp8_long_lens   (..., bq, bk, out_f32) */
 #define ARHIP_KERNEL_FLASH_F32_LENS "ar_flash_f32_lens"
 #define ARHIP_KERNEL_FLASH_BF16_LENS "ar_flash_bf16_lens"
 #define ARHIP_KERNEL_FLASH_BF16_LONG_LENS "ar_flash_bf16_long_lens"
+#define ARHIP_KERNEL_FLASH_BF16_MID_LENS "ar_flash_bf16_mid_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_LENS "ar_flash_sage_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_LONG_LENS "ar_flash_sage_long_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_MID_LENS "ar_flash_sage_mid_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_FP8_LENS "ar_flash_sage_fp8_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_FP8_LONG_LENS "ar_flash_sage_fp8_long_lens"
 

@@ -13,8 +13,10 @@
 //! | `ar_flash_f32_short` | 256   | `[ceil(n/32), b*h, 1]`  | same; few, short heads; `head_dim` 64        |
 //! | `ar_flash_bf16`      | 256   | `[ceil(n/128), b*h, 1]` | same                                         |
 //! | `ar_flash_bf16_long` | 512   | `[ceil(n/256), b*h, 1]` | same (`has_mask` must be 0)                  |
+//! | `ar_flash_bf16_mid`  | 256   | `[ceil(n/128), b*h, 1]` | same; the pipelined kernel with 4 waves      |
 //! | `ar_flash_sage`      | 256   | `[ceil(n/128), b*h, 1]` | same `+ bq, bk`; buffers `+ SQ, SK`; O is f32|
 //! | `ar_flash_sage_long` | 512   | `[ceil(n/256), b*h, 1]` | same `+ bq, bk, out_f32`                     |
+//! | `ar_flash_sage_mid`  | 256   | `[ceil(n/128), b*h, 1]` | same; the pipelined kernel with 4 waves      |
 //! | `ar_flash_sage_fp8`, `ar_flash_sage_fp8_long` | as the int8 pair, on E4M3 codes (`SageOptions::fp8`)        |
 //! | `<entry>_lens`       | as `<entry>` | as `<entry>`     | one more buffer after the mask slot: `L`, int32 `[b]` key lengths |
 //!
@@ -153,6 +155,12 @@ fn long_variant(dev: &str, b: i64, h: i64, n: i64, d: i64) -> bool {
     (wgs >= 2 * cus || (n >= 512 && 2 * wgs >= cus)) && (n + 320) * d * 2 < 1 << 31
 }
 
+/// ... and run with 4 waves / 128 queries per workgroup (`_mid`: two workgroups per compute unit, one's
+/// prologue and epilogue under the other's tiles) where a workgroup sees few tiles.
+fn mid_variant(dev: &str, b: i64, h: i64, n: i64) -> bool {
+    n <= 2048 || b * h * ((n + 255) / 256) < 2 * crate::runtime::ops_hip::compute_units(dev)
+}
+
 /// The fp32 kernels take 128 queries (keys) per workgroup when that still fills the chip, else 32
 /// with the tiles of the other side dealt out between the waves (`*_short`, `head_dim` 64).
 fn short_f32(dev: &str, b: i64, heads: i64, n: i64, d: i64) -> bool {
@@ -177,6 +185,8 @@ pub fn host_call_bf16(dev: &str, bufs: Vec<Buffer>, lens: Option<Buffer>, b: i64
     if !opts.has_mask && lens.is_none() && n <= 256 && b * h * ((n + 127) / 128) <= 4 * crate::runtime::ops_hip::compute_units(dev) {
         // all of K/V of a head in LDS at once: the ViT sequence lengths
         call("ar_flash_bf16_short", bufs, &[bf, bf, bf, bf, f], [(n + 127) / 128, b * h, 1], [512, 1, 1], vals(n, d, h, opts), &[])
+    } else if !opts.has_mask && long_variant(dev, b, h, n, d) && mid_variant(dev, b, h, n) {
+        attn_call("ar_flash_bf16_mid", bufs, &[bf, bf, bf, bf, f], lens, [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts))
     } else if !opts.has_mask && long_variant(dev, b, h, n, d) {
         attn_call("ar_flash_bf16_long", bufs, &[bf, bf, bf, bf, f], lens, [(n + 255) / 256, b * h, 1], [512, 1, 1], vals(n, d, h, opts))
     } else {
@@ -268,8 +278,13 @@ pub fn host_calls_sage(
     let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
     if !opts.has_mask && tile_uniform && long_variant(dev, b, h, n, d) {
         sv.push(!bf16_in as i64); // out_f32
-        calls.push(attn_call(long, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
-                             [(n + 255) / 256, b * h, 1], [512, 1, 1], sv));
+        if !sage.fp8 && mid_variant(dev, b, h, n) {
+            calls.push(attn_call("ar_flash_sage_mid", vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
+                                 [(n + 127) / 128, b * h, 1], [256, 1, 1], sv));
+        } else {
+            calls.push(attn_call(long, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
+                                 [(n + 255) / 256, b * h, 1], [512, 1, 1], sv));
+        }
     } else if !bf16_in {
         calls.push(attn_call(general, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f], lens,
                              [(n + 127) / 128, b * h, 1], [256, 1, 1], sv));

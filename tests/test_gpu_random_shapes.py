@@ -1,6 +1,7 @@
 """Seeded random sweep over shapes, head groupings, masks and tiling variants: every case is
 compared with the float64 oracle.  The tiling variant does not change the function, so the
-same case is also run with the workgroup size forced (1, 4 and 8 waves): ARHIP_ATTN_WAVES is read
+same case is also run with the tiling forced (the general kernel with 1 and 4 waves, the pipelined one with
+8 and, "40", 4 waves): ARHIP_ATTN_WAVES is read
 when a device is opened, so those runs open a device handle of their own."""
 import contextlib
 
@@ -46,7 +47,7 @@ def _cases(seed, count):
     return out
 
 
-@pytest.mark.parametrize("waves", [None, "1", "4", "8"])
+@pytest.mark.parametrize("waves", [None, "1", "4", "8", "40"])
 def test_flash_random_shapes(dev, waves, monkeypatch):
     with _device_with_waves(dev, waves, monkeypatch) as d:
         _flash_random_shapes(d)
@@ -69,7 +70,7 @@ def _flash_random_shapes(dev):
     assert worst[F32] <= 1e-5 and worst[BF16] <= 2e-2
 
 
-@pytest.mark.parametrize("waves", [None, "4", "8"])
+@pytest.mark.parametrize("waves", [None, "4", "8", "40"])
 def test_sage_random_shapes(dev, waves, monkeypatch):
     with _device_with_waves(dev, waves, monkeypatch) as d:
         _sage_random_shapes(d)

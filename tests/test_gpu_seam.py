@@ -388,8 +388,8 @@ def test_sage_lens_entries_by_name(dev, kernels, bq, bk):
 
 def test_decoder_shape_with_key_lengths_by_name(dev, kernels):
     """The causal decoder configuration (B4 H32 S2048 D128, per-batch key lengths uniform in [S/2, S]) launched by
-    name: `ar_flash_bf16_long_lens` through arhip_launch, sampled rows against the bf16 emulation with
-    the same lengths, within three bf16 steps."""
+    name: `ar_flash_bf16_long_lens` and `ar_flash_bf16_mid_lens` through arhip_launch, sampled rows against the
+    bf16 emulation with the same lengths, within three bf16 steps."""
     from gpu_util import bf16_ulps
     b, h, n, d = 4, 32, 2048, 128
     q, k, v = (synth.normal(3001 + i, (b, h, n, d)) for i in range(3))
@@ -397,10 +397,15 @@ def test_decoder_shape_with_key_lengths_by_name(dev, kernels):
     with Bufs(dev) as bufs:
         dq, dk, dv = (bufs.put(synth.to_bf16_bits(t)) for t in (q, k, v))
         dl = bufs.put(lens)
-        do = bufs.new(q.size * 2, zero=False)
+        do, dm = bufs.new(q.size * 2, zero=False), bufs.new(q.size * 2, zero=False)
         dev.launch(kernels, "ar_flash_bf16_long_lens", _grid(n, 256, b, h), (512, 1, 1), [dq, dk, dv, do, do, dl],
                    [n, d, 1, 0, h, h])
         got = synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+        # the 4-wave form (what the dispatchers pick at this length) computes the same function in the
+        # same order: bit-identical
+        dev.launch(kernels, "ar_flash_bf16_mid_lens", _grid(n, 128, b, h), (256, 1, 1), [dq, dk, dv, dm, dm, dl],
+                   [n, d, 1, 0, h, h])
+        assert np.array_equal(dm.copyout(np.uint16, q.shape), do.copyout(np.uint16, q.shape))
     assert np.isfinite(got).all()
     rows = np.array([0, 1, 63, 64, 255, 256, 1023, 1024, 1500, 2047], np.int32)
     for bi, hi in ((0, 0), (1, 17), (3, 31)):
@@ -434,3 +439,51 @@ def test_named_entries_refuse_launches_they_cannot_run(dev, kernels):
                 dev.launch(kernels, name, grid, block, bufs_, vals)
         # and the same entry with a launch it can serve still runs
         dev.launch(kernels, "ar_flash_bf16_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x], ok)
+
+
+@pytest.mark.parametrize("d,causal,n", [(64, False, 700), (128, False, 700), (128, True, 1000), (64, True, 129), (128, False, 64)])
+def test_ar_flash_bf16_mid_by_name(dev, kernels, d, causal, n):
+    """The pipelined kernel with 4 waves / 128 queries per workgroup (K ring of two tiles, V ring of
+    three): against the oracle, and bit for bit against the 8-wave form."""
+    b, hq, hkv = 2, 4, 2
+    q, k, v = synth.normal(11, (b, hq, n, d)), synth.normal(12, (b, hkv, n, d)), synth.normal(13, (b, hkv, n, d))
+    with Bufs(dev) as bufs:
+        dq, dk, dv = (bufs.put(synth.to_bf16_bits(t)) for t in (q, k, v))
+        do, dl = bufs.new(q.size * 2), bufs.new(q.size * 2)
+        vals = [n, d, int(causal), 0, hq, hkv]
+        dev.launch(kernels, "ar_flash_bf16_mid", _grid(n, 128, b, hq), (256, 1, 1), [dq, dk, dv, do, do], vals)
+        dev.launch(kernels, "ar_flash_bf16_long", _grid(n, 256, b, hq), (512, 1, 1), [dq, dk, dv, dl, dl], vals)
+        bits = do.copyout(np.uint16, q.shape)
+        assert np.array_equal(bits, dl.copyout(np.uint16, q.shape))
+        got = synth.from_bf16_bits(bits)
+    want = oracle.attn_bf16(q, k, v, causal=causal)
+    assert np.abs(got - want).max() <= 2.0 ** -6
+    assert np.abs(got - oracle.sdpa_f64(q, k, v, causal=causal)).max() <= 2e-2
+
+
+@pytest.mark.parametrize("d,causal,out_f32,n", [(128, False, False, 1000), (128, True, True, 1000), (64, True, True, 333)])
+def test_ar_flash_sage_mid_by_name(dev, kernels, d, causal, out_f32, n):
+    b, hq, hkv, bq, bk = 1, 4, 2, 128, 64
+    q = synth.normal(21, (b, hq, n, d))
+    k = synth.normal(22, (b, hkv, n, d)) + np.float32(3.0) * synth.normal(24, (1, hkv, 1, d))
+    v = synth.normal(23, (b, hkv, n, d))
+    with Bufs(dev) as bufs:
+        q8, sq, _, h_q8, h_sq, _ = _quantise_by_name(dev, kernels, bufs, q, bq, False, F32)
+        k8, sk, _, h_k8, h_sk, _ = _quantise_by_name(dev, kernels, bufs, k, bk, True, F32)
+        dv = bufs.put(synth.to_bf16_bits(v))
+        do, dl = bufs.new(q.size * 4), bufs.new(q.size * 4)
+        vals = [n, d, int(causal), 0, hq, hkv, bq, bk, int(out_f32)]
+        dev.launch(kernels, "ar_flash_sage_mid", _grid(n, 128, b, hq), (256, 1, 1), [q8, k8, dv, do, do, sq, sk], vals)
+        dev.launch(kernels, "ar_flash_sage_long", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, dl, dl, sq, sk], vals)
+        def fetch(buf):
+            if out_f32:
+                return buf.copyout(np.float32, q.shape)
+            return synth.from_bf16_bits(buf.copyout(np.uint16, (2 * q.size,))[:q.size].reshape(q.shape))
+        got, got_long = fetch(do), fetch(dl)
+    want = oracle.sage(h_q8, h_k8, h_sq, h_sk, v, bq, bk, causal=causal, round_out=not out_f32)
+    tol = 2.0 ** -8 * float(np.abs(v).max())
+    assert np.abs(got - want).max() <= tol
+    # The 8-wave form is the same function, but not bit for bit: the grid its exponent reference moves on
+    # follows the largest Q scale of a workgroup's queries (128 here, 256 there), and P is rounded to
+    # bf16 relative to that reference.
+    assert np.abs(got - got_long).max() <= tol
