@@ -76,13 +76,16 @@ static void launch_pipe(hipStream_t stream, const AttnParams &p, bool causal)
 
 // Which of the two: 128 queries per workgroup hide a workgroup's prologue and epilogue under its
 // neighbour's tiles and fill the chip with fewer heads, but request every K/V tile twice as often and
-// keep only one tile in flight.  Measured at D = 128 (B4 H32): causal N = 512 / 1024 / 2048 -15 / -7 / -5 %,
-// B1 H16 N = 2048 causal -25 %, B2 H16 N = 1024 -22 %; non-causal N = 2048 equal, N = 8192 +3 %, causal
-// N = 32768 +4.5 %.
-static bool pipe_wants_4_waves(arhip_device *dev, int64_t heads, int64_t N)
+// keep only one tile in flight.  Two workgroups of equal length that start together stay in step and
+// hide nothing, so the gain is in few or unequal workgroups.  Measured at D = 128, bf16 (B4 H32 unless
+// noted; 4 waves against 8): causal N = 512 / 1024 / 2048 -15 / -7 / -5 %, B1 H16 N = 2048 causal -25 %,
+// B2 H16 N = 1024 -22 %, N = 1024 -4 %; N = 2048 equal; N = 2048 causal with key lengths in [N/2, N]
+// (many equal workgroups) +3 %; N = 8192 +3 %, causal N = 32768 +4.5 %.
+static bool pipe_wants_4_waves(arhip_device *dev, int64_t heads, int64_t N, bool causal, bool has_len)
 {
     if (dev->attn_waves == 8 || dev->attn_waves == 40) return dev->attn_waves == 40;
-    return N <= 2048 || heads * ((N + 255) / 256) < 2 * (int64_t)dev->cus;
+    if (heads * ((N + 255) / 256) < 2 * (int64_t)dev->cus) return true;
+    return N <= 1024 || (N <= 2048 && causal && !has_len);
 }
 
 // The pipelined kernel addresses K and V through 32-bit buffer offsets (rows of one head, plus the
@@ -222,7 +225,7 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
     int nw = pick_waves(dev, B * Hq, N, D, hm);
     if (nw == 8 && !pipe_addressable(N, kv_strides[2], 2)) nw = 4;
     const bool pipe = nw == 8;  // the software-pipelined kernel; how many waves it runs with is its own choice
-    if (pipe && pipe_wants_4_waves(dev, B * Hq, N)) nw = 4;
+    if (pipe && pipe_wants_4_waves(dev, B * Hq, N, causal != 0, kv_len != nullptr)) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;  // few workgroups per CU: balance them globally
@@ -318,7 +321,7 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
     if (nw == 1) nw = 4;
     if (nw == 8 && !pipe_addressable(N, std::max<int64_t>(D, v_strides ? v_strides[2] : D), 2)) nw = 4;
     const bool pipe = nw == 8 && !per_key && !dbg;
-    const bool pipe4 = pipe && !fp8 && pipe_wants_4_waves(dev, B * Hq, N);  // (the FP8 variant keeps to 8 waves)
+    const bool pipe4 = pipe && !fp8 && pipe_wants_4_waves(dev, B * Hq, N, causal != 0, kv_len != nullptr);  // (the FP8 variant keeps to 8 waves)
     if (pipe4) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);

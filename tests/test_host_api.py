@@ -392,8 +392,8 @@ def test_key_lengths_through_the_tensor_api(hdev, api, dtype):
 @gpu
 def test_decoder_configuration_through_the_tensor_api(hdev):
     """Causal decoder attention, B4 H32 S2048 D128 bf16 with key lengths uniform in [S/2, S], from
-    Tensor::attention_with: the pipelined `_lens` entry (4 waves at this length), sampled rows within three
-    bf16 steps of the bf16 emulation."""
+    Tensor::attention_with: the pipelined `_lens` entry, sampled rows within three bf16 steps of the bf16
+    emulation."""
     from gpu_util import bf16_ulps
     b, h, n, d = 4, 32, 2048, 128
     q, k, v = (synth.normal(3001 + i, (b, h, n, d)) for i in range(3))
@@ -402,8 +402,16 @@ def test_decoder_configuration_through_the_tensor_api(hdev):
     sess = Session()
     sess.begin_capture()
     out = tq.attention_with(tk, tv, None, 0.0, True, sess, None, Tensor.from_i32(hdev, lens))
-    # n <= 2048: the pipelined kernel in its 4-wave form (two workgroups per compute unit)
-    assert sess.end_capture() == 1 and sess.step(0)[0] == "ar_flash_bf16_mid_lens" and sess.step_detail(0)[1] == [256, 1, 1]
+    assert sess.end_capture() == 1 and sess.step(0)[0] == "ar_flash_bf16_long_lens" and sess.step_detail(0)[1] == [512, 1, 1]
+    # without key lengths the same shape takes the 4-wave form (two workgroups per compute unit)
+    sess.begin_capture()
+    out2 = tq.attention_with(tk, tv, None, 0.0, True, sess)
+    assert sess.end_capture() == 1 and sess.step(0)[0] == "ar_flash_bf16_mid" and sess.step_detail(0)[1] == [256, 1, 1]
+    full = out2.to_list()
+    bi, hi = 3, 9
+    rr = np.array([0, 127, 128, 1000, 2047], np.int32)
+    want = oracle.attn_bf16(q[bi:bi + 1, hi:hi + 1], k[bi:bi + 1, hi:hi + 1], v[bi:bi + 1, hi:hi + 1], causal=True, rows=rr)
+    assert bf16_ulps(full[bi:bi + 1, hi:hi + 1][:, :, rr], want) <= 3.0
     got = out.to_list()
     rows = np.array([0, 63, 64, 255, 256, 1023, 1024, 1500, 2047], np.int32)
     for bi, hi in ((0, 3), (2, 30)):
