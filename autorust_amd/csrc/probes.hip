@@ -210,6 +210,53 @@ PROBE_ISSUE_MIX_KS(probe_mix_bf16_exp, true, false)
 PROBE_ISSUE_MIX_KS(probe_mix_i8_fma, false, true)
 PROBE_ISSUE_MIX_KS(probe_mix_i8_exp, true, true)
 
+// The same loop with 8 v_fma_f32 and S scalar instructions (s_add_u32) per matrix instruction: what a scalar
+// instruction costs the SIMD's instruction issue.  ticks as above.
+template <int S>
+__device__ __forceinline__ void probe_issue_salu_body(const uint4 *src, float *out, long long *ticks, int iters)
+{
+    float d[8], a = threadIdx.x * 0.001f, b = 1.0001f;
+    for (int i = 0; i < 8; ++i) d[i] = i * 0.5f;
+    const uint4 fa = src[threadIdx.x & 1023], fb = src[(threadIdx.x + 512) & 1023];
+    f32x16 o[4];
+    for (int n = 0; n < 4; ++n)
+        for (int r = 0; r < 16; ++r) o[n][r] = 0.f;
+    int sacc = 0;
+    const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            o[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa), __builtin_bit_cast(bf16x8, fb), o[j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) asm volatile("v_fma_f32 %0, %1, %2, %0" : "+v"(d[i & 7]) : "v"(a), "v"(b));
+#pragma unroll
+            for (int i = 0; i < S; ++i) asm volatile("s_add_u32 %0, %0, 1" : "+s"(sacc));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    const long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+    float r = (float)sacc;
+    for (int i = 0; i < 8; ++i) r += d[i];
+    for (int n = 0; n < 4; ++n)
+        for (int i = 0; i < 16; ++i) r += o[n][i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = r;
+    if ((threadIdx.x & 63) == 0) {
+        const int w = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
+        ticks[2 * w] = c1 - c0;
+        ticks[2 * w + 1] = r1 - r0;
+    }
+}
+#define PROBE_ISSUE_SALU(NAME, S)                                                                                      \
+    extern "C" __global__ void __launch_bounds__(768) NAME(const uint4 *src, float *out, long long *ticks, int iters)  \
+    {                                                                                                                  \
+        probe_issue_salu_body<S>(src, out, ticks, iters);                                                              \
+    }
+PROBE_ISSUE_SALU(probe_mix_salu_s0, 0)
+PROBE_ISSUE_SALU(probe_mix_salu_s2, 2)
+PROBE_ISSUE_SALU(probe_mix_salu_s4, 4)
+PROBE_ISSUE_SALU(probe_mix_salu_s8, 8)
+
 // How exactly the 8-bit floating-point matrix instructions add up their products: the dot product of
 // two vectors of 64 E4M3 codes, once with the 64-deep scaled instruction and once with four 16-deep
 // ones (every lane half takes the same bytes of both operands, so every element of the result is the

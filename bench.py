@@ -312,6 +312,15 @@ def issue_mix(dev):
                     cyc, ns = t[0] / (iters * 4) / waves, t[1] * 10.0 / (iters * 4) / waves
                     row["K=%d" % k] = [round(float(cyc), 1), round(float(ns), 2), round(float(t[0] / t[1] * 100.0))]
                 res["%s_mfma+%s_%dwaves" % (mat, op, waves)] = row
+    # scalar instructions: bf16 MFMA + 8 v_fma_f32 + S s_add_u32 per matrix instruction, two waves per SIMD
+    row = {}
+    for sc in (0, 2, 4, 8):
+        for _ in range(2):
+            dev.launch(mod, "probe_mix_salu_s%d" % sc, (256, 1, 1), (512, 1, 1), [src, out, ticks], [iters])
+        t = ticks.copyout(np.int64, (256 * 8, 2)).astype(np.float64).mean(axis=0)
+        row["S=%d" % sc] = [round(float(t[0] / (iters * 4) / 2), 1), round(float(t[1] * 10.0 / (iters * 4) / 2), 2),
+                            round(float(t[0] / t[1] * 100.0))]
+    res["bf16_mfma+8fma+S_salu_2waves"] = row
     src.free()
     out.free()
     ticks.free()
