@@ -81,9 +81,13 @@ static void launch_pipe(hipStream_t stream, const AttnParams &p, bool causal)
 // noted; 4 waves against 8): causal N = 512 / 1024 / 2048 -15 / -7 / -5 %, B1 H16 N = 2048 causal -25 %,
 // B2 H16 N = 1024 -22 %, N = 1024 -4 %; N = 2048 equal; N = 2048 causal with key lengths in [N/2, N]
 // (many equal workgroups) +3 %; N = 8192 +3 %, causal N = 32768 +4.5 %.
-static bool pipe_wants_4_waves(arhip_device *dev, int64_t heads, int64_t N, bool causal, bool has_len)
+// At D = 64 (B4 H32): N = 2048 -8 %, N = 8192 -2 %, causal N = 2048 -16 %, causal N = 8192 -4 %: always 4 waves.
+// (Three such workgroups per compute unit fit at D = 64, 154 registers and 40 KB of LDS each, and run no
+// faster than two.)
+static bool pipe_wants_4_waves(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bool causal, bool has_len)
 {
     if (dev->attn_waves == 8 || dev->attn_waves == 40) return dev->attn_waves == 40;
+    if (D == 64) return true;
     if (heads * ((N + 255) / 256) < 2 * (int64_t)dev->cus) return true;
     return N <= 1024 || (N <= 2048 && causal && !has_len);
 }
@@ -225,7 +229,7 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
     int nw = pick_waves(dev, B * Hq, N, D, hm);
     if (nw == 8 && !pipe_addressable(N, kv_strides[2], 2)) nw = 4;
     const bool pipe = nw == 8;  // the software-pipelined kernel; how many waves it runs with is its own choice
-    if (pipe && pipe_wants_4_waves(dev, B * Hq, N, causal != 0, kv_len != nullptr)) nw = 4;
+    if (pipe && pipe_wants_4_waves(dev, B * Hq, N, D, causal != 0, kv_len != nullptr)) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;  // few workgroups per CU: balance them globally
@@ -321,7 +325,7 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
     if (nw == 1) nw = 4;
     if (nw == 8 && !pipe_addressable(N, std::max<int64_t>(D, v_strides ? v_strides[2] : D), 2)) nw = 4;
     const bool pipe = nw == 8 && !per_key && !dbg;
-    const bool pipe4 = pipe && !fp8 && pipe_wants_4_waves(dev, B * Hq, N, causal != 0, kv_len != nullptr);  // (the FP8 variant keeps to 8 waves)
+    const bool pipe4 = pipe && !fp8 && pipe_wants_4_waves(dev, B * Hq, N, D, causal != 0, kv_len != nullptr);  // (the FP8 variant keeps to 8 waves)
     if (pipe4) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);

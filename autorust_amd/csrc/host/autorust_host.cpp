@@ -394,8 +394,9 @@ bool long_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int6
 
 // ... and run with 4 waves / 128 queries per workgroup (the `_mid` entry points, two workgroups per compute
 // unit) where a workgroup sees few tiles: the rule of arhip_flash_fwd / arhip_sage_fwd
-bool mid_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int64_t n, bool causal, bool has_lens)
+bool mid_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int64_t n, int64_t d, bool causal, bool has_lens)
 {
+    if (d == 64) return true;
     if (b * h * ((n + 255) / 256) < 2 * (int64_t)dev->compute_units()) return true;
     return n <= 1024 || (n <= 2048 && causal && !has_lens);
 }
@@ -444,7 +445,7 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
         if (!has_mask && !key_lengths && n <= 256 && b * h * ((n + 127) / 128) <= 4 * (int64_t)dev->compute_units())
             calls.push_back(make_call(dev, "ar_flash_bf16_short", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 127) / 128, b * h, 1}, {512, 1, 1}, vals));
-        else if (!has_mask && long_variant(dev, b, h, n, d) && mid_variant(dev, b, h, n, is_causal, key_lengths != nullptr))
+        else if (!has_mask && long_variant(dev, b, h, n, d) && mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr))
             calls.push_back(attn_call("ar_flash_bf16_mid", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 127) / 128, b * h, 1}, {256, 1, 1}, vals));
         else if (!has_mask && long_variant(dev, b, h, n, d))
@@ -504,7 +505,7 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     const bool tile_uniform = ((int64_t)64 << shift) == bk;
     if (!has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
         svals.push_back(bf16_in ? 0 : 1);  // out_f32
-        if (!st.sage_fp8 && mid_variant(dev, b, h, n, is_causal, key_lengths != nullptr))
+        if (!st.sage_fp8 && mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr))
             calls.push_back(attn_call("ar_flash_sage_mid", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
                                       {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
         else

@@ -156,9 +156,10 @@ fn long_variant(dev: &str, b: i64, h: i64, n: i64, d: i64) -> bool {
 }
 
 /// ... and run with 4 waves / 128 queries per workgroup (`_mid`: two workgroups per compute unit, one's
-/// prologue and epilogue under the other's tiles) where a workgroup sees few tiles.
-fn mid_variant(dev: &str, b: i64, h: i64, n: i64, causal: bool, has_lens: bool) -> bool {
-    if b * h * ((n + 255) / 256) < 2 * crate::runtime::ops_hip::compute_units(dev) {
+/// prologue and epilogue under the other's tiles) where a workgroup sees few tiles, and always at
+/// `head_dim` 64.
+fn mid_variant(dev: &str, b: i64, h: i64, n: i64, d: i64, causal: bool, has_lens: bool) -> bool {
+    if d == 64 || b * h * ((n + 255) / 256) < 2 * crate::runtime::ops_hip::compute_units(dev) {
         return true;
     }
     n <= 1024 || (n <= 2048 && causal && !has_lens)
@@ -188,7 +189,7 @@ pub fn host_call_bf16(dev: &str, bufs: Vec<Buffer>, lens: Option<Buffer>, b: i64
     if !opts.has_mask && lens.is_none() && n <= 256 && b * h * ((n + 127) / 128) <= 4 * crate::runtime::ops_hip::compute_units(dev) {
         // all of K/V of a head in LDS at once: the ViT sequence lengths
         call("ar_flash_bf16_short", bufs, &[bf, bf, bf, bf, f], [(n + 127) / 128, b * h, 1], [512, 1, 1], vals(n, d, h, opts), &[])
-    } else if !opts.has_mask && long_variant(dev, b, h, n, d) && mid_variant(dev, b, h, n, opts.causal, lens.is_some()) {
+    } else if !opts.has_mask && long_variant(dev, b, h, n, d) && mid_variant(dev, b, h, n, d, opts.causal, lens.is_some()) {
         attn_call("ar_flash_bf16_mid", bufs, &[bf, bf, bf, bf, f], lens, [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts))
     } else if !opts.has_mask && long_variant(dev, b, h, n, d) {
         attn_call("ar_flash_bf16_long", bufs, &[bf, bf, bf, bf, f], lens, [(n + 255) / 256, b * h, 1], [512, 1, 1], vals(n, d, h, opts))
@@ -281,7 +282,7 @@ pub fn host_calls_sage(
     let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
     if !opts.has_mask && tile_uniform && long_variant(dev, b, h, n, d) {
         sv.push(!bf16_in as i64); // out_f32
-        if !sage.fp8 && mid_variant(dev, b, h, n, opts.causal, lens.is_some()) {
+        if !sage.fp8 && mid_variant(dev, b, h, n, d, opts.causal, lens.is_some()) {
             calls.push(attn_call("ar_flash_sage_mid", vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
                                  [(n + 127) / 128, b * h, 1], [256, 1, 1], sv));
         } else {
