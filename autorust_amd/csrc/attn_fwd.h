@@ -325,6 +325,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
         sq_lane = p.sq[(size_t)bh * nqb + min(q_row, N - 1) / p.bq];
     }
     const float c_scale = p.scale * LOG2E;
+    const float sq_c = (sq_lane * p.scale) * LOG2E;  // per-key scales: the query's share of the exponent factor
     // ---- per-block pipeline ----------------------------------------------------------
     // A tile is two blocks of 32 keys.  For every block the wave alternates between the
     // matrix pipe and the vector ALU, and every LDS fragment is requested one phase before
@@ -432,6 +433,38 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
                 // src/runtime/cuda_flash_sage.rs:315-322.  The row sum bounds the largest probability
                 // (max <= sum <= 16 max), so only a sum that is too large (or not finite: the very first
                 // block, or a jump of the maximum) sends the wave to the exact path below.
+                if constexpr (PER_KEY) {
+                    // one factor per key (the reference's own granularity, src/runtime/cuda_flash_sage.rs:264-268,
+                    // 315-322): the tile's K scales sit in LDS, and element r of a lane is key
+                    // 8 (r / 4) + 4 h + r % 4 of the block, so four 16-byte reads fetch the lane's sixteen
+                    // (the query's part of the factor, (sq scale) log2 e, is a per-lane constant: one multiply per
+                    // key instead of three; against (sq sk) scale the factor moves by two units in the last place)
+                    float cr[16];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const float4 sk4 = *(const float4 *)(vl + V_TILE + (blk * 32 + 8 * g + 4 * h) * 4);
+                        cr[4 * g + 0] = sq_c * sk4.x;
+                        cr[4 * g + 1] = sq_c * sk4.y;
+                        cr[4 * g + 2] = sq_c * sk4.z;
+                        cr[4 * g + 3] = sq_c * sk4.w;
+                    }
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[r], cr[r], -m_run));
+                    rs = row_sum();
+                    if (__any(!(rs <= 16.0f * LAZY_LIMIT))) {
+                        float y[16];
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) y[r] = (float)s[r] * cr[r];
+                        float mx = max3(y[0], y[1], y[2]);
+#pragma unroll
+                        for (int r = 3; r < 15; r += 2) mx = max3(mx, y[r], y[r + 1]);
+                        mx = xhalf_max(fmaxf(mx, y[15]));
+                        move_reference(mx);
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[r], cr[r], -m_run));
+                        rs = row_sum();
+                    }
+                } else {
                 const float c = (MODE != MODE_BF16) ? ((sq_lane * f_tile) * p.scale) * LOG2E : c_scale;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[r], c, -m_run));
@@ -446,6 +479,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
 #pragma unroll
                     for (int r = 0; r < 16; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[r], c, -m_run));
                     rs = row_sum();
+                }
                 }
             } else {
 #pragma unroll
@@ -574,7 +608,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     __syncthreads();
     auto nothing = [] {};
 
-    if constexpr (!CAUSAL && !HAS_MASK && !PER_KEY) {
+    if constexpr (!CAUSAL && !HAS_MASK) {
         // only the last tile can hold masked keys: keep it out of the loop
         const int nfull = kend / BK;
 #pragma clang loop unroll(disable)
@@ -597,7 +631,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
             if (it < my_tiles) {
                 const int k0 = it * BK;
                 const bool masked = (k0 + BK > kend) || (CAUSAL && (k0 + BK - 1 > wq0));
-                if (HAS_MASK || PER_KEY || masked) tile_body(std::true_type{}, it, stage_ahead);
+                if (HAS_MASK || masked) tile_body(std::true_type{}, it, stage_ahead);
                 else tile_body(std::false_type{}, it, stage_ahead);
             } else {
                 stage_ahead();
