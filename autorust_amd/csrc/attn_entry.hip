@@ -14,14 +14,13 @@
 //   ar_flash_f32        [256,1,1]  [ceil(n/128), B*hq, 1]    fp32 exact (cuda_flash.rs)
 //   ar_flash_f32_short  [256,1,1]  [ceil(n/32), B*hq, 1]     fp32 exact for few, short heads; head_dim 64
 //   ar_flash_bf16       [256,1,1]  [ceil(n/128), B*hq, 1]    bf16 (cuda_flash_bf16.rs), any mask
-//   ar_flash_bf16_long  [512,1,1]  [ceil(n/256), B*hq, 1]    bf16 pipelined, has_mask must be 0
+//   ar_flash_bf16_long  [512,1,1]  [ceil(n/256), B*hq, 1]    bf16 software-pipelined, has_mask must be 0
 //   ar_flash_bf16_mid   [256,1,1]  [ceil(n/128), B*hq, 1]    the same with 4 waves (two workgroups per CU): short / causal
-//   ar_flash_bf16_short [512,1,1]  [ceil(n/128), B*hq, 1]    bf16, n <= 256, has_mask must be 0
 //   ar_flash_sage       [256,1,1]  [ceil(n/128), B*hq, 1]    int8 (cuda_flash_sage.rs), any mask, any
 //                                                            block sizes incl. per-row scales; O f32
 //   ar_flash_sage_long  [512,1,1]  [ceil(n/256), B*hq, 1]    int8 pipelined: has_mask 0, bk = 64 * 2^n
 //   ar_flash_sage_mid   [256,1,1]  [ceil(n/128), B*hq, 1]    the same with 4 waves
-//   ar_flash_sage_fp8_long  the same on E4M3 codes
+//   ar_flash_sage_fp8_long, ar_flash_sage_fp8_mid  the same on E4M3 codes
 // The Sage entries take pre-quantised operands (the quantiser is the pre-pass below, not part of
 // the attention kernel as in the reference):
 //     (Q8, K8, V, O, M, SQ, SK,  N, head_dim, causal, has_mask, hq, hkv, bq, bk [, out_f32])
@@ -38,7 +37,7 @@
 // a batch with L[b] = 0 yields zeros), with the same scalars, grid and block:
 //     ar_flash_f32_lens, ar_flash_bf16_lens, ar_flash_bf16_long_lens, ar_flash_bf16_mid_lens   (Q, K, V, O, M, L,  6 ints)
 //     ar_flash_sage_lens, ar_flash_sage_long_lens, ar_flash_sage_mid_lens, ar_flash_sage_fp8_lens,
-//     ar_flash_sage_fp8_long_lens                                             (Q8, K8, V, O, M, L, SQ, SK,  ints as above)
+//     ar_flash_sage_fp8_long_lens, ar_flash_sage_fp8_mid_lens                 (Q8, K8, V, O, M, L, SQ, SK,  ints as above)
 // (The reference's fused kernels take a dense [n, n] mask only, src/models/flash_attention.rs:389-396; its
 // Tensor API reaches key-padding masks through the general path, src/tensor/mod.rs:2405-2447.)
 // head_dim must be 64 or 128; any other value makes the kernel return without writing.
@@ -319,25 +318,6 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16_lens(const uint1
     flash_bf16_entry(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
 }
 
-// sequences of at most 256 keys: all of K/V of the head in LDS at once, 8 waves (two per 32 queries on
-// the even / odd key tiles).  has_mask must be 0 and N <= 256; anything else returns without writing.
-extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_short(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
-                                                                       uint16_t *O, const float *M, int N, int head_dim,
-                                                                       int causal, int has_mask, int hq, int hkv)
-{
-    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<128, 8, MODE_BF16, false, true>()];
-    if (has_mask || N > 256) return;
-    AttnParams p = dense_params(Q, K, V, O, M, N, head_dim, 0, hq, hkv);
-    const int wg = linear_wg();
-    if (head_dim == 64) {
-        if (causal) attn_fwd_body<64, 8, true, false, MODE_BF16, false, false, false, true, 2>(p, lds, wg);
-        else attn_fwd_body<64, 8, false, false, MODE_BF16, false, false, false, true, 2>(p, lds, wg);
-    } else if (head_dim == 128) {
-        if (causal) attn_fwd_body<128, 8, true, false, MODE_BF16, false, false, false, true, 2>(p, lds, wg);
-        else attn_fwd_body<128, 8, false, false, MODE_BF16, false, false, false, true, 2>(p, lds, wg);
-    }
-}
-
 namespace {
 template <int NW>
 __device__ __forceinline__ void flash_bf16_long_entry(unsigned char *lds, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
@@ -550,6 +530,25 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long_lens(co
 {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8>()];
     flash_sage_long_entry<MODE_FP8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_mid(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
+                                                                            void *O, const float *M, const float *SQ, const float *SK,
+                                                                            int N, int head_dim, int causal, int has_mask, int hq,
+                                                                            int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 4>()];
+    flash_sage_long_entry<MODE_FP8, 4>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_mid_lens(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
+                                                                                 void *O, const float *M, const int *L, const float *SQ,
+                                                                                 const float *SK, int N, int head_dim, int causal,
+                                                                                 int has_mask, int hq, int hkv, int bq, int bk,
+                                                                                 int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 4>()];
+    flash_sage_long_entry<MODE_FP8, 4>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
 // ---- Sage pre-pass (the quantiser the reference runs inside its attention kernel,

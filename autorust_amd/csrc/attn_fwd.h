@@ -13,8 +13,7 @@
 //           workgroup (two stages, one barrier per tile) and two tiles ahead of
 //           the math: in the middle of the iteration that computes tile i, tile
 //           i+1 goes from registers to the stage tile i-1 vacated, and the
-//           128-bit global loads of tile i+2 are issued.  Sequences of at most
-//           256 keys are brought into LDS in one go instead (SMALL).
+//           128-bit global loads of tile i+2 are issued.
 //   blocks: inside a tile the online softmax advances 32 keys at a time and the
 //           wave alternates between the matrix pipe and the vector ALU; every
 //           LDS fragment is requested one phase before the MFMAs that use it.
@@ -136,30 +135,22 @@ __device__ __forceinline__ uint2 lds_read_tr16(const unsigned char *p)
 __device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
 // LDS bytes attn_fwd_body needs for a tiling variant
-template <int D, int NW, int MODE, bool PER_KEY, bool SMALL = false>
+template <int D, int NW, int MODE, bool PER_KEY>
 constexpr int attn_fwd_lds_bytes()
 {
     constexpr int QKB = (MODE != MODE_BF16) ? 1 : 2;
-    return (SMALL ? 4 : 2) * (BK * (D * QKB + 16) + BK * (D * 2 + 64) + (PER_KEY ? BK * 4 : 0));
+    return 2 * (BK * (D * QKB + 16) + BK * (D * 2 + 64) + (PER_KEY ? BK * 4 : 0));
 }
 
 // The kernel body.  lds: attn_fwd_lds_bytes<...>() bytes of workgroup memory, 16-byte aligned;
 // wg_linear: this workgroup's index in [0, p.total) (the entry points below and the named entry
 // points of the loadable code object derive it from their grids).
-template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false,
-          int KSPLIT = 1>
+template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG>
 __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
-    // KSPLIT = 2 (with SMALL): waves w and w + NW/2 own the same 32 queries and take the even / odd
-    // key tiles; their (m, l, O) are merged through LDS at the end.  A short sequence gives a wave
-    // only a handful of blocks, each a serial MFMA -> softmax -> MFMA chain: two waves per SIMD on
-    // half the blocks each overlap those chains and halve their length.
-    static_assert(KSPLIT == 1 || (KSPLIT == 2 && SMALL && NW % 2 == 0), "key splitting is built for the preloading variant");
-    constexpr int QW = NW / KSPLIT;  // waves that own distinct queries
-    // SMALL: the whole sequence (at most 4 tiles) is brought into LDS up front, all global loads
-    // in flight at once and a single barrier: short sequences are latency bound, not math bound.
-    constexpr int NSTAGE = SMALL ? 4 : 2;
-    constexpr int NSLOT = SMALL ? 4 : 1;  // register sets for tiles in flight
+    constexpr int QW = NW;      // waves of a workgroup, each with 32 queries of its own
+    constexpr int NSTAGE = 2;
+    constexpr int NSLOT = 1;    // register sets for tiles in flight
     constexpr int T = NW * 64;
     constexpr int BQ = QW * 32;
     constexpr int QK_BYTES = (MODE != MODE_BF16) ? 1 : 2;        // bytes per q/k element
@@ -182,7 +173,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     static_assert(!PER_KEY || MODE != MODE_BF16, "per-key scales belong to the 8-bit paths");
     static_assert(!DBG || MODE == MODE_I8, "the logits export is int32");
 
-    static_assert(NSTAGE * STAGE == attn_fwd_lds_bytes<D, NW, MODE, PER_KEY, SMALL>(), "LDS size bookkeeping");
+    static_assert(NSTAGE * STAGE == attn_fwd_lds_bytes<D, NW, MODE, PER_KEY>(), "LDS size bookkeeping");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -215,8 +206,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     const int N = p.N;
 
     const int qblk = qt * BQ;
-    const int qwave = wave % QW, kpart = wave / QW;
-    const int wq0 = qblk + qwave * 32;  // first query of this wave
+    const int wq0 = qblk + wave * 32;  // first query of this wave
     const int q_row = wq0 + i32;
 
     int kvl = N;
@@ -542,60 +532,6 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
         }
     };
 
-    if constexpr (SMALL) {
-        static_assert(!PER_KEY, "the preloading variant has no per-key scales");
-#pragma unroll
-        for (int t = 0; t < NSLOT; ++t)
-            if (t < ntiles) load_tile(t * BK, t);
-#pragma unroll
-        for (int t = 0; t < NSLOT; ++t)
-            if (t < ntiles) store_tile(t, t);
-        __syncthreads();
-        auto nothing = [] {};
-        for (int it = kpart; it < my_tiles; it += KSPLIT) {
-            const int k0 = it * BK;
-            const bool masked = (k0 + BK > kend) || (CAUSAL && (k0 + BK - 1 > wq0));
-            if (HAS_MASK || masked) tile_body(std::true_type{}, it, nothing);
-            else tile_body(std::false_type{}, it, nothing);
-        }
-        if constexpr (KSPLIT == 2) {
-            // merge the two key halves: m = max, l and O rescaled by 2^(m_part - m)
-            // per query group: O as float4 [DB * 4][64 lanes], then (m, l) as float2 [64 lanes]: 16-byte
-            // accesses at consecutive addresses, lane-major
-            constexpr int SLAB = DB * 16 * 64 + 128;  // floats per query group
-            static_assert(QW * SLAB * 4 <= NSTAGE * STAGE, "merge buffer fits the tile stages");
-            __syncthreads();  // every wave is done with the tiles
-            float *mb = (float *)lds + qwave * SLAB;
-            float4 *mb4 = (float4 *)mb;
-            float2 *ml = (float2 *)(mb + DB * 16 * 64);
-            if (kpart == 1) {
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-                        mb4[(db * 4 + g) * 64 + lane] = make_float4(oacc[db][4 * g], oacc[db][4 * g + 1], oacc[db][4 * g + 2], oacc[db][4 * g + 3]);
-                ml[lane] = make_float2(m_run, l_run);
-            }
-            __syncthreads();
-            if (kpart == 1) return;
-            const float2 ml1 = ml[lane];
-            const float m1 = ml1.x, l1 = ml1.y;
-            const float m = fmaxf(m_run, m1);
-            const float f0 = __builtin_amdgcn_exp2f(m_run - m), f1 = __builtin_amdgcn_exp2f(m1 - m);
-            l_run = l_run * f0 + l1 * f1;
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const float4 o1 = mb4[(db * 4 + g) * 64 + lane];
-                    oacc[db][4 * g + 0] = oacc[db][4 * g + 0] * f0 + o1.x * f1;
-                    oacc[db][4 * g + 1] = oacc[db][4 * g + 1] * f0 + o1.y * f1;
-                    oacc[db][4 * g + 2] = oacc[db][4 * g + 2] * f0 + o1.z * f1;
-                    oacc[db][4 * g + 3] = oacc[db][4 * g + 3] * f0 + o1.w * f1;
-                }
-            m_run = m;
-        }
-    } else {
     // Staging runs two tiles ahead of the math with one set of registers: in the middle of the
     // iteration that computes tile i, tile i+1 (loaded during iteration i-1) goes from registers
     // to the LDS stage that tile i-1 vacated at the last barrier, and the loads of tile i+2 are
@@ -639,7 +575,6 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
             __syncthreads();
         }
     }
-    }
 
     // ---- normalise and store: acc * (l > 0 ? 1/l : 0), cuda_flash_bf16.rs:414-426 ----
     const float l_tot = xhalf_sum(l_run);
@@ -670,12 +605,11 @@ __device__ __forceinline__ void attn_fwd_body(const AttnParams &p, unsigned char
     }
 }
 
-template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG, bool SMALL = false,
-          int KSPLIT = 1>
-__global__ void __launch_bounds__(NW * 64, (NW == 4 && !SMALL ? 2 : 1)) attn_fwd_kernel(const AttnParams p)
+template <int D, int NW, bool CAUSAL, bool HAS_MASK, int MODE, bool PER_KEY, bool OUT_F32, bool DBG>
+__global__ void __launch_bounds__(NW * 64, (NW == 4 ? 2 : 1)) attn_fwd_kernel(const AttnParams p)
 {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<D, NW, MODE, PER_KEY, SMALL>()];
-    attn_fwd_body<D, NW, CAUSAL, HAS_MASK, MODE, PER_KEY, OUT_F32, DBG, SMALL, KSPLIT>(p, lds, (int)blockIdx.x);
+    __shared__ __attribute__((aligned(16))) unsigned char lds[attn_fwd_lds_bytes<D, NW, MODE, PER_KEY>()];
+    attn_fwd_body<D, NW, CAUSAL, HAS_MASK, MODE, PER_KEY, OUT_F32, DBG>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

@@ -437,7 +437,6 @@ const named_entry NAMED[] = {
     {"ar_flash_bf16_long_lens", 6, 6, 512, 256, false, true, true, 0, false},
     {"ar_flash_bf16_mid", 5, 6, 256, 128, false, true, true, 0, false},
     {"ar_flash_bf16_mid_lens", 6, 6, 256, 128, false, true, true, 0, false},
-    {"ar_flash_bf16_short", 5, 6, 512, 128, false, true, false, 256, false},
     {"ar_flash_sage", 7, 8, 256, 128, false, false, false, 0, false},
     {"ar_flash_sage_lens", 8, 8, 256, 128, false, false, false, 0, false},
     {"ar_flash_sage_fp8", 7, 8, 256, 128, false, false, false, 0, false},
@@ -446,6 +445,8 @@ const named_entry NAMED[] = {
     {"ar_flash_sage_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
     {"ar_flash_sage_mid", 7, 9, 256, 128, false, true, true, 0, false},
     {"ar_flash_sage_mid_lens", 8, 9, 256, 128, false, true, true, 0, false},
+    {"ar_flash_sage_fp8_mid", 7, 9, 256, 128, false, true, true, 0, false},
+    {"ar_flash_sage_fp8_mid_lens", 8, 9, 256, 128, false, true, true, 0, false},
     {"ar_flash_sage_fp8_long", 7, 9, 512, 256, false, true, true, 0, false},
     {"ar_flash_sage_fp8_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
     {"ar_fl_fwd", 6, 6, 256, 128, false, false, false, 0, false},

@@ -99,20 +99,18 @@ static bool pipe_addressable(int64_t N, int64_t kv_token_stride, int64_t elem_by
     return (N + 5 * 64) * kv_token_stride * elem_bytes < ((int64_t)1 << 31);
 }
 
-// Tiling variants = waves (of 32 queries) per workgroup.
-//   1  32 queries per workgroup: short sequences, spreads the heads over the chip
-//   4  128 queries
-//   8  256 queries, two waves per SIMD (long sequences)
+// Which kernel.  Launches without an additive mask, per-key scales or the logits export take the
+// software-pipelined kernel (returned as 8; whether it runs with 8 or 4 waves per workgroup is
+// pipe_wants_4_waves' choice): with its 4-wave form it is the fastest kernel down to the shortest sequences
+// (bf16, against the kernels that used to serve them: B8 H12 N197 D64 7.8 -> 7.0 us, B4 H16 N256 D128 11.8 ->
+// 9.0 us, B32 H12 N64 D64 9.1 -> 5.6 us, B8 H12 N400 D64 27.8 -> 12.9 us).  The others take the general
+// kernel with 4 waves of 32 queries, or 1 at D = 64 when that still leaves compute units idle.
 static int pick_waves(arhip_device *dev, int64_t heads, int64_t N, int64_t D, bool special)
 {
-    // masks, per-key scales and the debug export are built for 4 waves (and 1 at D = 64) only
-    // The 8-wave kernel is the software-pipelined one: it hides the memory latency of a tile
-    // behind the tiles before, which from ~8 tiles per workgroup on outweighs leaving compute units
-    // without a workgroup (B8 H6 N789 D64: 23 us against 56 us with 1200 one-wave workgroups).
-    const int64_t cus = dev->cus, wg256 = heads * ((N + 255) / 256), wg128 = heads * ((N + 127) / 128);
+    const int64_t cus = dev->cus, wg128 = heads * ((N + 127) / 128);
     int nw;
-    if (!special && (wg256 >= 2 * cus || (N >= 512 && 2 * wg256 >= cus))) nw = 8;
-    else if (D == 64 && wg128 < 2 * cus && (special || N < 512)) nw = 1;
+    if (!special) nw = 8;
+    else if (D == 64 && wg128 < 2 * cus) nw = 1;
     else nw = 4;
     // ARHIP_ATTN_WAVES (read once when the device is opened) is a tuning aid; results do not depend on it
     // (1, 4: the general kernel with that many waves; 8, 40: the pipelined kernel with 8 / 4 waves)
@@ -234,20 +232,7 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;  // few workgroups per CU: balance them globally
     if (int rc = t.begin()) return rc;
-    if (N <= 256 && !hm && B * Hq * ((N + 127) / 128) <= 4 * (int64_t)dev->cus && dev->attn_waves == 0) {
-        // short sequence: bring all of K/V into LDS at once (128 queries per workgroup)
-        p.nq = (int)((N + 127) / 128);
-        p.total = (int)(p.nq * B * Hq);
-        // 8 waves: two per 32 queries, one on the even and one on the odd key tiles
-        const dim3 grid((unsigned)p.total), block(512);
-        if (D == 64) {
-            if (c) hipLaunchKernelGGL((attn_fwd_kernel<64, 8, true, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
-            else hipLaunchKernelGGL((attn_fwd_kernel<64, 8, false, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
-        } else {
-            if (c) hipLaunchKernelGGL((attn_fwd_kernel<128, 8, true, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
-            else hipLaunchKernelGGL((attn_fwd_kernel<128, 8, false, false, MODE_BF16, false, false, false, true, 2>), grid, block, 0, dev->stream, p);
-        }
-    } else if (D == 64) {
+    if (D == 64) {
         if (pipe && nw == 4) launch_pipe<64, MODE_BF16, false, 4>(dev->stream, p, c);
         else if (pipe) launch_pipe<64, MODE_BF16, false>(dev->stream, p, c);
         else if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
@@ -325,7 +310,7 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
     if (nw == 1) nw = 4;
     if (nw == 8 && !pipe_addressable(N, std::max<int64_t>(D, v_strides ? v_strides[2] : D), 2)) nw = 4;
     const bool pipe = nw == 8 && !per_key && !dbg;
-    const bool pipe4 = pipe && !fp8 && pipe_wants_4_waves(dev, B * Hq, N, D, causal != 0, kv_len != nullptr);  // (the FP8 variant keeps to 8 waves)
+    const bool pipe4 = pipe && pipe_wants_4_waves(dev, B * Hq, N, D, causal != 0, kv_len != nullptr);
     if (pipe4) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
@@ -362,7 +347,10 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
         if (f32o) launch_attn<DD, 4, MODE_FP8, PK, true, false, true>(dev->stream, p, c, hm);          \
         else launch_attn<DD, 4, MODE_FP8, PK, false, false, true>(dev->stream, p, c, hm);              \
     } while (0)
-    if (fp8 && nw == 8 && !per_key) {
+    if (fp8 && pipe4) {
+        if (D == 64) { if (f32o) launch_pipe<64, MODE_FP8, true, 4>(dev->stream, p, c); else launch_pipe<64, MODE_FP8, false, 4>(dev->stream, p, c); }
+        else { if (f32o) launch_pipe<128, MODE_FP8, true, 4>(dev->stream, p, c); else launch_pipe<128, MODE_FP8, false, 4>(dev->stream, p, c); }
+    } else if (fp8 && pipe) {
         if (D == 64) { if (f32o) launch_pipe<64, MODE_FP8, true>(dev->stream, p, c); else launch_pipe<64, MODE_FP8, false>(dev->stream, p, c); }
         else { if (f32o) launch_pipe<128, MODE_FP8, true>(dev->stream, p, c); else launch_pipe<128, MODE_FP8, false>(dev->stream, p, c); }
     } else if (fp8) {

@@ -384,12 +384,11 @@ HostCall make_call(const std::shared_ptr<Device> &dev, const char *name, const s
     return c;
 }
 
-// The pipelined kernels want enough workgroups of 256 queries to fill the chip twice (or, from 8
-// tiles per workgroup on, half of it once) and address K/V with 32-bit byte offsets.
-bool long_variant(const std::shared_ptr<Device> &dev, int64_t b, int64_t h, int64_t n, int64_t d)
+// The software-pipelined kernels serve every launch without an additive mask whose K/V they can address
+// with 32-bit byte offsets ...
+bool long_variant(int64_t n, int64_t d)
 {
-    const int64_t cus = dev->compute_units(), wgs = b * h * ((n + 255) / 256);
-    return (wgs >= 2 * cus || (n >= 512 && 2 * wgs >= cus)) && (n + 320) * d * 2 < ((int64_t)1 << 31);
+    return (n + 320) * d * 2 < ((int64_t)1 << 31);
 }
 
 // ... and run with 4 waves / 128 queries per workgroup (the `_mid` entry points, two workgroups per compute
@@ -442,13 +441,10 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
         return calls;
     }
     if (kern == Kernel::FlashBf16) {
-        if (!has_mask && !key_lengths && n <= 256 && b * h * ((n + 127) / 128) <= 4 * (int64_t)dev->compute_units())
-            calls.push_back(make_call(dev, "ar_flash_bf16_short", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
-                                      {(n + 127) / 128, b * h, 1}, {512, 1, 1}, vals));
-        else if (!has_mask && long_variant(dev, b, h, n, d) && mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr))
+        if (!has_mask && long_variant(n, d) && mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr))
             calls.push_back(attn_call("ar_flash_bf16_mid", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 127) / 128, b * h, 1}, {256, 1, 1}, vals));
-        else if (!has_mask && long_variant(dev, b, h, n, d))
+        else if (!has_mask && long_variant(n, d))
             calls.push_back(attn_call("ar_flash_bf16_long", {q, k, v, out, mslot}, {BF, BF, BF, BF, F},
                                       {(n + 255) / 256, b * h, 1}, {512, 1, 1}, vals));
         else
@@ -503,11 +499,11 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     int shift = 0;
     while (((int64_t)64 << shift) < bk) ++shift;
     const bool tile_uniform = ((int64_t)64 << shift) == bk;
-    if (!has_mask && tile_uniform && long_variant(dev, b, h, n, d)) {
+    if (!has_mask && tile_uniform && long_variant(n, d)) {
         svals.push_back(bf16_in ? 0 : 1);  // out_f32
-        if (!st.sage_fp8 && mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr))
-            calls.push_back(attn_call("ar_flash_sage_mid", {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, X, F, F, F},
-                                      {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
+        if (mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr))
+            calls.push_back(attn_call(st.sage_fp8 ? "ar_flash_sage_fp8_mid" : "ar_flash_sage_mid", {q8, k8, vb, out, mslot, sq, sk},
+                                      {I8, I8, BF, X, F, F, F}, {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
         else
             calls.push_back(attn_call(st.sage_fp8 ? "ar_flash_sage_fp8_long" : "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk},
                                       {I8, I8, BF, X, F, F, F}, {(n + 255) / 256, b * h, 1}, {512, 1, 1}, svals));

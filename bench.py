@@ -169,13 +169,13 @@ class FlashWorkload:
         peak = PEAK_BF16 if self.dt == BF16 else PEAK_F32
         if ai > peak * 1e12 / (PEAK_HBM * 1e9):
             ach = self.ops / secs / 1e12
-            kern = "flash_f32_kernel" if self.dt != BF16 else ("attn_pipe_kernel<bf16>" if self.S > 256 else "attn_fwd_kernel<bf16>")
+            kern = "flash_f32_kernel" if self.dt != BF16 else "attn_pipe_kernel<bf16>"
             return {"bound": "mfma", "achieved": ach, "peak": peak, "unit": "TFLOP/s", "frac": ach / peak,
                     "traffic": None, "kernel": kern, "launch_ms": secs * 1e3, "ops_per_launch": self.ops,
                     "peak_note": "dense %s MFMA" % self.dtype}
         ach = self.kernel_bytes / secs / 1e9
         return {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM, "unit": "GB/s", "frac": ach / PEAK_HBM,
-                "traffic": None, "kernel": "attn_fwd_kernel<bf16>" if self.dt == BF16 else "flash_f32_kernel",
+                "traffic": None, "kernel": "attn_pipe_kernel<bf16>" if self.dt == BF16 else "flash_f32_kernel",
                 "launch_ms": secs * 1e3, "bytes_per_launch": self.kernel_bytes,
                 "tflops": self.ops / secs / 1e12}
 

@@ -58,14 +58,10 @@
 /* the software-pipelined variant for long sequences: same arguments, has_mask must be 0,
  * (N + 320) * head_dim * 2 < 2^31; long tiling. */
 #define ARHIP_KERNEL_FLASH_BF16_LONG "ar_flash_bf16_long"
-/* the same kernel with 4 waves and 128 queries per workgroup (mid tiling), for launches whose workgroups
- * see few tiles (n <= 2048, or fewer than two 256-query workgroups per compute unit): same arguments and
- * limits as ar_flash_bf16_long. */
+/* the same kernel with 4 waves and 128 queries per workgroup (mid tiling, two workgroups per compute unit),
+ * for launches whose workgroups see few tiles, down to the shortest sequences: same arguments and limits as
+ * ar_flash_bf16_long. */
 #define ARHIP_KERNEL_FLASH_BF16_MID "ar_flash_bf16_mid"
-/* the variant for sequences of at most 256 keys (all of K/V of a head in LDS at once): same
- * arguments, has_mask must be 0, N <= 256; block [512,1,1], grid [ceil(N/128), B*hq, 1]. */
-#define ARHIP_KERNEL_FLASH_BF16_SHORT "ar_flash_bf16_short"
-
 /* Sage int8: replaces `ar_flash_sage`, src/runtime/cuda_flash_sage.rs:168-414, on pre-quantised
  * operands (the quantiser is the pre-pass below):
  * (const int8 *Q8, *K8, const bf16 *V, float *O, const float *M, const float *SQ, const float *SK,
@@ -110,7 +106,7 @@
  * and the same scalars, grid and block.
  *   ar_flash_f32_lens, ar_flash_bf16_lens, ar_flash_bf16_long_lens, ar_flash_bf16_mid_lens   (Q, K, V, O, M, L, 6 ints)
  *   ar_flash_sage_lens, ar_flash_sage_fp8_lens                           (Q8, K8, V, O, M, L, SQ, SK, 6 ints, bq, bk)
- *   ar_flash_sage_long_lens, ar_flash_sage_mid_lens, ar_flash_sage_fp8_long_lens   (..., bq, bk, out_f32) */
+ *   ar_flash_sage_long_lens, ar_flash_sage_mid_lens, ar_flash_sage_fp8_long_lens, ar_flash_sage_fp8_mid_lens   (..., bq, bk, out_f32) */
 #define ARHIP_KERNEL_FLASH_F32_LENS "ar_flash_f32_lens"
 #define ARHIP_KERNEL_FLASH_BF16_LENS "ar_flash_bf16_lens"
 #define ARHIP_KERNEL_FLASH_BF16_LONG_LENS "ar_flash_bf16_long_lens"
@@ -120,12 +116,14 @@
 #define ARHIP_KERNEL_FLASH_SAGE_MID_LENS "ar_flash_sage_mid_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_FP8_LENS "ar_flash_sage_fp8_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_FP8_LONG_LENS "ar_flash_sage_fp8_long_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_MID_LENS "ar_flash_sage_fp8_mid_lens"
 
 /* FP8 E4M3 variant (the reference's `src(fp8 = true)`, src/runtime/cuda_flash_sage.rs:82-84, 92-147):
  * the same argument lists as ar_flash_sage / ar_sage_quant_{blocks,rows}_*, with E4M3 codes
  * (scale = absmax / 448) in place of int8 values. */
 #define ARHIP_KERNEL_FLASH_SAGE_FP8 "ar_flash_sage_fp8"
 #define ARHIP_KERNEL_FLASH_SAGE_FP8_LONG "ar_flash_sage_fp8_long"   /* as ar_flash_sage_long */
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_MID "ar_flash_sage_fp8_mid"     /* as ar_flash_sage_mid */
 #define ARHIP_KERNEL_SAGE_QUANT_BLOCKS_FP8_F32 "ar_sage_quant_blocks_fp8_f32"
 #define ARHIP_KERNEL_SAGE_QUANT_BLOCKS_FP8_BF16 "ar_sage_quant_blocks_fp8_bf16"
 #define ARHIP_KERNEL_SAGE_QUANT_ROWS_FP8_F32 "ar_sage_quant_rows_fp8_f32"

@@ -17,14 +17,14 @@
 //! | `ar_flash_sage`      | 256   | `[ceil(n/128), b*h, 1]` | same `+ bq, bk`; buffers `+ SQ, SK`; O is f32|
 //! | `ar_flash_sage_long` | 512   | `[ceil(n/256), b*h, 1]` | same `+ bq, bk, out_f32`                     |
 //! | `ar_flash_sage_mid`  | 256   | `[ceil(n/128), b*h, 1]` | same; the pipelined kernel with 4 waves      |
-//! | `ar_flash_sage_fp8`, `ar_flash_sage_fp8_long` | as the int8 pair, on E4M3 codes (`SageOptions::fp8`)        |
+//! | `ar_flash_sage_fp8`, `ar_flash_sage_fp8_long`, `ar_flash_sage_fp8_mid` | as the int8 entries, on E4M3 codes (`SageOptions::fp8`) |
 //! | `<entry>_lens`       | as `<entry>` | as `<entry>`     | one more buffer after the mask slot: `L`, int32 `[b]` key lengths |
 //!
 //! Key-padding masks: the CUDA fused kernels admit a dense `[n, n]` mask only
 //! (`src/models/flash_attention.rs:389-396`); here a per-batch key length keeps a padded batch on the
 //! fused kernels.  Every builder takes `lens: Option<Buffer>`; with `Some`, the `_lens` twin of the
-//! entry is named and the buffer is inserted after the mask slot.  `ar_flash_f32_short` and
-//! `ar_flash_bf16_short` have no twin: the builders fall through to the general entries then.
+//! entry is named and the buffer is inserted after the mask slot.  `ar_flash_f32_short` has no twin: the
+//! builder falls through to `ar_flash_f32_lens` then.
 //!
 //! Unlike the CUDA Sage kernel, which quantises inside the attention kernel (K once per query
 //! block, `cuda_flash_sage.rs:248-278`), the quantiser is a pre-pass of its own here, with K
@@ -147,12 +147,10 @@ fn vals(n: i64, d: i64, h: i64, opts: Options) -> Vec<i64> {
     vec![n, d, opts.causal as i64, opts.has_mask as i64, h, opts.h_kv]
 }
 
-/// The pipelined kernels want enough workgroups of 256 queries to fill the chip twice (or, from 8
-/// tiles per workgroup on, half of it once) and address K/V with 32-bit byte offsets.
-fn long_variant(dev: &str, b: i64, h: i64, n: i64, d: i64) -> bool {
-    let cus = crate::runtime::ops_hip::compute_units(dev);
-    let wgs = b * h * ((n + 255) / 256);
-    (wgs >= 2 * cus || (n >= 512 && 2 * wgs >= cus)) && (n + 320) * d * 2 < 1 << 31
+/// The software-pipelined kernels serve every launch without an additive mask whose K/V they can address
+/// with 32-bit byte offsets ...
+fn long_variant(n: i64, d: i64) -> bool {
+    (n + 320) * d * 2 < 1 << 31
 }
 
 /// ... and run with 4 waves / 128 queries per workgroup (`_mid`: two workgroups per compute unit, one's
@@ -186,12 +184,9 @@ pub fn host_call_f32(dev: &str, bufs: Vec<Buffer>, lens: Option<Buffer>, b: i64,
 #[allow(clippy::too_many_arguments)]
 pub fn host_call_bf16(dev: &str, bufs: Vec<Buffer>, lens: Option<Buffer>, b: i64, h: i64, n: i64, d: i64, opts: Options) -> HostCall {
     let (bf, f) = (dtype::BFLOAT16, dtype::FLOAT32);
-    if !opts.has_mask && lens.is_none() && n <= 256 && b * h * ((n + 127) / 128) <= 4 * crate::runtime::ops_hip::compute_units(dev) {
-        // all of K/V of a head in LDS at once: the ViT sequence lengths
-        call("ar_flash_bf16_short", bufs, &[bf, bf, bf, bf, f], [(n + 127) / 128, b * h, 1], [512, 1, 1], vals(n, d, h, opts), &[])
-    } else if !opts.has_mask && long_variant(dev, b, h, n, d) && mid_variant(dev, b, h, n, d, opts.causal, lens.is_some()) {
+    if !opts.has_mask && long_variant(n, d) && mid_variant(dev, b, h, n, d, opts.causal, lens.is_some()) {
         attn_call("ar_flash_bf16_mid", bufs, &[bf, bf, bf, bf, f], lens, [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts))
-    } else if !opts.has_mask && long_variant(dev, b, h, n, d) {
+    } else if !opts.has_mask && long_variant(n, d) {
         attn_call("ar_flash_bf16_long", bufs, &[bf, bf, bf, bf, f], lens, [(n + 255) / 256, b * h, 1], [512, 1, 1], vals(n, d, h, opts))
     } else {
         attn_call("ar_flash_bf16", bufs, &[bf, bf, bf, bf, f], lens, [(n + 127) / 128, b * h, 1], [256, 1, 1], vals(n, d, h, opts))
@@ -280,10 +275,10 @@ pub fn host_calls_sage(
     sv.push(bq);
     sv.push(bk);
     let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
-    if !opts.has_mask && tile_uniform && long_variant(dev, b, h, n, d) {
+    if !opts.has_mask && tile_uniform && long_variant(n, d) {
         sv.push(!bf16_in as i64); // out_f32
-        if !sage.fp8 && mid_variant(dev, b, h, n, d, opts.causal, lens.is_some()) {
-            calls.push(attn_call("ar_flash_sage_mid", vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
+        if mid_variant(dev, b, h, n, d, opts.causal, lens.is_some()) {
+            calls.push(attn_call(if sage.fp8 { "ar_flash_sage_fp8_mid" } else { "ar_flash_sage_mid" }, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
                                  [(n + 127) / 128, b * h, 1], [256, 1, 1], sv));
         } else {
             calls.push(attn_call(long, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,

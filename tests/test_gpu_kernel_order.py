@@ -1,4 +1,4 @@
-"""The attention kernels (pipelined int8, bf16, FP8; short-sequence bf16) against a numpy restatement of THEIR OWN order of operations
+"""The attention kernels (pipelined int8, bf16, FP8) against a numpy restatement of THEIR OWN order of operations
 (autorust_amd/csrc/attn_pipe.h), wave by wave: 32-key blocks in sequence, the biased-float logits
 (12582912 + sum) * c' - m_bias with c' cut to 21 bits, the lazy exponent reference on its grid, the
 rescue path (row maximum, reference moved up to the grid, accumulators rescaled, block redone with
@@ -258,80 +258,3 @@ def test_fp8_pipelined_kernel_matches_its_own_order_of_operations(dev):
                 medians.append(float(np.median(err)))
         # (the first causal rows see few keys: one noisy logit moves them more; measured worst 7e-4)
         assert worst < 2e-3 and max(medians) < 5e-6, (causal, worst, medians)
-
-
-def _wave_short(qb, kb, vb, scale, N, tiles):
-    """The short-sequence bf16 kernel (autorust_amd/csrc/attn_fwd.h, all of K/V in LDS, no causal mask):
-    one wave's state (m, l per lane half, O) after the 64-key tiles `tiles`.  A tile with keys past N
-    takes the general path (rounded products, maximum-based reference, sentinel for the hidden keys)."""
-    D = kb.shape[1]
-    m = np.full(32, SENTINEL, F)
-    l = np.zeros((32, 2), F)
-    o = np.zeros((32, D), F)
-    c = F(F(scale) * LOG2E)
-    for t in tiles:
-        general = 64 * t + 64 > N
-        for blk in (2 * t, 2 * t + 1):
-            kb0 = blk * 32
-            nvis = max(0, min(32, N - kb0))
-            kblk = np.zeros((32, D), F)
-            kblk[:nvis] = kb[kb0:kb0 + nvis]
-            vblk = np.zeros((32, D), np.float64)
-            vblk[:nvis] = vb[kb0:kb0 + nvis]
-            s = (qb.astype(np.float64) @ kblk.astype(np.float64).T).astype(F)
-            hidden = np.broadcast_to(np.arange(kb0, kb0 + 32)[None, :] >= N, (32, 32))
-            if general:
-                x = np.where(hidden, SENTINEL, F(s * c))
-                mx = x.max(axis=1)
-                if np.any(mx > F(m + F(60.0))):
-                    m_new = np.maximum(m, mx)
-                    alpha = _exp2(m - m_new)
-                    m, l, o = m_new, F(l * alpha[:, None]), F(o * alpha[:, None])
-                p = _exp2(F(x - m[:, None]))
-                rs = _row_sums(p)
-            else:
-                p = _exp2(_fl32(s.astype(np.float64) * np.float64(c) - m[:, None].astype(np.float64)))
-                rs = _row_sums(p)
-                if not np.all(rs <= LIMIT):
-                    m_new = np.maximum(m, F(s.max(axis=1) * c))
-                    alpha = _exp2(m - m_new)
-                    m, l, o = m_new, F(l * alpha[:, None]), F(o * alpha[:, None])
-                    p = _exp2(_fl32(s.astype(np.float64) * np.float64(c) - m[:, None].astype(np.float64)))
-                    rs = _row_sums(p)
-            l = F(l + rs)
-            pb = oracle.bf16_round(p).astype(np.float64)
-            for ks in (0, 1):
-                o = (o.astype(np.float64) + pb[:, 16 * ks:16 * ks + 16] @ vblk[16 * ks:16 * ks + 16]).astype(F)
-    return m, l, o
-
-
-def test_bf16_short_sequence_kernel_matches_its_own_order_of_operations(dev):
-    """The ViT-B/16 shape (B8 H12 S197 D64): two waves per 32 queries on the even and the odd key tiles,
-    the last tile on the general path, the two partial results merged, bf16 output."""
-    B, H, N, D = 8, 12, 197, 64
-    q, k, v = synth.normal(741, (B, H, N, D)), synth.normal(742, (B, H, N, D)), synth.normal(743, (B, H, N, D))
-    got_all = run_flash(dev, q, k, v, BF16)
-    qb, kb, vb = oracle.bf16_round(q), oracle.bf16_round(k), oracle.bf16_round(v)
-    scale = F(1.0) / np.sqrt(F(D))
-    same = total = 0
-    for b, h in ((0, 0), (3, 7), (7, 11)):
-        for wave in range(7):
-            rows = np.arange(32 * wave, 32 * wave + 32)
-            rr = np.minimum(rows, N - 1)
-            real = rows < N
-            m0, l0, o0 = _wave_short(qb[b, h, rr], kb[b, h], vb[b, h], scale, N, (0, 2))
-            m1, l1, o1 = _wave_short(qb[b, h, rr], kb[b, h], vb[b, h], scale, N, (1, 3))
-            m = np.maximum(m0, m1)
-            f0, f1 = _exp2(m0 - m), _exp2(m1 - m)
-            l = F(F(l0 * f0[:, None]) + F(l1 * f1[:, None]))
-            o = F(F(o0 * f0[:, None]) + F(o1 * f1[:, None]))
-            l_tot = F(l[:, 0] + l[:, 1])
-            want = F(o * (F(1.0) / l_tot)[:, None])
-            wb = oracle.bf16_round(want)[real]
-            got = got_all[b, h, rr[real]]
-            big = np.maximum(np.maximum(np.abs(got), np.abs(wb)), F(2.0 ** -100)).astype(np.float64)
-            step = np.exp2(np.floor(np.log2(big)) - 7.0)
-            assert np.all(np.abs(got.astype(np.float64) - wb) <= step + 1e-5 + 1e-4 * float(np.abs(want).max()))
-            same += int((got == wb).sum())
-            total += got.size
-    assert same >= 0.99 * total, (same, total)

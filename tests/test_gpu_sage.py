@@ -176,7 +176,10 @@ def test_zero_block_and_outliers(dev):
     assert sq[0, 0, 0] == 1.0 and not q8[0, 0, :128].any()
     assert k8[0, 0, 70, 5] == 127
     want = oracle.sage(q8, k8, sq, sk, v, 128, 64)
-    assert np.abs(r["out"] - want).max() < 4e-3
+    # The outlier makes rows nearly one-hot: the emulation's largest probability is exactly 1, the kernel's
+    # sits anywhere in its exponent window and is rounded to bf16 (2^-9 relative), so the derived bound
+    # 2^-8 max|v| (one rounding of P on each side) is the one that holds here.
+    assert np.abs(r["out"] - want).max() <= 2.0 ** -8 * float(np.abs(v).max())
 
 
 @pytest.mark.parametrize("D", [64, 128])

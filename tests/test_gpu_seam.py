@@ -272,12 +272,15 @@ def test_ar_flash_sage_fp8_by_name(dev, kernels):
     assert np.abs(got - want).max() < 2e-3
 
 
-@pytest.mark.parametrize("d,causal,out_f32", [(128, True, 1), (64, False, 0)])
-def test_ar_flash_sage_fp8_long_by_name(dev, kernels, d, causal, out_f32):
-    """The software-pipelined FP8 entry by name, on codes from the by-name quantiser, against the
-    general FP8 entry on the same codes (both within 2e-3 of the emulation)."""
-    b, hq, hkv, n, bq, bk = 1, 4, 2, 700, 128, 64
+@pytest.mark.parametrize("form,per_wg,block", [("long", 256, 512), ("mid", 128, 256)])
+@pytest.mark.parametrize("d,causal,out_f32,with_lens", [(128, True, 1, False), (64, False, 0, False), (128, False, 1, True)])
+def test_ar_flash_sage_fp8_pipelined_by_name(dev, kernels, form, per_wg, block, d, causal, out_f32, with_lens):
+    """The software-pipelined FP8 entries (8 waves / 256 queries and 4 waves / 128 queries per workgroup,
+    with and without key lengths) by name, on codes from the by-name quantiser, against the general FP8
+    entry on the same codes (both within 2e-3 of the emulation)."""
+    b, hq, hkv, n, bq, bk = 2, 4, 2, 700, 128, 64
     q, k, v = fill_qkv(b, hq, hkv, n, d)
+    lens = np.array([411, n], np.int32) if with_lens else None
     with Bufs(dev) as bufs:
         def quant(x, blk, heads):
             dx, x8 = bufs.put(x), bufs.new(x.size)
@@ -290,34 +293,20 @@ def test_ar_flash_sage_fp8_long_by_name(dev, kernels, d, causal, out_f32):
         k8, sk = quant(k, bk, hkv)
         dv = bufs.put(synth.to_bf16_bits(v))
         do, dg = bufs.new(q.size * 4), bufs.new(q.size * 4)
-        dev.launch(kernels, "ar_flash_sage_fp8_long", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, do, do, sq, sk],
-                   [n, d, int(causal), 0, hq, hkv, bq, bk, out_f32])
-        dev.launch(kernels, "ar_flash_sage_fp8", _grid(n, 128, b, hq), (256, 1, 1), [q8, k8, dv, dg, dg, sq, sk],
+        dl = [bufs.put(lens)] if with_lens else []
+        sfx = "_lens" if with_lens else ""
+        dev.launch(kernels, "ar_flash_sage_fp8_" + form + sfx, _grid(n, per_wg, b, hq), (block, 1, 1),
+                   [q8, k8, dv, do, do] + dl + [sq, sk], [n, d, int(causal), 0, hq, hkv, bq, bk, out_f32])
+        dev.launch(kernels, "ar_flash_sage_fp8" + sfx, _grid(n, 128, b, hq), (256, 1, 1), [q8, k8, dv, dg, dg] + dl + [sq, sk],
                    [n, d, int(causal), 0, hq, hkv, bq, bk])
         got = do.copyout(np.float32, q.shape) if out_f32 else synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
         general = dg.copyout(np.float32, q.shape)
     w_q8, w_sq = oracle.quant_blocks_fp8(q, bq)
     w_k8, w_sk = oracle.quant_blocks_fp8(k, bk)
-    want = oracle.sage_fp8(w_q8, w_k8, w_sq, w_sk, v, bq, bk, causal=causal)
+    want = oracle.sage_fp8(w_q8, w_k8, w_sq, w_sk, v, bq, bk, causal=causal, kv_len=lens)
     tol = 2e-3 if out_f32 else 2e-3 + 2.0 ** -8 * np.abs(want).max()
     assert np.abs(got - want).max() < tol
     assert np.abs(got - general).max() < 2 * tol
-
-
-@pytest.mark.parametrize("n,d,causal,hkv", [(197, 64, False, 6), (256, 128, True, 3), (1, 64, False, 6), (130, 128, False, 1)])
-def test_ar_flash_bf16_short_by_name(dev, kernels, n, d, causal, hkv):
-    """The variant for sequences of at most 256 keys (8 waves, two per 32 queries on the even / odd
-    key tiles), at the ViT length among others."""
-    b, hq = 2, 6
-    q, k, v = fill_qkv(b, hq, hkv, n, d)
-    with Bufs(dev) as bufs:
-        dq, dk, dv = (bufs.put(synth.to_bf16_bits(t)) for t in (q, k, v))
-        do = bufs.new(q.size * 2)
-        dev.launch(kernels, "ar_flash_bf16_short", _grid(n, 128, b, hq), (512, 1, 1), [dq, dk, dv, do, do],
-                   [n, d, int(causal), 0, hq, hkv])
-        got = synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
-    want = oracle.attn_bf16(q, k, v, causal=causal)
-    assert np.abs(got - want).max() < 5e-3
 
 
 # ---- key lengths on the named-kernel seam (the `_lens` twins) --------------------------------------
@@ -427,7 +416,6 @@ def test_named_entries_refuse_launches_they_cannot_run(dev, kernels):
             ("ar_flash_bf16_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, m], [n, d, 0, 1, hq, hq], "no additive mask"),
             ("ar_flash_bf16_long", _grid(n, 256, b, hq), (256, 1, 1), [x, x, x, x, x], ok, r"block \[512,1,1\]"),
             ("ar_flash_bf16_long", _grid(n, 128, b, hq), (512, 1, 1), [x, x, x, x, x], ok, "grid"),
-            ("ar_flash_bf16_short", _grid(n, 128, b, hq), (512, 1, 1), [x, x, x, x, x], ok, "exceeds 256"),
             ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x, x], [n, 96, 0, 0, hq, hq], "head_dim 96"),
             ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x], ok, "takes 5 buffers"),
             ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x, x], [n, d, 0, 0, hq, 3], "hkv"),
@@ -441,7 +429,8 @@ def test_named_entries_refuse_launches_they_cannot_run(dev, kernels):
         dev.launch(kernels, "ar_flash_bf16_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x], ok)
 
 
-@pytest.mark.parametrize("d,causal,n", [(64, False, 700), (128, False, 700), (128, True, 1000), (64, True, 129), (128, False, 64)])
+@pytest.mark.parametrize("d,causal,n", [(64, False, 700), (128, False, 700), (128, True, 1000), (64, True, 129), (128, False, 64),
+                                        (64, False, 197), (128, True, 256), (64, False, 1), (128, False, 130)])
 def test_ar_flash_bf16_mid_by_name(dev, kernels, d, causal, n):
     """The pipelined kernel with 4 waves / 128 queries per workgroup (K ring of two tiles, V ring of
     three): against the oracle, and bit for bit against the 8-wave form."""

@@ -207,17 +207,17 @@ def test_sage_fp8_setting(hdev):
     out = tq.sage_attention_with(tk, tv, None, 0.0, True, sess, st)
     n_calls = sess.end_capture()
     names = [sess.step(i)[0] for i in range(n_calls)]
-    assert names[0] == "ar_sage_quant_blocks_fp8_f32" and "ar_flash_sage_fp8" in names
+    assert names[0] == "ar_sage_quant_blocks_fp8_f32" and "ar_flash_sage_fp8_mid" in names
     assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v, causal=True)).max()) < 6e-2
-    # enough 256-query workgroups: the pipelined FP8 entry, as for int8
-    b, h, n = 2, 32, 1024
+    # enough long 256-query workgroups: the 8-wave pipelined FP8 entry, as for int8
+    b, h, n = 2, 32, 2048
     q, k, v = _fill((b, h, n, d), 3), _fill((b, h, n, d), 11), _fill((b, h, n, d), 19)
     tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape) for a in (q, k, v))
     sess.begin_capture()
     out = tq.sage_attention_with(tk, tv, None, 0.0, False, sess, st)
     n_calls = sess.end_capture()
     assert "ar_flash_sage_fp8_long" in [sess.step(i)[0] for i in range(n_calls)]
-    rows = np.array([0, 255, 256, 777, 1023])
+    rows = np.array([0, 255, 256, 777, 2047])
     assert float(np.abs(out.to_list()[:, :, rows] - oracle.sdpa_f64(q, k, v, rows=rows)).max()) < 6e-2
 
 
@@ -278,9 +278,9 @@ def test_attention_debug_line_and_kernel_info(hdev, capfd, monkeypatch):
 
 
 @gpu
-def test_short_sequences_take_the_short_kernel(hdev):
-    """ViT-B/16's sequence length through the host API: the dispatcher's HostCall names the
-    short-sequence entry (all of K/V of a head in LDS at once)."""
+def test_short_sequences_take_the_pipelined_kernel(hdev):
+    """ViT-B/16's sequence length through the host API: the dispatcher's HostCall names the 4-wave form of
+    the software-pipelined kernel (128 queries per workgroup, two workgroups per compute unit)."""
     b, h, n, d = 2, 12, 197, 64
     q, k, v = (synth.normal(710 + i, (b, h, n, d)) for i in range(3))
     tq, tk, tv = (Tensor.from_slice(hdev, a, a.shape, BFLOAT16) for a in (q, k, v))
@@ -289,7 +289,7 @@ def test_short_sequences_take_the_short_kernel(hdev):
     out = tq.attention_with(tk, tv, None, 0.0, False, sess)
     assert sess.end_capture() == 1
     name, grid, vals = sess.step(0)
-    assert name == "ar_flash_bf16_short" and grid == [2, b * h, 1] and sess.step_detail(0)[1] == [512, 1, 1]
+    assert name == "ar_flash_bf16_mid" and grid == [2, b * h, 1] and sess.step_detail(0)[1] == [256, 1, 1]
     assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v)).max()) < 2e-2
 
 
@@ -324,10 +324,10 @@ def test_capture_and_replay(hdev):
     o2 = tq.sage_attention_with(tk, tv, None, 0.0, True, sess)
     nsteps = sess.end_capture()
     # one launch for flash; for Sage the pre-pass launches (quantise Q, K mean in two steps, quantise
-    # K), the attention kernel and the f32 -> bf16 cast of its output, each a HostCall of its own
+    # K) and the attention kernel, which stores bf16 itself, each a HostCall of its own
     names = [sess.step(i)[0] for i in range(nsteps)]
-    assert names == ["ar_flash_bf16", "ar_sage_quant_blocks_bf16", "ar_sage_kmean_partial_bf16", "ar_sage_kmean_final",
-                     "ar_sage_quant_blocks_bf16", "ar_flash_sage", "ar_cast_bf16"]
+    assert names == ["ar_flash_bf16_mid", "ar_sage_quant_blocks_bf16", "ar_sage_kmean_partial_bf16", "ar_sage_kmean_final",
+                     "ar_sage_quant_blocks_bf16", "ar_flash_sage_mid"]
     name, grid, vals = sess.step(0)
     # grid [query tiles of 128, b*h, 1], vals [n, head_dim, causal, has_mask, hq, hkv] (cuda_flash_bf16.rs:550-599)
     assert grid == [(n + 127) // 128, b * h, 1] and vals == [n, d, 1, 0, h, h]
@@ -335,7 +335,7 @@ def test_capture_and_replay(hdev):
     assert src.endswith("attn_kernels.hsaco") and local == [256, 1, 1] and (nbufs, nvals) == (5, 6)
     BF, F, I32 = 1, 0, 4
     assert sig == [(0, BF), (1, BF), (2, BF), (3, BF), (4, F)] + [(5 + i, I32) for i in range(6)]   # cuda_flash_bf16.rs:563-578
-    assert sess.step(5)[2] == [n, d, 1, 0, h, h] and sess.step_detail(5)[2:4] == (7, 8)
+    assert sess.step(5)[2] == [n, d, 1, 0, h, h] and sess.step_detail(5)[2:4] == (7, 9)   # the six common scalars; then bq, bk, out_f32
     first = out.to_list().copy()
     first2 = o2.to_list().copy()
     allocs = hdev.raw_allocs
@@ -364,11 +364,9 @@ def test_key_lengths_through_the_tensor_api(hdev, api, dtype):
     sess.begin_capture()
     out = getattr(tq, api)(tk, tv, None, 0.0, True, sess, None, tl)
     nsteps = sess.end_capture()
-    name, grid, vals = sess.step(nsteps - 1)
-    if api == "sage_attention_with" and dtype == BFLOAT16:
-        name, grid, vals = sess.step(nsteps - 2)      # the general int8 kernel stores f32; a cast follows
-    assert name.endswith("_lens"), name
-    src, local, nbufs, nvals, sig = sess.step_detail(nsteps - (2 if (api == "sage_attention_with" and dtype == BFLOAT16) else 1))
+    at = [i for i in range(nsteps) if sess.step(i)[0].startswith("ar_fl")]     # the attention kernel among the pre-passes
+    assert len(at) == 1 and sess.step(at[0])[0].endswith("_lens"), [sess.step(i)[0] for i in range(nsteps)]
+    src, local, nbufs, nvals, sig = sess.step_detail(at[0])
     assert sig[5][1] == 4                                # DType::Int32 in the slot after the mask
     got = out.to_list()
     if api == "sage_attention_with":
@@ -376,7 +374,8 @@ def test_key_lengths_through_the_tensor_api(hdev, api, dtype):
         q8, sq = oracle.quant_blocks(qr, 128)
         k8, sk = oracle.quant_blocks(kr, 64, sub=oracle.k_mean(kr))
         want = oracle.sage(q8, k8, sq, sk, v, 128, 64, causal=True, kv_len=lens, round_out=dtype == BFLOAT16)
-        assert np.abs(got - want).max() <= (2.0 ** -6 if dtype == BFLOAT16 else 4e-3)
+        # P is rounded to bf16 on both sides (2^-9 relative each), at different rounding points
+        assert np.abs(got - want).max() <= (2.0 ** -6 if dtype == BFLOAT16 else 2.0 ** -8 * float(np.abs(v).max()))
     elif dtype == BFLOAT16:
         assert np.abs(got - oracle.attn_bf16(q, k, v, causal=True, kv_len=lens)).max() <= 2.0 ** -6
     else:
