@@ -229,6 +229,16 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     const int v_c = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
     const int v_addr[2] = {v_r0 * 64 + (v_c ^ h) * 16 + (lane & 1) * 8,
                            (v_r0 + 8) * 64 + (v_c ^ (h + 2)) * 16 + (lane & 1) * 8};
+    // The offset field of an LDS read has 16 bits and the four stages of the 8-wave form span 96 KB: where the
+    // stage of a tile is a compile-time constant (the four-tiles-per-trip loop), reads of stages 2 and 3 go
+    // through a second set of address registers that already contain 2 STAGE, so that what is left fits the
+    // field and no read needs an address computation of its own: 10 vector instructions fewer per tile, Sage
+    // B4 H32 S8192 -2 %.  (The compiler would rebuild a register it can derive from the first set, hence the
+    // empty assembly.)
+    constexpr int HI_BASE = 2 * STAGE;
+    int k_addr_hi[2] = {k_addr[0] + HI_BASE, k_addr[1] + HI_BASE};
+    int v_addr_hi[2] = {v_addr[0] + HI_BASE, v_addr[1] + HI_BASE};
+    asm("" : "+v"(k_addr_hi[0]), "+v"(k_addr_hi[1]), "+v"(v_addr_hi[0]), "+v"(v_addr_hi[1]));
 
     typedef typename std::conditional<MODE == MODE_I8, i32x16, f32x16>::type acc_t;
     f32x16 oacc[DB];
@@ -509,10 +519,14 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     constexpr int SM_SPLIT = (MODE != MODE_BF16) ? (SM_OPS * R2_SLOTS) / (R2_SLOTS + KSTEPS) : SM_HALF;
     // mc / mn: block j / block j+1 has masked keys (causal diagonal, key-length edge); rel_cur /
     // rel_next are their mask offsets (see lim4h).  sc and sk point at K tiles, sv at a V tile.
+    // chi / vhi / khi: the pointer sc / sv / sk is short of its tile by HI_BASE and the read adds it back through
+    // the second set of address registers.
     auto pipe_block = [&](auto mc, auto mn, acc_t &s_old, acc_t &s_new, uint4 (&p_cur)[2], uint4 (&p_nxt)[2],
                           const unsigned char *sc, int cb,
                           const unsigned char *sv, int vb, const unsigned char *sk, int kb, float c_cur, float c_next,
-                          int rel_cur, int rel_next) __attribute__((always_inline)) {
+                          int rel_cur, int rel_next, auto chi, auto vhi, auto khi) __attribute__((always_inline)) {
+        const int *ka = decltype(khi)::value ? k_addr_hi : k_addr;
+        const int *va = decltype(vhi)::value ? v_addr_hi : v_addr;
         // ---- R1 ----
         s_new = s_init;
         ARHIP_FENCE();
@@ -526,16 +540,17 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             // refill behind the MFMA that read the fragment (FP8: behind the odd step, both halves)
             if constexpr (MODE == MODE_FP8) {
                 if constexpr (st % 2 == 1) {
-                    kf[st - 1] = *(const uint4 *)(sk + k_addr[(st - 1) & 1] + ((st - 1) >> 1) * 4096 + kb * 2048);
-                    kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
+                    kf[st - 1] = *(const uint4 *)(sk + ka[(st - 1) & 1] + ((st - 1) >> 1) * 4096 + kb * 2048);
+                    kf[st] = *(const uint4 *)(sk + ka[st & 1] + (st >> 1) * 4096 + kb * 2048);
                 }
             } else {
-                kf[st] = *(const uint4 *)(sk + k_addr[st & 1] + (st >> 1) * 4096 + kb * 2048);
+                kf[st] = *(const uint4 *)(sk + ka[st & 1] + (st >> 1) * 4096 + kb * 2048);
             }
             ARHIP_FENCE();
         });
         rs = sm_half[0] + sm_half[1];
-        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0)) fix_reference(mc, sc, cb, s_old, c_cur, rel_cur, p_cur, rs);
+        if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0))
+            fix_reference(mc, sc + (decltype(chi)::value ? HI_BASE : 0), cb, s_old, c_cur, rel_cur, p_cur, rs);
         l_run += rs;
         set_bias(c_next);  // the reference is final for block j+1 from here to the end of its softmax
         ARHIP_FENCE();
@@ -554,8 +569,8 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             if constexpr (ks == 1) {
 #pragma unroll
                 for (int k2 = 0; k2 < 2; ++k2) {
-                    vf[db][k2][0] = lds_read_tr16(sv + v_addr[0] + db * 4096 + (vb * 2 + k2) * 1024);
-                    vf[db][k2][1] = lds_read_tr16(sv + v_addr[1] + db * 4096 + (vb * 2 + k2) * 1024);
+                    vf[db][k2][0] = lds_read_tr16(sv + va[0] + db * 4096 + (vb * 2 + k2) * 1024);
+                    vf[db][k2][1] = lds_read_tr16(sv + va[1] + db * 4096 + (vb * 2 + k2) * 1024);
                 }
             }
             ARHIP_FENCE();
@@ -634,9 +649,16 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
 
     // one tile: its two blocks; m0 / m1 / m2 say whether the first block, the second block and the
     // first block of the next tile have masked keys
-    auto tile_iter = [&](auto m0, auto m1, auto m2, int it) __attribute__((always_inline)) {
-        const unsigned char *k_cur = lds + k_base(it), *k_nxt = lds + k_base(it + 1);
-        const unsigned char *v_cur = lds + v_base(it), *v_nxt = lds + v_base(it + 1);
+    // stg: the stage of tile `it` where the caller knows it at compile time (it % 4), else -1
+    auto tile_iter = [&](auto m0, auto m1, auto m2, int it, auto stg) __attribute__((always_inline)) {
+        constexpr int S = decltype(stg)::value, S1 = (S + 1) & 3;
+        constexpr bool cur_hi = S >= 2, nxt_hi = S >= 0 && S1 >= 2;
+        const unsigned char *k_cur = lds + (S >= 0 ? S * STAGE - (cur_hi ? HI_BASE : 0) : k_base(it));
+        const unsigned char *k_nxt = lds + (S >= 0 ? S1 * STAGE - (nxt_hi ? HI_BASE : 0) : k_base(it + 1));
+        const unsigned char *v_cur = lds + (S >= 0 ? S * STAGE + K_TILE - (cur_hi ? HI_BASE : 0) : v_base(it));
+        const unsigned char *v_nxt = lds + (S >= 0 ? S1 * STAGE + K_TILE - (nxt_hi ? HI_BASE : 0) : v_base(it + 1));
+        const std::integral_constant<bool, cur_hi> hc;
+        const std::integral_constant<bool, nxt_hi> hn;
         // tile it + 3 goes to the stage tile it - 1 vacated at the last barrier (RINGS: K(it + 2) to where
         // K(it) was, read for the last time before that barrier, V(it + 2) to where V(it - 1) was)
         issue_tile(it + AHEAD);
@@ -645,8 +667,8 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         const float c_cur = c_carry, c_nxt = tile_c(it + 1, it);
         c_carry = c_nxt;
         const int rel0 = lim4h - it * BK;
-        pipe_block(m0, m1, s_a, s_b, p_a, p_b, k_cur, 0, v_cur, 1, k_nxt, 0, c_cur, c_cur, rel0, rel0 - 32);
-        pipe_block(m1, m2, s_b, s_a, p_b, p_a, k_cur, 1, v_nxt, 0, k_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64);
+        pipe_block(m0, m1, s_a, s_b, p_a, p_b, k_cur, 0, v_cur, 1, k_nxt, 0, c_cur, c_cur, rel0, rel0 - 32, hc, hc, hn);
+        pipe_block(m1, m2, s_b, s_a, p_b, p_a, k_cur, 1, v_nxt, 0, k_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64, hc, hn, hn);
         wait_vmem_le<RINGS ? 0 : XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
         __syncthreads();
     };
@@ -655,26 +677,27 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     if constexpr (RINGS) __syncthreads();
     // the last unmasked tile hands a masked block to the look-ahead: it is peeled off
     const int nplain = (nfull < ntiles) ? max(nfull - 1, 0) : nfull;
-    // 8-bit operands: four tiles per trip, so that the stage of a tile (it % 4) and with it every LDS
-    // offset and transfer destination is a constant (15 vector and 23 scalar instructions fewer per
-    // tile: Sage B4 H32 S8192 3.05 -> 2.96 ms).  The bf16 loop body is larger and gains nothing from it.
-    const int nplain4 = (MODE != MODE_BF16 && !RINGS) ? (nplain & ~3) : 0;
+    // Four tiles per trip, so that the stage of a tile (it % 4) and with it every LDS offset and transfer
+    // destination is a constant (int8: 15 vector and 23 scalar instructions fewer per tile, Sage B4 H32 S8192
+    // 3.05 -> 2.96 ms; bf16, once no offset needs a register of its own: S8192 -1.8 %).
+    const int nplain4 = !RINGS ? (nplain & ~3) : 0;
 #pragma clang loop unroll(disable)
     for (int it = 0; it < nplain4; it += 4) {
-        tile_iter(PLAIN, PLAIN, PLAIN, it);
-        tile_iter(PLAIN, PLAIN, PLAIN, it + 1);
-        tile_iter(PLAIN, PLAIN, PLAIN, it + 2);
-        tile_iter(PLAIN, PLAIN, PLAIN, it + 3);
+        tile_iter(PLAIN, PLAIN, PLAIN, it, std::integral_constant<int, 0>());
+        tile_iter(PLAIN, PLAIN, PLAIN, it + 1, std::integral_constant<int, 1>());
+        tile_iter(PLAIN, PLAIN, PLAIN, it + 2, std::integral_constant<int, 2>());
+        tile_iter(PLAIN, PLAIN, PLAIN, it + 3, std::integral_constant<int, 3>());
     }
+    const std::integral_constant<int, -1> any_stage;
 #pragma clang loop unroll(disable)
-    for (int it = nplain4; it < nplain; ++it) tile_iter(PLAIN, PLAIN, PLAIN, it);
-    if (nplain < nfull) tile_iter(PLAIN, PLAIN, MASKED, nplain);
+    for (int it = nplain4; it < nplain; ++it) tile_iter(PLAIN, PLAIN, PLAIN, it, any_stage);
+    if (nplain < nfull) tile_iter(PLAIN, PLAIN, MASKED, nplain, any_stage);
     // under the causal mask a wave is done once the tiles start past its last query; it keeps
     // feeding the transfers and the barriers the other waves rely on
     const int my_tiles = CAUSAL ? min(ntiles, (wq0 + 31) / BK + 1) : ntiles;
     // (two loops rather than a branch inside one: the accumulators would be copied at the join)
 #pragma clang loop unroll(disable)
-    for (int it = nfull; it < my_tiles; ++it) tile_iter(MASKED, MASKED, MASKED, it);
+    for (int it = nfull; it < my_tiles; ++it) tile_iter(MASKED, MASKED, MASKED, it, any_stage);
 #pragma clang loop unroll(disable)
     for (int it = max(nfull, my_tiles); it < ntiles; ++it) {
         issue_tile(it + AHEAD);
