@@ -453,26 +453,37 @@ __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const 
                                                       int head_dim, int causal, int has_mask, int hq, int hkv, int bq, int bk,
                                                       int out_f32)
 {
-    int shift = 0;
+    int shift = 0, key_shift = 0;
     while ((64 << shift) < bk) ++shift;
-    if (has_mask || (64 << shift) != bk) return;  // the general kernels cover those
+    while ((1 << key_shift) < bk) ++key_shift;
+    // int8: K scales over a power of two of keys below 64 take the per-key form
+    const bool keys = QMODE == MODE_I8 && bk < 64 && (1 << key_shift) == bk;
+    if (has_mask || ((64 << shift) != bk && !keys)) return;  // the general kernels cover those
     AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, 0, hq, hkv, L);
     p.sq = SQ; p.sk = SK;
     p.bq = bq; p.bk = bk;
     p.bk_tile_shift = shift;
+    p.bk_key_shift = keys ? key_shift : -1;
     const int wg = linear_wg();
-#define AR_SAGE_LONG(DD)                                                                  \
+#define AR_SAGE_LONG(DD, PK)                                                              \
     do {                                                                                  \
         if (out_f32) {                                                                    \
-            if (causal) attn_pipe_body<DD, true, QMODE, true, NW>(p, lds, wg);            \
-            else attn_pipe_body<DD, false, QMODE, true, NW>(p, lds, wg);                  \
+            if (causal) attn_pipe_body<DD, true, QMODE, true, NW, PK>(p, lds, wg);        \
+            else attn_pipe_body<DD, false, QMODE, true, NW, PK>(p, lds, wg);              \
         } else {                                                                          \
-            if (causal) attn_pipe_body<DD, true, QMODE, false, NW>(p, lds, wg);           \
-            else attn_pipe_body<DD, false, QMODE, false, NW>(p, lds, wg);                 \
+            if (causal) attn_pipe_body<DD, true, QMODE, false, NW, PK>(p, lds, wg);       \
+            else attn_pipe_body<DD, false, QMODE, false, NW, PK>(p, lds, wg);             \
         }                                                                                 \
     } while (0)
-    if (head_dim == 64) AR_SAGE_LONG(64);
-    else if (head_dim == 128) AR_SAGE_LONG(128);
+    if constexpr (QMODE == MODE_I8) {
+        if (keys) {
+            if (head_dim == 64) AR_SAGE_LONG(64, true);
+            else if (head_dim == 128) AR_SAGE_LONG(128, true);
+            return;
+        }
+    }
+    if (head_dim == 64) AR_SAGE_LONG(64, false);
+    else if (head_dim == 128) AR_SAGE_LONG(128, false);
 #undef AR_SAGE_LONG
 }
 
@@ -481,7 +492,7 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_
                                                                       int N, int head_dim, int causal, int has_mask, int hq,
                                                                       int hkv, int bq, int bk, int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8>()];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 8, true>()];
     flash_sage_long_entry<MODE_I8>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
@@ -490,7 +501,7 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long_lens(const 
                                                                            const float *SK, int N, int head_dim, int causal,
                                                                            int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8>()];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 8, true>()];
     flash_sage_long_entry<MODE_I8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
@@ -500,7 +511,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_mid(const int
                                                                         int N, int head_dim, int causal, int has_mask, int hq,
                                                                         int hkv, int bq, int bk, int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4>()];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4, true>()];
     flash_sage_long_entry<MODE_I8, 4>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
@@ -509,7 +520,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_mid_lens(cons
                                                                              const float *SK, int N, int head_dim, int causal,
                                                                              int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4>()];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4, true>()];
     flash_sage_long_entry<MODE_I8, 4>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 

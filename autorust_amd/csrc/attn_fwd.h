@@ -80,6 +80,7 @@ struct AttnParams {
     long vs[3];    // V's own strides (the int8 path reads a dense K8 next to a V that may be strided)
     int bq, bk;
     int bk_tile_shift;  // log2(bk / 64) when the K scales are tile-uniform
+    int bk_key_shift;   // log2(bk) for the pipelined kernel's per-key form (bk a power of two below 64)
     int nq;        // query tiles per head
     int total;     // workgroups
     int lpt;       // causal: order the whole grid longest-tile-first (small grids)

@@ -71,11 +71,14 @@ __device__ __forceinline__ void static_for(F &&f)
 }
 
 // LDS bytes attn_pipe_body needs: [piece][64 rows][64 B] K and V tiles, four stages of both (NW = 8), or a
-// ring of two K tiles and one of three V tiles (NW = 4)
-template <int D, int MODE, int NW = 8>
+// ring of two K tiles and one of three V tiles (NW = 4).  PER_KEY (a scale per key, or per block of fewer than
+// 64 keys): behind the tiles, a ring of four times 64 raw key scales and, per wave, two times 64 pairs of
+// derived factors.
+template <int D, int MODE, int NW = 8, bool PER_KEY = false>
 constexpr int attn_pipe_lds_bytes()
 {
-    return 4096 * ((NW == 8 ? 4 : 2) * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64) + (NW == 8 ? 4 : 3) * (D * 2 / 64));
+    return 4096 * ((NW == 8 ? 4 : 2) * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64) + (NW == 8 ? 4 : 3) * (D * 2 / 64)) +
+           (PER_KEY ? 1024 + NW * 1024 : 0);
 }
 
 // workgroup index -> (batch * heads + head, query tile of 256), as in attn_fwd_kernel
@@ -96,10 +99,11 @@ __device__ __forceinline__ void pipe_work_item(const AttnParams &p, int wg, int 
 
 // The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
 // aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below.
-template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS, int NW = 8>
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS, int NW = 8, bool PER_KEY = false>
 __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
+    static_assert(!PER_KEY || BIAS, "per-key scales ride on the biased int8 accumulators");
     static_assert(NW == 8 || NW == 4, "8 waves (one workgroup per CU) or 4 (two)");
     constexpr bool RINGS = NW == 4;  // K and V in rings of their own, two and three tiles deep
     constexpr int BQ = NW * 32;
@@ -111,7 +115,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     constexpr int STAGE = K_TILE + V_TILE;
     constexpr int NSTAGE = 4;
     constexpr int AHEAD = RINGS ? 2 : 3;          // a tile is requested this many iterations before the one that computes on it
-    constexpr int LDS_BYTES = attn_pipe_lds_bytes<D, MODE, NW>();
+    constexpr int LDS_BYTES = attn_pipe_lds_bytes<D, MODE, NW>();  // the tiles (PER_KEY: the scale areas follow)
+    constexpr int SK_RAW = LDS_BYTES;          // PER_KEY: [4][64] raw scales of the tiles in flight
+    constexpr int SK_OWN = LDS_BYTES + 1024;   // PER_KEY: [wave][2][2][64] factors of the current and the next tile
     constexpr int XFERS = (KP + VP) * 4;          // 1 KB transfers per tile
     constexpr int XPW = (XFERS + NW - 1) / NW;    // at most this many per wave
     constexpr int XPW_MIN = XFERS / NW;           // at least this many per wave
@@ -172,6 +178,12 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     };
     const i32x4 k_rsrc = make_rsrc((const unsigned char *)p.k + kv_off * QK_BYTES, (uint32_t)kend * k_rowb);
     const i32x4 v_rsrc = make_rsrc(p.v + (size_t)b * p.vs[0] + (size_t)kvh * p.vs[1], (uint32_t)kend * v_rowb);
+    // PER_KEY: this head's key scales, one per block of 1 << bk_key_shift keys
+    i32x4 sk_rsrc = k_rsrc;
+    if constexpr (PER_KEY) {
+        const int nkeyb = (N + p.bk - 1) >> p.bk_key_shift;
+        sk_rsrc = make_rsrc(p.sk + (size_t)kv_bh * nkeyb, (uint32_t)nkeyb * 4);
+    }
 
     // transfer x of a tile (x = wave + 8 j): rows 16 g .. 16 g + 15 of piece pc of K (x < 4 KP) or V;
     // lane l fetches row 16 g + l / 4, chunk (l % 4) ^ ((l / 16) % 4) of that piece
@@ -197,6 +209,17 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     auto issue_tile = [&](int tile) __attribute__((always_inline)) {
         const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
         const uint32_t dst_k = lds0 + k_base(tile), dst_v = lds0 + v_base(tile);
+        if constexpr (PER_KEY) {
+            // the scales of the tile's 64 keys, 4 bytes per lane, by one wave; first, so that a wait that leaves
+            // the newest XPW_MIN transfers of a wave in flight covers it as it covers the tile before
+            if (wave == 0) {
+                const uint32_t off = (uint32_t)((tile * BK + lane) >> p.bk_key_shift) * 4;
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, 0 offen lds"
+                             :
+                             : "s"(lds0 + SK_RAW + (RINGS ? tile % 3 : tile & 3) * 256), "v"(off), "s"(sk_rsrc)
+                             : "memory", "m0");
+            }
+        }
 #pragma unroll
         for (int j = 0; j < XPW; ++j) {
             const int x = wave + NW * j;
@@ -269,7 +292,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         asm volatile("" : "+v"(s_init));  // a register block of its own: the matrix instruction's C operand
     }
     float m_bias = NEG_SENTINEL;  // what the pipelined softmax subtracts for the block it works on
-    auto set_bias = [&](float c) __attribute__((always_inline)) { m_bias = BIAS ? __builtin_fmaf(BIAS_F, c, m_run) : m_run; };
+    auto set_bias = [&](float c) __attribute__((always_inline)) {
+        m_bias = (BIAS && !PER_KEY) ? __builtin_fmaf(BIAS_F, c, m_run) : m_run;
+    };
     float m_grid = 1.0f, m_grid_inv = 1.0f;  // set in the prologue (BIAS only)
     // a logit accumulator as a float (before the factor c)
     auto as_logit = [&](const acc_t &a, int r) __attribute__((always_inline)) -> float {
@@ -295,8 +320,12 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     };
     // exponent factor of the keys of tile t (in the group of tile `it` or the next one): scale log2(e),
     // times sq sk for int8 (s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322)
+    // PER_KEY: the keys' own scales are applied per logit (see convert_sk); what is left is the lane's factor
+    const float sq_c = (sq_lane * p.scale) * LOG2E;
     auto tile_c = [&](int t, int it) __attribute__((always_inline)) -> float {
-        if constexpr (MODE != MODE_BF16) {
+        if constexpr (PER_KEY) {
+            return sq_c;
+        } else if constexpr (MODE != MODE_BF16) {
             const int a = __builtin_amdgcn_readlane(__float_as_int(skv_cur), t & 63);
             const int bnext = __builtin_amdgcn_readlane(__float_as_int(skv_nxt), t & 63);
             const float f = __int_as_float(((t >> 6) == (it >> 6)) ? a : bnext);
@@ -311,13 +340,44 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // wait makes the new vector's arrival explicit (once per 64 tiles) so that no wait for it is
     // left at its uses.
     auto advance_sk_group = [&](int it) __attribute__((always_inline)) {
-        if constexpr (MODE != MODE_BF16) {
+        if constexpr (MODE != MODE_BF16 && !PER_KEY) {
             if ((it & 63) == 0 && it > 0) {
                 skv_cur = skv_nxt;
                 skv_nxt = load_sk_group((it >> 6) + 1);
                 wait_vmem_le<0>();
             }
         }
+    };
+
+    // PER_KEY.  A logit is acc sk_j (sq_i scale log2 e) - m.  The accumulator, read as a float, is 12582912 + acc, so
+    //   t = fma(12582912 + acc, ck_j, -12582912 ck_j)    (exactly fl(acc ck_j): ck_j is sk_j cut to 21 bits, so the
+    //                                                      second product is exact and the fma rounds once)
+    //   x = fma(t, sq_c, -m)
+    // costs one instruction per logit more than a per-tile scale, provided ck_j and -12582912 ck_j come from
+    // somewhere: every wave derives them from the raw scales of a tile (lane = key) one tile ahead, into its own
+    // two slots of LDS (no other wave reads them, LDS operations of a wave complete in order: no barrier), and
+    // reads them back four keys at a time in the order its lanes hold the logits.
+    float *const sk_own = (float *)(lds + SK_OWN + wave * 1024);
+    auto convert_sk = [&](int tile) __attribute__((always_inline)) {
+        if constexpr (PER_KEY) {
+            const float raw = *(const float *)(lds + SK_RAW + (RINGS ? tile % 3 : tile & 3) * 256 + lane * 4);
+            const float ck = __uint_as_float((__float_as_uint(raw) + 4u) & ~7u);
+            float *dst = sk_own + (tile & 1) * 128;
+            dst[lane] = ck;
+            dst[64 + lane] = -BIAS_F * ck;
+        }
+    };
+    // factors of block blk of tile t as this lane's registers want them: keys 4 h + 8 G .. + 3 at [8 G], their
+    // negated bias products 64 floats further on
+    auto key_factors = [&](int t, int blk) __attribute__((always_inline)) -> const float * {
+        return PER_KEY ? sk_own + (t & 1) * 128 + blk * 32 + 4 * h : nullptr;
+    };
+    float kc[8], kn[8];  // ck_j and -12582912 ck_j of the half block the softmax list works on next
+    auto load_factors = [&](const float *kp, int G, int part) __attribute__((always_inline)) {
+        // part 0 / 1: ck of group G / G + 1 into kc[0..3] / kc[4..7]; 2 / 3: their bias products into kn likewise
+        const float4 v = *(const float4 *)(kp + (part >= 2 ? 64 : 0) + 8 * (G + (part & 1)));
+        float *d = (part >= 2 ? kn : kc) + 4 * (part & 1);
+        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
     };
 
     uint4 kf[KSTEPS];
@@ -371,7 +431,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         float m_new = fmaxf(m_run, mx);
         // BIAS: up to the next multiple of m_grid (softmax does not depend on the reference; a row
         // with no visible key yet keeps the sentinel)
-        if (BIAS && m_new > -1e29f) m_new = __builtin_ceilf(m_new * m_grid_inv) * m_grid;
+        if (BIAS && !PER_KEY && m_new > -1e29f) m_new = __builtin_ceilf(m_new * m_grid_inv) * m_grid;
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;
         l_run *= alpha;
@@ -383,13 +443,15 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // probabilities of an unmasked block against the current reference, the scale folded into the
     // exponent; row sum over the unrounded values (src/runtime/cuda_flash_bf16.rs:365-377); bf16
     // pack in the B-operand layout.  Done in two halves of 8 keys so that only 8 values are live.
-    auto exp_pack = [&](const acc_t &s, float c, uint4 (&pb)[2], float &rs) __attribute__((always_inline)) {
+    // (PER_KEY: y holds the logits already multiplied by their keys' factors)
+    auto exp_pack = [&](const acc_t &s, const float (&y)[16], float c, uint4 (&pb)[2], float &rs) __attribute__((always_inline)) {
         float half[2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             float x[8];
 #pragma unroll
-            for (int r = 0; r < 8; ++r) x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)s[ks * 8 + r], c, -m_run));
+            for (int r = 0; r < 8; ++r)
+                x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(PER_KEY ? y[ks * 8 + r] : (float)s[ks * 8 + r], c, -m_run));
             half[ks] = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
             pb[ks].x = pack_bf16x2(x[0], x[1]);
             pb[ks].y = pack_bf16x2(x[2], x[3]);
@@ -405,7 +467,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // (RINGS: K of the block is gone from LDS by now; its logits are still in their registers, s_blk, as
     // the matrix instructions left them, i.e. with the bias in the int8 case.)
     auto fix_reference = [&](auto masked, const unsigned char *st, int blk, const acc_t &s_blk, float c, int rel, uint4 (&pb)[2],
-                             float &rs) __attribute__((always_inline)) {
+                             float &rs, const float *kp) __attribute__((always_inline)) {
         constexpr bool M = decltype(masked)::value;
         acc_t s;
         if constexpr (RINGS) {
@@ -429,10 +491,20 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         // max3 is inline assembly, which the compiler leaves out when it pads the distance between a
         // matrix instruction and the first vector read of its result: the scaled copies below are
         // ordinary vector instructions, so the result has landed by the time max3 runs
-        float x[16];
+        float x[16], y[16];
+        if constexpr (PER_KEY) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 f = *(const float4 *)(kp + 8 * g);
+                y[4 * g + 0] = (float)s[4 * g + 0] * f.x;   // the same fl(acc ck) as the pipelined fma
+                y[4 * g + 1] = (float)s[4 * g + 1] * f.y;
+                y[4 * g + 2] = (float)s[4 * g + 2] * f.z;
+                y[4 * g + 3] = (float)s[4 * g + 3] * f.w;
+            }
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            x[r] = (float)s[r] * c;
+            x[r] = (PER_KEY ? y[r] : (float)s[r]) * c;
             if (M && 8 * (r >> 2) + (r & 3) > rel) x[r] = NEG_SENTINEL;
         }
         float mx = max3(x[0], x[1], x[2]);
@@ -459,7 +531,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             }
             rs = half[0] + half[1];
         } else {
-            exp_pack(s, c, pb, rs);
+            exp_pack(s, y, c, pb, rs);
         }
     };
 
@@ -470,31 +542,41 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // The softmax of an unmasked block as a list of single vector instructions, so that they can be
     // dealt out between the matrix instructions by hand.  Per half of 8 keys: [convert (int8 only)]
     // 8 x fma(s, c, -m), 8 x exp2, 7 adds (row sum of the unrounded values), 4 bf16 packs.
+    // PER_KEY: 8 x fma(s, ck, -12582912 ck) first, then 4 LDS reads that refill kc / kn for the NEXT half block
+    // (the second half of this block, or the first half of the next one, whose factors start at kpn), so that
+    // they have the rest of the list to arrive; kp are this block's factors.
     constexpr int SM_CVT = (MODE == MODE_I8 && !BIAS) ? 8 : 0;
-    constexpr int SM_HALF = SM_CVT + 8 + 8 + 7 + 4;
+    constexpr int SM_KEY = PER_KEY ? 12 : 0;
+    constexpr int SM_PRE = SM_CVT + SM_KEY;
+    constexpr int SM_HALF = SM_PRE + 8 + 8 + 7 + 4;
     constexpr int SM_OPS = 2 * SM_HALF;
     float sm_t[8], sm_x[8], sm_a[6], sm_half[2];
-    auto sm_op = [&](auto masked, auto ic, const acc_t &s, float c, int rel, uint4 (&pn)[2]) __attribute__((always_inline)) {
+    auto sm_op = [&](auto masked, auto ic, const acc_t &s, float c, int rel, uint4 (&pn)[2], const float *kp, const float *kpn)
+                     __attribute__((always_inline)) {
         constexpr bool M = decltype(masked)::value;
         constexpr int i = decltype(ic)::value;
         constexpr int ks = i / SM_HALF, k = i % SM_HALF;
         if constexpr (k < SM_CVT) {
             sm_t[k] = (float)s[ks * 8 + k];
-        } else if constexpr (k < SM_CVT + 8) {
-            constexpr int r = k - SM_CVT;
-            sm_t[r] = __builtin_fmaf(SM_CVT ? sm_t[r] : as_logit(s, ks * 8 + r), c, -m_bias);
+        } else if constexpr (PER_KEY && k < 8) {
+            sm_t[k] = __builtin_fmaf(as_logit(s, ks * 8 + k), kc[k], kn[k]);
+        } else if constexpr (PER_KEY && k < SM_KEY) {
+            load_factors(ks == 0 ? kp : kpn, ks == 0 ? 2 : 0, k - 8);
+        } else if constexpr (k < SM_PRE + 8) {
+            constexpr int r = k - SM_PRE;
+            sm_t[r] = __builtin_fmaf((SM_CVT || PER_KEY) ? sm_t[r] : as_logit(s, ks * 8 + r), c, -m_bias);
             // a masked key: exp2 of the sentinel is exactly 0
             if (M && 8 * ((ks * 8 + r) >> 2) + (r & 3) > rel) sm_t[r] = NEG_SENTINEL;
-        } else if constexpr (k < SM_CVT + 16) {
-            constexpr int r = k - SM_CVT - 8;
+        } else if constexpr (k < SM_PRE + 16) {
+            constexpr int r = k - SM_PRE - 8;
             sm_x[r] = __builtin_amdgcn_exp2f(sm_t[r]);
-        } else if constexpr (k < SM_CVT + 23) {
-            constexpr int a = k - SM_CVT - 16;  // ((x0+x1)+(x2+x3)) + ((x4+x5)+(x6+x7))
+        } else if constexpr (k < SM_PRE + 23) {
+            constexpr int a = k - SM_PRE - 16;  // ((x0+x1)+(x2+x3)) + ((x4+x5)+(x6+x7))
             if constexpr (a < 4) sm_a[a] = sm_x[2 * a] + sm_x[2 * a + 1];
             else if constexpr (a < 6) sm_a[a] = sm_a[2 * (a - 4)] + sm_a[2 * (a - 4) + 1];
             else sm_half[ks] = sm_a[4] + sm_a[5];
         } else {
-            constexpr int j = k - SM_CVT - 23;
+            constexpr int j = k - SM_PRE - 23;
             const uint32_t w = pack_bf16x2(sm_x[2 * j], sm_x[2 * j + 1]);
             if constexpr (j == 0) pn[ks].x = w;
             else if constexpr (j == 1) pn[ks].y = w;
@@ -524,7 +606,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     auto pipe_block = [&](auto mc, auto mn, acc_t &s_old, acc_t &s_new, uint4 (&p_cur)[2], uint4 (&p_nxt)[2],
                           const unsigned char *sc, int cb,
                           const unsigned char *sv, int vb, const unsigned char *sk, int kb, float c_cur, float c_next,
-                          int rel_cur, int rel_next, auto chi, auto vhi, auto khi) __attribute__((always_inline)) {
+                          int rel_cur, int rel_next, auto chi, auto vhi, auto khi, const float *kp0, const float *kp1,
+                          const float *kp2) __attribute__((always_inline)) {
+        // kp0 / kp1 / kp2: the key factors of blocks j, j+1, j+2 (PER_KEY)
         const int *ka = decltype(khi)::value ? k_addr_hi : k_addr;
         const int *va = decltype(vhi)::value ? v_addr_hi : v_addr;
         // ---- R1 ----
@@ -536,7 +620,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             qk_step(si, s_new, kf[pv], kf[st], qreg[pv], qreg[st]);
             ARHIP_FENCE();
             constexpr int lo = SM_SPLIT + st * (SM_OPS - SM_SPLIT) / KSTEPS, hi = SM_SPLIT + (st + 1) * (SM_OPS - SM_SPLIT) / KSTEPS;
-            static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mc, ic, s_old, c_cur, rel_cur, p_cur); });
+            static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mc, ic, s_old, c_cur, rel_cur, p_cur, kp0, kp1); });
             // refill behind the MFMA that read the fragment (FP8: behind the odd step, both halves)
             if constexpr (MODE == MODE_FP8) {
                 if constexpr (st % 2 == 1) {
@@ -550,7 +634,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         });
         rs = sm_half[0] + sm_half[1];
         if (__builtin_expect(__any(!(rs <= 16.0f * LAZY_LIMIT)), 0))
-            fix_reference(mc, sc + (decltype(chi)::value ? HI_BASE : 0), cb, s_old, c_cur, rel_cur, p_cur, rs);
+            fix_reference(mc, sc + (decltype(chi)::value ? HI_BASE : 0), cb, s_old, c_cur, rel_cur, p_cur, rs, kp0);
         l_run += rs;
         set_bias(c_next);  // the reference is final for block j+1 from here to the end of its softmax
         ARHIP_FENCE();
@@ -564,7 +648,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             ARHIP_FENCE();
             if constexpr (g >= 2) {
                 constexpr int lo = (g - 2) * SM_SPLIT / R2_SLOTS, hi = (g - 1) * SM_SPLIT / R2_SLOTS;
-                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mn, ic, s_new, c_next, rel_next, p_nxt); });
+                static_for<lo, hi>([&](auto ic) __attribute__((always_inline)) { sm_op(mn, ic, s_new, c_next, rel_next, p_nxt, kp1, kp2); });
             }
             if constexpr (ks == 1) {
 #pragma unroll
@@ -593,14 +677,14 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         for (int s = 0; s < KSTEPS; ++s) qreg[s] = *(const uint4 *)(qb + s * 32 + h * 16);
     }
 
-    if constexpr (MODE != MODE_BF16) {
+    if constexpr (MODE != MODE_BF16 && !PER_KEY) {
         skv_cur = load_sk_group(0);
         skv_nxt = load_sk_group(1);
     }
     // BIAS: the largest Q scale of the workgroup's queries and the largest K scale of the head, read
     // behind the transfers issued above so that their latency is spent under them
     float mq = 0.f, mk = 0.f;
-    if constexpr (BIAS) {
+    if constexpr (BIAS && !PER_KEY) {
         const int nqb = (N + p.bq - 1) / p.bq, nkb = (N + p.bk - 1) / p.bk;
         const int qb0 = qblk / p.bq, qb1 = min(qblk + BQ - 1, N - 1) / p.bq;
         for (int i = qb0 + lane; i <= qb1; i += 64) mq = fmaxf(mq, fabsf(p.sq[(size_t)bh * nqb + i]));
@@ -608,7 +692,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     }
     wait_vmem_le<0>();
     __syncthreads();
-    if constexpr (BIAS) {
+    if constexpr (BIAS && !PER_KEY) {
         // The exponent reference stays on a grid no finer than the unit in the last place of
         // 12582912 c for the largest c = sq sk scale log2(e) the workgroup can meet; every wave reduces
         // the same scales, so the grid is uniform over the workgroup.
@@ -635,16 +719,21 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     constexpr std::false_type PLAIN{};
     constexpr std::true_type MASKED{};
     if (ntiles > 0) {
+        convert_sk(0);
         load_kf(lds + k_base(0), 0);
         s_a = mfma_qk();
         load_kf(lds + k_base(0), 1);
         load_vf(lds + v_base(0), 0);
         const float c0 = tile_c(0, 0);
         set_bias(c0);
+        const float *f0 = key_factors(0, 0), *f1 = key_factors(0, 1);
+        if constexpr (PER_KEY) {
+            static_for<0, 4>([&](auto pi) __attribute__((always_inline)) { load_factors(f0, 0, decltype(pi)::value); });
+        }
         if (nfull > 0)
-            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(PLAIN, ic, s_a, c0, 0, p_a); });
+            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(PLAIN, ic, s_a, c0, 0, p_a, f0, f1); });
         else
-            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(MASKED, ic, s_a, c0, lim4h, p_a); });
+            static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(MASKED, ic, s_a, c0, lim4h, p_a, f0, f1); });
     }
 
     // one tile: its two blocks; m0 / m1 / m2 say whether the first block, the second block and the
@@ -663,12 +752,14 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         // K(it) was, read for the last time before that barrier, V(it + 2) to where V(it - 1) was)
         issue_tile(it + AHEAD);
         advance_sk_group(it);
+        convert_sk(it + 1);  // visible since the barrier that ended the last iteration
+        const float *f00 = key_factors(it, 0), *f01 = key_factors(it, 1), *f10 = key_factors(it + 1, 0), *f11 = key_factors(it + 1, 1);
         // (tile_iter runs on consecutive tiles from 0 on: this tile's factor is last iteration's c_nxt)
         const float c_cur = c_carry, c_nxt = tile_c(it + 1, it);
         c_carry = c_nxt;
         const int rel0 = lim4h - it * BK;
-        pipe_block(m0, m1, s_a, s_b, p_a, p_b, k_cur, 0, v_cur, 1, k_nxt, 0, c_cur, c_cur, rel0, rel0 - 32, hc, hc, hn);
-        pipe_block(m1, m2, s_b, s_a, p_b, p_a, k_cur, 1, v_nxt, 0, k_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64, hc, hn, hn);
+        pipe_block(m0, m1, s_a, s_b, p_a, p_b, k_cur, 0, v_cur, 1, k_nxt, 0, c_cur, c_cur, rel0, rel0 - 32, hc, hc, hn, f00, f01, f10);
+        pipe_block(m1, m2, s_b, s_a, p_b, p_a, k_cur, 1, v_nxt, 0, k_nxt, 1, c_cur, c_nxt, rel0 - 32, rel0 - 64, hc, hn, hn, f01, f10, f11);
         wait_vmem_le<RINGS ? 0 : XPW_MIN>();  // tile it + 2 has landed (tile it + 3 may still be in flight)
         __syncthreads();
     };
@@ -759,17 +850,17 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
 }
 
 // int8 uses the biased accumulators (see s_init); bf16 and FP8 the plain ones.
-template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8>
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false>
 __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
-    attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS), NW>(p, lds, wg_linear);
+    attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS), NW, PER_KEY>(p, lds, wg_linear);
 }
 
-template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8>
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false>
 __global__ void __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) attn_pipe_kernel(const AttnParams p)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<D, MODE, NW>()];
-    attn_pipe_body<D, CAUSAL, MODE, OUT_F32, NW>(p, lds, (int)blockIdx.x);
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<D, MODE, NW, PER_KEY>()];
+    attn_pipe_body<D, CAUSAL, MODE, OUT_F32, NW, PER_KEY>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

@@ -66,12 +66,12 @@ static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bo
 
 // The software-pipelined kernel (no additive mask, tile-uniform K scales): 8 waves per workgroup, or 4
 // (two workgroups per compute unit) where a workgroup sees few tiles.
-template <int D, int MODE, bool OUT_F32, int NW = 8>
+template <int D, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false>
 static void launch_pipe(hipStream_t stream, const AttnParams &p, bool causal)
 {
     const dim3 grid((unsigned)p.total), block(NW * 64);
-    if (causal) hipLaunchKernelGGL((attn_pipe_kernel<D, true, MODE, OUT_F32, NW>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((attn_pipe_kernel<D, false, MODE, OUT_F32, NW>), grid, block, 0, stream, p);
+    if (causal) hipLaunchKernelGGL((attn_pipe_kernel<D, true, MODE, OUT_F32, NW, PER_KEY>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_pipe_kernel<D, false, MODE, OUT_F32, NW, PER_KEY>), grid, block, 0, stream, p);
 }
 
 // Which of the two: 128 queries per workgroup hide a workgroup's prologue and epilogue under its
@@ -306,10 +306,16 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
     while (((int64_t)64 << shift) < bk) ++shift;
     const bool per_key = ((int64_t)64 << shift) != bk;
     p.bk_tile_shift = shift;
-    int nw = pick_waves(dev, B * Hq, N, D, hm || per_key || dbg);
+    // ... in the general kernel; int8 scales over a power of two of keys below 64 (the reference's bk = 1 among
+    // them) have a form of the pipelined kernel that applies them per logit
+    int key_shift = 0;
+    while (((int64_t)1 << key_shift) < bk) ++key_shift;
+    const bool pipe_keys = per_key && !fp8 && ((int64_t)1 << key_shift) == bk;
+    p.bk_key_shift = pipe_keys ? key_shift : -1;
+    int nw = pick_waves(dev, B * Hq, N, D, hm || (per_key && !pipe_keys) || dbg);
     if (nw == 1) nw = 4;
     if (nw == 8 && !pipe_addressable(N, std::max<int64_t>(D, v_strides ? v_strides[2] : D), 2)) nw = 4;
-    const bool pipe = nw == 8 && !per_key && !dbg;
+    const bool pipe = nw == 8 && (!per_key || pipe_keys) && !dbg;
     const bool pipe4 = pipe && pipe_wants_4_waves(dev, B * Hq, N, D, causal != 0, kv_len != nullptr);
     if (pipe4) nw = 4;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
@@ -335,6 +341,11 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
         if (dbg) {                                                                                     \
             if (per_key) SAGE_V(DD, 4, true, true, false);                                             \
             else SAGE_V(DD, 4, false, true, false);                                                    \
+        } else if (pipe && pipe_keys) {                                                                \
+            if (pipe4 && f32o) launch_pipe<DD, MODE_I8, true, 4, true>(dev->stream, p, c);             \
+            else if (pipe4) launch_pipe<DD, MODE_I8, false, 4, true>(dev->stream, p, c);               \
+            else if (f32o) launch_pipe<DD, MODE_I8, true, 8, true>(dev->stream, p, c);                 \
+            else launch_pipe<DD, MODE_I8, false, 8, true>(dev->stream, p, c);                          \
         } else if (per_key) SAGE_V(DD, 4, true, false, true);                                          \
         else if (pipe4 && f32o) launch_pipe<DD, MODE_I8, true, 4>(dev->stream, p, c);                  \
         else if (pipe4) launch_pipe<DD, MODE_I8, false, 4>(dev->stream, p, c);                         \

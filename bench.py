@@ -117,7 +117,7 @@ class SageWorkload:
         ach = self.ops / secs / 1e12
         return {"bound": "mfma", "achieved": ach, "peak": PEAK_INT8, "unit": "TOP/s", "frac": ach / PEAK_INT8,
                 "traffic": MEASURED_TRAFFIC.get(self.name), "traffic_source": "rocprofv3 --pmc profile (profiles/), not this run",
-                "kernel": "attn_fwd_kernel<int8>" if self.bk == 1 else "attn_pipe_kernel<%s>" % self.dtype, "launch_ms": secs * 1e3,
+                "kernel": "attn_pipe_kernel<int8, per-key scales>" if self.bk == 1 else "attn_pipe_kernel<%s>" % self.dtype, "launch_ms": secs * 1e3,
                 "ops_per_launch": self.ops, "peak_note": "dense %s MFMA; half of the ops are bf16 (P.V)" % self.dtype,
                 "frac_of_mixed_int8_bf16_bound": t_min / secs}
 

@@ -56,17 +56,21 @@ def _exp2(t):
         return np.exp2(np.asarray(t, np.float64)).astype(F)
 
 
-def _wave(qw, kk, vb, scale, rows, causal=False, kvl=None, sq_rows=None, sk_tiles=None, grid=None):
+def _wave(qw, kk, vb, scale, rows, causal=False, kvl=None, sq_rows=None, sk_tiles=None, grid=None, sk_keys=None, wg_rows=256):
     """One wave of 32 queries (global indices `rows`, consecutive, first a multiple of 32).
     int8 kernel: qw [32, D] / kk [N, D] int8 with sq_rows [32], sk_tiles [ceil(N/64)] and the workgroup's
     grid.  FP8 kernel (grid None): qw, kk hold the values of the E4M3 codes, fp32 logits, the uncut
-    factor, no bias.  bf16 kernel (sq_rows None): qw, kk hold bf16 values.  vb [N, D] bf16 values."""
+    factor, no bias.  bf16 kernel (sq_rows None): qw, kk hold bf16 values.  vb [N, D] bf16 values.
+    int8 with a scale per key (sk_keys [N], no grid): t = fl(acc ck_j) with ck_j the key's scale cut to 21 bits
+    (the kernel's fma(12582912 + acc, ck_j, -12582912 ck_j) is exactly that), then fma(t, sq scale log2 e, -m);
+    the exponent reference is not kept on a grid.  wg_rows: queries per workgroup (256, or 128 in the 4-wave form)."""
+    per_key = sk_keys is not None
     int8 = sq_rows is not None and grid is not None
     fp8 = sq_rows is not None and grid is None
     N, D = kk.shape
     kvl = N if kvl is None else int(kvl)
-    qblk = (int(rows[0]) // 256) * 256
-    kend = min(kvl, min(N, qblk + 256)) if causal else kvl
+    qblk = (int(rows[0]) // wg_rows) * wg_rows
+    kend = min(kvl, min(N, qblk + wg_rows)) if causal else kvl
     ntiles = (kend + 63) // 64
     nfull = min(kend // 64, qblk // 64) if causal else kend // 64        # tiles without a masked key for any wave
     my_tiles = min(ntiles, (int(rows[0]) + 31) // 64 + 1) if causal else ntiles
@@ -87,7 +91,15 @@ def _wave(qw, kk, vb, scale, rows, causal=False, kvl=None, sq_rows=None, sk_tile
         vblk[:nvis] = vb[kb0:kb0 + nvis]
         masked_tile = (blk // 2) >= nfull
         hidden = keys[None, :] > lim[:, None]                            # [32, 32]
-        if int8:
+        if per_key:
+            acc = qw.astype(np.int64) @ kblk.astype(np.int64).T          # exact
+            ck = np.zeros(32, F)
+            ck[:max(0, min(32, N - kb0))] = _cut21(sk_keys[kb0:kb0 + 32])
+            logit = _fl32(acc.astype(np.float64) * ck.astype(np.float64)[None, :])      # t: one rounding
+            c = F(F(sq_rows * F(scale)) * LOG2E)
+            c64 = c.astype(np.float64)
+            t = _fl32(logit.astype(np.float64) * c64[:, None] - m[:, None].astype(np.float64))
+        elif int8:
             acc = qw.astype(np.int64) @ kblk.astype(np.int64).T          # exact
             c = _cut21(F(F(F(sq_rows * sk_tiles[min(kb0 // 64, len(sk_tiles) - 1)]) * F(scale)) * LOG2E))
             c64 = c.astype(np.float64)
@@ -258,3 +270,33 @@ def test_fp8_pipelined_kernel_matches_its_own_order_of_operations(dev):
                 medians.append(float(np.median(err)))
         # (the first causal rows see few keys: one noisy logit moves them more; measured worst 7e-4)
         assert worst < 2e-3 and max(medians) < 5e-6, (causal, worst, medians)
+
+
+@pytest.mark.parametrize("N", [2048, 1000])
+def test_int8_per_key_pipelined_kernel_matches_its_own_order_of_operations(dev, N):
+    """A scale per query row and per key (the reference's granularity, src/runtime/cuda_flash_sage.rs:209-222):
+    the pipelined kernel's per-key form, 8 waves (N = 2048) and 4 waves (N = 1000, a ragged last tile) per
+    workgroup, causal and not."""
+    B, H, D = 2, 32, 128
+    q, k, v = synth.normal(731, (B, H, N, D)), synth.normal(732, (B, H, N, D)), synth.normal(733, (B, H, N, D))
+    gain = F(2.0) ** np.linspace(-6.0, 4.0, H, dtype=F)
+    q = q * gain[None, :, None, None]
+    k = (k * (F(1.0) + F(3.0) * (synth.uniform(734, N) < 0.1)).astype(F)[None, None, :, None]).astype(F)   # uneven key scales
+    scale = F(1.0) / np.sqrt(F(D))
+    for causal in (False, True):
+        wg_rows = 128 if (N <= 1024 or causal) else 256       # the dispatcher's choice between the two forms at this shape
+        r = run_sage(dev, q, k, v, 1, 1, smooth=True, out_dtype=F32, causal=causal)
+        q8, sq, k8, sk, vb = r["q8"], r["sq"], r["k8"], r["sk"], r["vb"]
+        worst, medians = 0.0, []
+        for b, h in ((0, 0), (0, 13), (1, 22), (1, 31)):
+            for wave in (0, 5, (N - 1) // 32):
+                rows = np.arange(32 * wave, 32 * wave + 32)
+                rr = np.minimum(rows, N - 1)
+                real = rows < N
+                want, moves = _wave(q8[b, h, rr], k8[b, h], vb[b, h], scale, rows, causal=causal,
+                                    sq_rows=sq[b, h, rr], sk_keys=sk[b, h], wg_rows=wg_rows)
+                err = np.abs(r["out"][b, h, rr[real]] - want[real])
+                worst = max(worst, float(err.max()))
+                medians.append(float(np.median(err)))
+                assert moves >= 1
+        assert worst < 1e-4 and max(medians) < 1e-6, (causal, worst, medians)

@@ -363,16 +363,18 @@ def test_sage_lens_entries_by_name(dev, kernels, bq, bk):
         # relative to the final maximum; rows that few keys carry differ by up to 2 * 2^-9 * max|v|
         tol = 2.0 ** -8 * float(np.abs(v).max())
         assert np.abs(got - want).max() < tol
-        if bk == 64:
-            dp = bufs.new(q.size * 4)
-            dev.launch(kernels, "ar_flash_sage_long_lens", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, dp, dp, dl, sq, sk],
+        # the pipelined entries take both granularities: scales uniform over a tile, and (int8) scales over a
+        # power of two of keys below 64, applied per logit
+        dp = bufs.new(q.size * 4)
+        for name, per_wg, block in (("ar_flash_sage_long_lens", 256, 512), ("ar_flash_sage_mid_lens", 128, 256)):
+            dp.zero()
+            dev.launch(kernels, name, _grid(n, per_wg, b, hq), (block, 1, 1), [q8, k8, dv, dp, dp, dl, sq, sk],
                        [n, d, 1, 0, hq, hkv, bq, bk, 1])
-            assert np.abs(dp.copyout(np.float32, q.shape) - want).max() < tol
-        else:
-            # per-key scales are the general kernel's: the pipelined entry refuses them on the host
-            with pytest.raises(_lib.ArhipError, match="bk = 64"):
-                dev.launch(kernels, "ar_flash_sage_long_lens", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, do, do, dl, sq, sk],
-                           [n, d, 1, 0, hq, hkv, bq, bk, 1])
+            assert np.abs(dp.copyout(np.float32, q.shape) - want).max() < tol, name
+        # scales over a number of keys that is no power of two stay with the general kernel
+        with pytest.raises(_lib.ArhipError, match="power of two"):
+            dev.launch(kernels, "ar_flash_sage_long_lens", _grid(n, 256, b, hq), (512, 1, 1), [q8, k8, dv, do, do, dl, sq, sk],
+                       [n, d, 1, 0, hq, hkv, bq, 48, 1])
 
 
 def test_decoder_shape_with_key_lengths_by_name(dev, kernels):
@@ -419,7 +421,8 @@ def test_named_entries_refuse_launches_they_cannot_run(dev, kernels):
             ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x, x], [n, 96, 0, 0, hq, hq], "head_dim 96"),
             ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x], ok, "takes 5 buffers"),
             ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x, x], [n, d, 0, 0, hq, 3], "hkv"),
-            ("ar_flash_sage_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x, x, x], [n, d, 0, 0, hq, hq, 128, 48, 0], "bk = 64"),
+            ("ar_flash_sage_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x, x, x], [n, d, 0, 0, hq, hq, 128, 48, 0], "power of two"),
+            ("ar_flash_sage_fp8_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x, x, x], [n, d, 0, 0, hq, hq, 128, 32, 0], "whole 64-key tiles"),
             ("ar_fl_bwd_dkv_short", _grid(n, 32, b, hq), (256, 1, 1), [x] * 9, [n, 128, 0, 0, hq, hq], "64 only"),
         ]
         for name, grid, block, bufs_, vals, msg in bad:
