@@ -456,8 +456,8 @@ __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const 
     int shift = 0, key_shift = 0;
     while ((64 << shift) < bk) ++shift;
     while ((1 << key_shift) < bk) ++key_shift;
-    // int8: K scales over a power of two of keys below 64 take the per-key form
-    const bool keys = QMODE == MODE_I8 && bk < 64 && (1 << key_shift) == bk;
+    // K scales over a power of two of keys below 64 take the per-key form
+    const bool keys = bk < 64 && (1 << key_shift) == bk;
     if (has_mask || ((64 << shift) != bk && !keys)) return;  // the general kernels cover those
     AttnParams p = dense_params(Q8, K8, V, O, M, N, head_dim, 0, hq, hkv, L);
     p.sq = SQ; p.sk = SK;
@@ -475,12 +475,10 @@ __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const 
             else attn_pipe_body<DD, false, QMODE, false, NW, PK>(p, lds, wg);             \
         }                                                                                 \
     } while (0)
-    if constexpr (QMODE == MODE_I8) {
-        if (keys) {
-            if (head_dim == 64) AR_SAGE_LONG(64, true);
-            else if (head_dim == 128) AR_SAGE_LONG(128, true);
-            return;
-        }
+    if (keys) {
+        if (head_dim == 64) AR_SAGE_LONG(64, true);
+        else if (head_dim == 128) AR_SAGE_LONG(128, true);
+        return;
     }
     if (head_dim == 64) AR_SAGE_LONG(64, false);
     else if (head_dim == 128) AR_SAGE_LONG(128, false);
@@ -529,7 +527,7 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long(const u
                                                                           int N, int head_dim, int causal, int has_mask, int hq,
                                                                           int hkv, int bq, int bk, int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8>()];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 8, true>()];
     flash_sage_long_entry<MODE_FP8>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
@@ -539,7 +537,7 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long_lens(co
                                                                                int has_mask, int hq, int hkv, int bq, int bk,
                                                                                int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8>()];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 8, true>()];
     flash_sage_long_entry<MODE_FP8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
@@ -548,7 +546,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_mid(const
                                                                             int N, int head_dim, int causal, int has_mask, int hq,
                                                                             int hkv, int bq, int bk, int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 4>()];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 4, true>()];
     flash_sage_long_entry<MODE_FP8, 4>(lds, Q8, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
@@ -558,7 +556,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_mid_lens(
                                                                                  int has_mask, int hq, int hkv, int bq, int bk,
                                                                                  int out_f32)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 4>()];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 4, true>()];
     flash_sage_long_entry<MODE_FP8, 4>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 

@@ -103,7 +103,7 @@ template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS, int NW = 8, boo
 __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
-    static_assert(!PER_KEY || BIAS, "per-key scales ride on the biased int8 accumulators");
+    static_assert(!PER_KEY || BIAS || MODE == MODE_FP8, "per-key scales: int8 (on the biased accumulators) and FP8");
     static_assert(NW == 8 || NW == 4, "8 waves (one workgroup per CU) or 4 (two)");
     constexpr bool RINGS = NW == 4;  // K and V in rings of their own, two and three tiles deep
     constexpr int BQ = NW * 32;
@@ -361,10 +361,11 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     auto convert_sk = [&](int tile) __attribute__((always_inline)) {
         if constexpr (PER_KEY) {
             const float raw = *(const float *)(lds + SK_RAW + (RINGS ? tile % 3 : tile & 3) * 256 + lane * 4);
-            const float ck = __uint_as_float((__float_as_uint(raw) + 4u) & ~7u);
+            // (FP8: fp32 accumulators, t = acc sk_j needs neither the cut nor the bias product)
+            const float ck = BIAS ? __uint_as_float((__float_as_uint(raw) + 4u) & ~7u) : raw;
             float *dst = sk_own + (tile & 1) * 128;
             dst[lane] = ck;
-            dst[64 + lane] = -BIAS_F * ck;
+            if constexpr (BIAS) dst[64 + lane] = -BIAS_F * ck;
         }
     };
     // factors of block blk of tile t as this lane's registers want them: keys 4 h + 8 G .. + 3 at [8 G], their
@@ -546,7 +547,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // (the second half of this block, or the first half of the next one, whose factors start at kpn), so that
     // they have the rest of the list to arrive; kp are this block's factors.
     constexpr int SM_CVT = (MODE == MODE_I8 && !BIAS) ? 8 : 0;
-    constexpr int SM_KEY = PER_KEY ? 12 : 0;
+    constexpr int SM_KEY = PER_KEY ? (BIAS ? 12 : 10) : 0;
     constexpr int SM_PRE = SM_CVT + SM_KEY;
     constexpr int SM_HALF = SM_PRE + 8 + 8 + 7 + 4;
     constexpr int SM_OPS = 2 * SM_HALF;
@@ -559,7 +560,8 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         if constexpr (k < SM_CVT) {
             sm_t[k] = (float)s[ks * 8 + k];
         } else if constexpr (PER_KEY && k < 8) {
-            sm_t[k] = __builtin_fmaf(as_logit(s, ks * 8 + k), kc[k], kn[k]);
+            if constexpr (BIAS) sm_t[k] = __builtin_fmaf(as_logit(s, ks * 8 + k), kc[k], kn[k]);
+            else sm_t[k] = (float)s[ks * 8 + k] * kc[k];
         } else if constexpr (PER_KEY && k < SM_KEY) {
             load_factors(ks == 0 ? kp : kpn, ks == 0 ? 2 : 0, k - 8);
         } else if constexpr (k < SM_PRE + 8) {
@@ -728,7 +730,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
         set_bias(c0);
         const float *f0 = key_factors(0, 0), *f1 = key_factors(0, 1);
         if constexpr (PER_KEY) {
-            static_for<0, 4>([&](auto pi) __attribute__((always_inline)) { load_factors(f0, 0, decltype(pi)::value); });
+            static_for<0, SM_KEY - 8>([&](auto pi) __attribute__((always_inline)) { load_factors(f0, 0, decltype(pi)::value); });
         }
         if (nfull > 0)
             static_for<0, SM_SPLIT>([&](auto ic) __attribute__((always_inline)) { sm_op(PLAIN, ic, s_a, c0, 0, p_a, f0, f1); });

@@ -486,12 +486,10 @@ int check_named_entry(const char *name, const unsigned grid[3], const unsigned b
         ARHIP_REQUIRE((n + 320) * d * 2 < ((int64_t)1 << 31), "arhip_launch: %s addresses K/V with 32-bit offsets: (n + 320) * head_dim * 2 "
                       "must stay below 2^31", name);
         if (e->nvals >= 8) {
-            // int8: any power of two (below 64 keys the kernel applies the scales per logit); FP8: whole tiles only
+            // any power of two (below 64 keys the kernel applies the scales per logit)
             const int64_t bk = vals[7];
-            const bool fp8 = strstr(name, "_fp8") != nullptr;
-            ARHIP_REQUIRE((bk & (bk - 1)) == 0 && (bk >= 64 || !fp8),
-                          "arhip_launch: %s needs K scales over %s, got bk = %lld", name,
-                          fp8 ? "whole 64-key tiles (bk = 64 * 2^j)" : "a power of two of keys (bk = 2^j)", (long long)bk);
+            ARHIP_REQUIRE((bk & (bk - 1)) == 0, "arhip_launch: %s needs K scales over a power of two of keys (bk = 2^j), got bk = %lld",
+                          name, (long long)bk);
         }
     }
     return ARHIP_OK;

@@ -306,11 +306,11 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
     while (((int64_t)64 << shift) < bk) ++shift;
     const bool per_key = ((int64_t)64 << shift) != bk;
     p.bk_tile_shift = shift;
-    // ... in the general kernel; int8 scales over a power of two of keys below 64 (the reference's bk = 1 among
-    // them) have a form of the pipelined kernel that applies them per logit
+    // ... in the general kernel; scales over a power of two of keys below 64 (the reference's bk = 1 among them)
+    // have a form of the pipelined kernel that applies them per logit
     int key_shift = 0;
     while (((int64_t)1 << key_shift) < bk) ++key_shift;
-    const bool pipe_keys = per_key && !fp8 && ((int64_t)1 << key_shift) == bk;
+    const bool pipe_keys = per_key && ((int64_t)1 << key_shift) == bk;
     p.bk_key_shift = pipe_keys ? key_shift : -1;
     int nw = pick_waves(dev, B * Hq, N, D, hm || (per_key && !pipe_keys) || dbg);
     if (nw == 1) nw = 4;
@@ -358,17 +358,28 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
         if (f32o) launch_attn<DD, 4, MODE_FP8, PK, true, false, true>(dev->stream, p, c, hm);          \
         else launch_attn<DD, 4, MODE_FP8, PK, false, false, true>(dev->stream, p, c, hm);              \
     } while (0)
-    if (fp8 && pipe4) {
-        if (D == 64) { if (f32o) launch_pipe<64, MODE_FP8, true, 4>(dev->stream, p, c); else launch_pipe<64, MODE_FP8, false, 4>(dev->stream, p, c); }
-        else { if (f32o) launch_pipe<128, MODE_FP8, true, 4>(dev->stream, p, c); else launch_pipe<128, MODE_FP8, false, 4>(dev->stream, p, c); }
-    } else if (fp8 && pipe) {
-        if (D == 64) { if (f32o) launch_pipe<64, MODE_FP8, true>(dev->stream, p, c); else launch_pipe<64, MODE_FP8, false>(dev->stream, p, c); }
-        else { if (f32o) launch_pipe<128, MODE_FP8, true>(dev->stream, p, c); else launch_pipe<128, MODE_FP8, false>(dev->stream, p, c); }
+#define SAGE_FP(DD, NWW, PK)                                                                          \
+    do {                                                                                               \
+        if (f32o) launch_pipe<DD, MODE_FP8, true, NWW, PK>(dev->stream, p, c);                         \
+        else launch_pipe<DD, MODE_FP8, false, NWW, PK>(dev->stream, p, c);                             \
+    } while (0)
+#define SAGE_FPD(NWW, PK)                                                                              \
+    do {                                                                                               \
+        if (D == 64) SAGE_FP(64, NWW, PK);                                                             \
+        else SAGE_FP(128, NWW, PK);                                                                    \
+    } while (0)
+    if (fp8 && pipe) {
+        if (pipe4 && pipe_keys) SAGE_FPD(4, true);
+        else if (pipe4) SAGE_FPD(4, false);
+        else if (pipe_keys) SAGE_FPD(8, true);
+        else SAGE_FPD(8, false);
     } else if (fp8) {
         if (D == 64) { if (per_key) SAGE_F(64, true); else SAGE_F(64, false); }
         else { if (per_key) SAGE_F(128, true); else SAGE_F(128, false); }
     } else if (D == 64) SAGE_D(64);
     else SAGE_D(128);
+#undef SAGE_FPD
+#undef SAGE_FP
 #undef SAGE_F
 #undef SAGE_D
 #undef SAGE_V

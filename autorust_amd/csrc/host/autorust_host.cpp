@@ -499,8 +499,8 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     int shift = 0;
     while (((int64_t)64 << shift) < bk) ++shift;
     const bool tile_uniform = ((int64_t)64 << shift) == bk;
-    // int8: scales over a power of two of keys below 64 (the reference's bk = 1) are applied per logit
-    const bool key_scales = !st.sage_fp8 && bk < 64 && (bk & (bk - 1)) == 0;
+    // scales over a power of two of keys below 64 (the reference's bk = 1) are applied per logit
+    const bool key_scales = bk < 64 && (bk & (bk - 1)) == 0;
     if (!has_mask && (tile_uniform || key_scales) && long_variant(n, d)) {
         svals.push_back(bf16_in ? 0 : 1);  // out_f32
         if (mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr))

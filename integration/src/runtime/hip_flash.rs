@@ -275,8 +275,8 @@ pub fn host_calls_sage(
     sv.push(bq);
     sv.push(bk);
     let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
-    // int8: scales over a power of two of keys below 64 (the CUDA kernel's bk = 1) are applied per logit
-    let key_scales = !sage.fp8 && bk >= 1 && bk < 64 && bk.count_ones() == 1;
+    // scales over a power of two of keys below 64 (the CUDA kernel's bk = 1) are applied per logit
+    let key_scales = bk >= 1 && bk < 64 && bk.count_ones() == 1;
     if !opts.has_mask && (tile_uniform || key_scales) && long_variant(n, d) {
         sv.push(!bf16_in as i64); // out_f32
         if mid_variant(dev, b, h, n, d, opts.causal, lens.is_some()) {

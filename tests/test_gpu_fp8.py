@@ -81,12 +81,13 @@ def test_fp8_attention_matches_emulation(dev, bq, bk, smooth, in_dtype, causal, 
     assert np.abs(out - want).max() < 2e-3
 
 
-@pytest.mark.parametrize("d,bk", [(128, 64), (64, 128)])
+@pytest.mark.parametrize("d,bk", [(128, 64), (64, 128), (128, 1), (64, 16)])
 @pytest.mark.parametrize("causal,use_len", [(False, False), (True, False), (True, True), (False, True)])
 def test_fp8_long_sequence_kernel_matches_emulation(dev, d, bk, causal, use_len):
     """Shapes with enough 256-query workgroups for the software-pipelined kernel, which multiplies
     E4M3 operands 64 at a time (v_mfma_f32_32x32x64_f8f6f4); ragged length, grouped heads, per-batch
-    key lengths.  The same 2e-3 against the emulation as the general kernel, three runs bit-equal."""
+    key lengths; K scales over whole tiles and (bk below 64) applied per logit.  The same 2e-3 against
+    the emulation as the general kernel, three runs bit-equal."""
     b, hq, hkv, n = 2, 16, 8, 1024 + 40
     q, k, v = fill_qkv(b, hq, hkv, n, d)
     k = k + np.float32(0.5) * synth.normal(7, (1, hkv, 1, d))

@@ -422,7 +422,7 @@ def test_named_entries_refuse_launches_they_cannot_run(dev, kernels):
             ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x], ok, "takes 5 buffers"),
             ("ar_flash_bf16", _grid(n, 128, b, hq), (256, 1, 1), [x, x, x, x, x], [n, d, 0, 0, hq, 3], "hkv"),
             ("ar_flash_sage_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x, x, x], [n, d, 0, 0, hq, hq, 128, 48, 0], "power of two"),
-            ("ar_flash_sage_fp8_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x, x, x], [n, d, 0, 0, hq, hq, 128, 32, 0], "whole 64-key tiles"),
+            ("ar_flash_sage_fp8_long", _grid(n, 256, b, hq), (512, 1, 1), [x, x, x, x, x, x, x], [n, d, 0, 0, hq, hq, 128, 24, 0], "power of two"),
             ("ar_fl_bwd_dkv_short", _grid(n, 32, b, hq), (256, 1, 1), [x] * 9, [n, 128, 0, 0, hq, hq], "64 only"),
         ]
         for name, grid, block, bufs_, vals, msg in bad:
