@@ -522,6 +522,77 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_mid_lens(cons
     flash_sage_long_entry<MODE_I8, 4>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
+// ar_flash_sage_qf_long / _mid: the pipelined int8 kernel with the Q quantiser in its prologue.  Q holds bf16
+// values; SQ [b*hq, ceil(n/128)] RECEIVES the scales (bq must be 128); K8 / SK as from the K quantiser with
+// bk = 64 * 2^j.  Same grid and block as ar_flash_sage_long / _mid.
+template <int NW>
+__device__ __forceinline__ void flash_sage_qf_entry(unsigned char *lds, const uint16_t *Q, const void *K8, const uint16_t *V, void *O,
+                                                    const float *M, const int *L, float *SQ, const float *SK, int N, int head_dim,
+                                                    int causal, int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
+{
+    int shift = 0;
+    while ((64 << shift) < bk) ++shift;
+    if (has_mask || (64 << shift) != bk || bq != 128) return;  // refused on the host
+    AttnParams p = dense_params(Q, K8, V, O, M, N, head_dim, 0, hq, hkv, L);
+    p.sk = SK;
+    p.sq_out = SQ;
+    p.bq = bq; p.bk = bk;
+    p.bk_tile_shift = shift;
+    p.bk_key_shift = -1;
+    const int wg = linear_wg();
+#define AR_SAGE_QF(DD)                                                                        \
+    do {                                                                                      \
+        if (out_f32) {                                                                        \
+            if (causal) attn_pipe_body<DD, true, MODE_I8, true, NW, false, true>(p, lds, wg); \
+            else attn_pipe_body<DD, false, MODE_I8, true, NW, false, true>(p, lds, wg);       \
+        } else {                                                                              \
+            if (causal) attn_pipe_body<DD, true, MODE_I8, false, NW, false, true>(p, lds, wg);\
+            else attn_pipe_body<DD, false, MODE_I8, false, NW, false, true>(p, lds, wg);      \
+        }                                                                                     \
+    } while (0)
+    if (head_dim == 64) AR_SAGE_QF(64);
+    else if (head_dim == 128) AR_SAGE_QF(128);
+#undef AR_SAGE_QF
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_qf_long(const uint16_t *Q, const int8_t *K8, const uint16_t *V,
+                                                                         void *O, const float *M, float *SQ, const float *SK,
+                                                                         int N, int head_dim, int causal, int has_mask, int hq,
+                                                                         int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 8, false, true>()];
+    flash_sage_qf_entry<8>(lds, Q, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_qf_long_lens(const uint16_t *Q, const int8_t *K8, const uint16_t *V,
+                                                                              void *O, const float *M, const int *L, float *SQ,
+                                                                              const float *SK, int N, int head_dim, int causal,
+                                                                              int has_mask, int hq, int hkv, int bq, int bk,
+                                                                              int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 8, false, true>()];
+    flash_sage_qf_entry<8>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_qf_mid(const uint16_t *Q, const int8_t *K8, const uint16_t *V,
+                                                                           void *O, const float *M, float *SQ, const float *SK,
+                                                                           int N, int head_dim, int causal, int has_mask, int hq,
+                                                                           int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4, false, true>()];
+    flash_sage_qf_entry<4>(lds, Q, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_qf_mid_lens(const uint16_t *Q, const int8_t *K8, const uint16_t *V,
+                                                                                void *O, const float *M, const int *L, float *SQ,
+                                                                                const float *SK, int N, int head_dim, int causal,
+                                                                                int has_mask, int hq, int hkv, int bq, int bk,
+                                                                                int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4, false, true>()];
+    flash_sage_qf_entry<4>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
 extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
                                                                           void *O, const float *M, const float *SQ, const float *SK,
                                                                           int N, int head_dim, int causal, int has_mask, int hq,

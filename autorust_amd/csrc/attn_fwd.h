@@ -71,6 +71,8 @@ struct AttnParams {
     const float *sq;         // MODE_I8: [B,Hq,ceil(N/bq)]
     const float *sk;         // MODE_I8: [B,Hkv,ceil(N/bk)]
     float *lse;              // optional [B,Hq,N]: log-sum-exp of the scaled, masked logits (natural log)
+    float *sq_out;           // fused Q quantiser: optional [B,Hq,ceil(N/128)] scales it derived
+    int8_t *q8_out;          // fused Q quantiser: optional [B,Hq,N,D] codes it derived
     int32_t *dbg;            // MODE_I8 debug: [32][64] raw logits
     int dbg_bh, dbg_qt, dbg_kt;
     int Hq, Hkv, N;

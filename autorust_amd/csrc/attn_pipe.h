@@ -74,11 +74,12 @@ __device__ __forceinline__ void static_for(F &&f)
 // ring of two K tiles and one of three V tiles (NW = 4).  PER_KEY (a scale per key, or per block of fewer than
 // 64 keys): behind the tiles, a ring of four times 64 raw key scales and, per wave, two times 64 pairs of
 // derived factors.
-template <int D, int MODE, int NW = 8, bool PER_KEY = false>
+// QFUSE (Q arrives as bf16 and is quantised in the prologue): 256 bytes for the exchange of the waves' maxima.
+template <int D, int MODE, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 constexpr int attn_pipe_lds_bytes()
 {
     return 4096 * ((NW == 8 ? 4 : 2) * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64) + (NW == 8 ? 4 : 3) * (D * 2 / 64)) +
-           (PER_KEY ? 1024 + NW * 1024 : 0);
+           (PER_KEY ? 1024 + NW * 1024 : 0) + (QFUSE ? 256 : 0);
 }
 
 // workgroup index -> (batch * heads + head, query tile of 256), as in attn_fwd_kernel
@@ -99,9 +100,14 @@ __device__ __forceinline__ void pipe_work_item(const AttnParams &p, int wg, int 
 
 // The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
 // aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below.
-template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS, int NW = 8, bool PER_KEY = false>
+// QFUSE (int8, Q scales over blocks of 128 queries, K scales over whole tiles): p.q holds bf16 values and the
+// prologue is the quantiser of sage_quant_kernels.h for this workgroup's queries, operation for operation
+// (absmax over the block, scale = absmax / 127 or 1, x8 = clamp(rint(x * (1 / scale)), +-127)), so the result is
+// bit for bit that of quantising first; p.sq_out / p.q8_out, where not null, receive the scales and the codes.
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
+    static_assert(!QFUSE || (BIAS && !PER_KEY), "the fused Q quantiser: int8, K scales over whole tiles");
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
     static_assert(!PER_KEY || BIAS || MODE == MODE_FP8, "per-key scales: int8 (on the biased accumulators) and FP8");
     static_assert(NW == 8 || NW == 4, "8 waves (one workgroup per CU) or 4 (two)");
@@ -118,6 +124,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     constexpr int LDS_BYTES = attn_pipe_lds_bytes<D, MODE, NW>();  // the tiles (PER_KEY: the scale areas follow)
     constexpr int SK_RAW = LDS_BYTES;          // PER_KEY: [4][64] raw scales of the tiles in flight
     constexpr int SK_OWN = LDS_BYTES + 1024;   // PER_KEY: [wave][2][2][64] factors of the current and the next tile
+    constexpr int QF_RED = LDS_BYTES;          // QFUSE: [wave] largest |q| of the wave's 32 queries
     constexpr int XFERS = (KP + VP) * 4;          // 1 KB transfers per tile
     constexpr int XPW = (XFERS + NW - 1) / NW;    // at most this many per wave
     constexpr int XPW_MIN = XFERS / NW;           // at least this many per wave
@@ -303,7 +310,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     };
     float sq_lane = 1.f;
     const int nkb = (MODE != MODE_BF16) ? (N + p.bk - 1) / p.bk : 0;
-    if (MODE != MODE_BF16) {
+    if (MODE != MODE_BF16 && !QFUSE) {
         const int nqb = (N + p.bq - 1) / p.bq;
         sq_lane = p.sq[(size_t)bh * nqb + min(q_row, N - 1) / p.bq];
     }
@@ -672,7 +679,15 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     static_for<0, AHEAD>([&](auto ti) __attribute__((always_inline)) { issue_tile(decltype(ti)::value); });
     // Q operand, resident in registers.  Everything in flight is awaited here once, Q included, so
     // that no wait for a global load is left inside the loops.
-    {
+    uint4 qraw[QFUSE ? KSTEPS : 1][2];  // QFUSE: the 16 bf16 values behind each 16-byte piece of the operand
+    if constexpr (QFUSE) {
+        const uint16_t *qb = (const uint16_t *)p.q + (size_t)b * p.qs[0] + (size_t)head * p.qs[1] + (size_t)min(q_row, N - 1) * p.qs[2];
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            qraw[s][0] = *(const uint4 *)(qb + s * 32 + h * 16);
+            qraw[s][1] = *(const uint4 *)(qb + s * 32 + h * 16 + 8);
+        }
+    } else {
         const unsigned char *qb = (const unsigned char *)p.q +
                                   ((size_t)b * p.qs[0] + (size_t)head * p.qs[1] + (size_t)min(q_row, N - 1) * p.qs[2]) * QK_BYTES;
 #pragma unroll
@@ -689,11 +704,61 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     if constexpr (BIAS && !PER_KEY) {
         const int nqb = (N + p.bq - 1) / p.bq, nkb = (N + p.bk - 1) / p.bk;
         const int qb0 = qblk / p.bq, qb1 = min(qblk + BQ - 1, N - 1) / p.bq;
-        for (int i = qb0 + lane; i <= qb1; i += 64) mq = fmaxf(mq, fabsf(p.sq[(size_t)bh * nqb + i]));
+        if constexpr (!QFUSE)
+            for (int i = qb0 + lane; i <= qb1; i += 64) mq = fmaxf(mq, fabsf(p.sq[(size_t)bh * nqb + i]));
         for (int i = lane; i < nkb; i += 64) mk = fmaxf(mk, fabsf(p.sk[(size_t)kv_bh * nkb + i]));
     }
     wait_vmem_le<0>();
     __syncthreads();
+    if constexpr (QFUSE) {
+        // bf16 -> f32 is a shift; the quantiser's own operations from there on
+        auto val = [&](int s, int e) __attribute__((always_inline)) -> float {
+            const uint4 w = qraw[s][e >> 3];
+            const uint32_t u = (e & 7) < 2 ? w.x : (e & 7) < 4 ? w.y : (e & 7) < 6 ? w.z : w.w;
+            return __uint_as_float((e & 1) ? (u & 0xffff0000u) : (u << 16));
+        };
+        float mx = 0.f;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, fabsf(val(s, e)));
+        mx = xhalf_max(mx);  // the two lanes of a query
+#pragma unroll
+        for (int o = 16; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        float *red = (float *)(lds + QF_RED);
+        if (lane == 0) red[wave] = mx;
+        __syncthreads();
+        // a block of 128 queries is four waves (a block past the last query holds copies of the last row and is
+        // neither used nor written back)
+        const int w0 = wave & ~3;
+        mx = fmaxf(fmaxf(red[w0], red[w0 + 1]), fmaxf(red[w0 + 2], red[w0 + 3]));
+        const float scale = (mx > 0.f) ? mx / 127.0f : 1.f;
+        const float inv = 1.f / scale;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                int iv = (int)rintf(val(s, e) * inv);
+                iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
+                w[e >> 2] |= ((uint32_t)iv & 0xffu) << ((e & 3) * 8);
+            }
+            qreg[s] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+        sq_lane = scale;
+        // the workgroup's largest Q scale, for the grid below: every wave reads every wave's maximum
+        float wg_mx = red[0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) wg_mx = fmaxf(wg_mx, red[w]);
+        mq = (wg_mx > 0.f) ? wg_mx / 127.0f : 1.f;
+        const int blk = q_row >> 7, nqb = (N + 127) >> 7;
+        if (p.sq_out != nullptr && lane == 0 && (wave & 3) == 0 && blk < nqb) p.sq_out[(size_t)bh * nqb + blk] = scale;
+        if (p.q8_out != nullptr && q_row < N) {
+            int8_t *dst = p.q8_out + ((size_t)bh * N + q_row) * D;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) *(uint4 *)(dst + s * 32 + h * 16) = qreg[s];
+        }
+    }
     if constexpr (BIAS && !PER_KEY) {
         // The exponent reference stays on a grid no finer than the unit in the last place of
         // 12582912 c for the largest c = sq sk scale log2(e) the workgroup can meet; every wave reduces
@@ -852,17 +917,17 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
 }
 
 // int8 uses the biased accumulators (see s_init); bf16 and FP8 the plain ones.
-template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false>
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 __device__ __forceinline__ void attn_pipe_body(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
-    attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS), NW, PER_KEY>(p, lds, wg_linear);
+    attn_pipe_impl<D, CAUSAL, MODE, OUT_F32, (MODE == MODE_I8 && ARHIP_PIPE_INT_BIAS), NW, PER_KEY, QFUSE>(p, lds, wg_linear);
 }
 
-template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false>
+template <int D, bool CAUSAL, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 __global__ void __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) attn_pipe_kernel(const AttnParams p)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<D, MODE, NW, PER_KEY>()];
-    attn_pipe_body<D, CAUSAL, MODE, OUT_F32, NW, PER_KEY>(p, lds, (int)blockIdx.x);
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<D, MODE, NW, PER_KEY, QFUSE>()];
+    attn_pipe_body<D, CAUSAL, MODE, OUT_F32, NW, PER_KEY, QFUSE>(p, lds, (int)blockIdx.x);
 }
 
 }  // namespace arhip

@@ -66,12 +66,12 @@ static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bo
 
 // The software-pipelined kernel (no additive mask, tile-uniform K scales): 8 waves per workgroup, or 4
 // (two workgroups per compute unit) where a workgroup sees few tiles.
-template <int D, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false>
+template <int D, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 static void launch_pipe(hipStream_t stream, const AttnParams &p, bool causal)
 {
     const dim3 grid((unsigned)p.total), block(NW * 64);
-    if (causal) hipLaunchKernelGGL((attn_pipe_kernel<D, true, MODE, OUT_F32, NW, PER_KEY>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((attn_pipe_kernel<D, false, MODE, OUT_F32, NW, PER_KEY>), grid, block, 0, stream, p);
+    if (causal) hipLaunchKernelGGL((attn_pipe_kernel<D, true, MODE, OUT_F32, NW, PER_KEY, QFUSE>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((attn_pipe_kernel<D, false, MODE, OUT_F32, NW, PER_KEY, QFUSE>), grid, block, 0, stream, p);
 }
 
 // Which of the two: 128 queries per workgroup hide a workgroup's prologue and epilogue under its
@@ -383,6 +383,57 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
 #undef SAGE_F
 #undef SAGE_D
 #undef SAGE_V
+    arhip_note_selected(ARHIP_K_SAGE);
+    return t.end();
+}
+
+// Q quantised inside the attention kernel (as the reference does, src/runtime/cuda_flash_sage.rs:201-223): the
+// pipelined int8 kernel with bf16 queries, scales over blocks of 128 queries.
+extern "C" int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const int8_t *k8, const float *sk,
+                                     const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
+                                     int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
+                                     int causal, int out_dtype, float scale, int wait, double *secs)
+{
+    if (int rc = check_common("arhip_sage_fwd_qfused", dev, q, k8, v, o, nullptr, B, Hq, Hkv, N, D)) return rc;
+    ARHIP_REQUIRE(sk, "arhip_sage_fwd_qfused: null scale pointer");
+    ARHIP_REQUIRE(out_dtype == ARHIP_F32 || out_dtype == ARHIP_BF16, "arhip_sage_fwd_qfused: out_dtype %d", out_dtype);
+    int shift = 0;
+    while (((int64_t)64 << shift) < bk) ++shift;
+    ARHIP_REQUIRE(((int64_t)64 << shift) == bk, "arhip_sage_fwd_qfused: K scales over whole 64-key tiles (bk = 64 * 2^j), got bk = %lld",
+                  (long long)bk);
+    ARHIP_REQUIRE(pipe_addressable(N, D, 2), "arhip_sage_fwd_qfused: (N + 320) * D * 2 must stay below 2^31 (N = %lld)", (long long)N);
+    ARHIP_REQUIRE(q8_out == nullptr || arhip_aligned16(q8_out), "arhip_sage_fwd_qfused: q8_out must be 16-byte aligned");
+    ARHIP_HIP(hipSetDevice(dev->ordinal));
+    AttnParams p = {};
+    p.q = q; p.k = k8; p.v = v; p.o = o;
+    p.kv_len = kv_len;
+    p.sk = sk;
+    p.sq_out = sq_out; p.q8_out = q8_out;
+    p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
+    dense_strides(p.qs, Hq, N, D);
+    dense_strides(p.ks, Hkv, N, D);
+    dense_strides(p.vs, Hkv, N, D);
+    dense_strides(p.os, Hq, N, D);
+    p.bq = 128; p.bk = (int)bk;
+    p.bk_tile_shift = shift;
+    p.bk_key_shift = -1;
+    p.scale = scale;
+    const bool c = causal != 0, f32o = out_dtype == ARHIP_F32;
+    const int nw = pipe_wants_4_waves(dev, B * Hq, N, D, c, kv_len != nullptr) ? 4 : 8;
+    p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
+    p.total = (int)(p.nq * B * Hq);
+    p.lpt = p.total <= 16 * dev->cus;
+    arhip_call_timer t{dev, wait, secs};
+    t.kernel = ARHIP_K_SAGE;
+    if (int rc = t.begin()) return rc;
+#define SAGE_QF(DD, NWW)                                                                               \
+    do {                                                                                               \
+        if (f32o) launch_pipe<DD, MODE_I8, true, NWW, false, true>(dev->stream, p, c);                 \
+        else launch_pipe<DD, MODE_I8, false, NWW, false, true>(dev->stream, p, c);                     \
+    } while (0)
+    if (D == 64) { if (nw == 4) SAGE_QF(64, 4); else SAGE_QF(64, 8); }
+    else { if (nw == 4) SAGE_QF(128, 4); else SAGE_QF(128, 8); }
+#undef SAGE_QF
     arhip_note_selected(ARHIP_K_SAGE);
     return t.end();
 }

@@ -235,6 +235,17 @@ class Device:
                                           ctypes.byref(s)))
         return s.value if wait else None
 
+    def sage_fwd_qfused(self, q, k8, sk, v, o, B, Hq, Hkv, N, D, bk, out_dtype=BF16, sq_out=None, q8_out=None, kv_len=None,
+                        causal=False, scale=None, wait=True):
+        """sage_quant of Q (bf16, blocks of 128 queries) inside the attention kernel; sq_out / q8_out receive the
+        scales and codes it derived."""
+        scale = float(1.0 / np.sqrt(np.float32(D))) if scale is None else float(scale)
+        s = ctypes.c_double()
+        check(self.lib.arhip_sage_fwd_qfused(self.handle, self._ptr(q), self._ptr(k8), self._ptr(sk), self._ptr(v), self._ptr(o),
+                                             self._ptr(sq_out), self._ptr(q8_out), self._ptr(kv_len), B, Hq, Hkv, N, D, bk,
+                                             int(causal), out_dtype, scale, int(wait), ctypes.byref(s)))
+        return s.value if wait else None
+
     def sage_quant_static(self, x, x8, scales, B, H, N, D, block, dtype, mean=None, smooth=False, wait=True):
         """sage_quant with the partial sums in the library's own device array (no allocation)."""
         s = ctypes.c_double()

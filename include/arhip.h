@@ -255,6 +255,17 @@ int arhip_sage_fwd(arhip_device *dev, const int8_t *q8, const int8_t *k8,
                    int32_t *dbg_logits, const int32_t dbg_sel[3],
                    int wait, double *secs);
 
+/* arhip_sage_fwd_qfused: arhip_sage_quant of Q (bf16 input, blocks of 128 queries, no smoothing) and
+ *   arhip_sage_fwd in one launch: the reference quantises Q inside its attention kernel
+ *   (src/runtime/cuda_flash_sage.rs:201-223), and so does the pipelined kernel's prologue here, with the
+ *   quantiser's own operations in its own order, so o is bit for bit what the two calls give.
+ *   q bf16 [B,Hq,N,D]; k8 / sk from arhip_sage_quant with bk = 64 * 2^j; v bf16; no additive mask.
+ *   sq_out [B,Hq,ceil(N/128)] and q8_out [B,Hq,N,D] receive the scales and codes where not NULL. */
+int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const int8_t *k8, const float *sk,
+                          const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
+                          int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
+                          int causal, int out_dtype, float scale, int wait, double *secs);
+
 /* arhip_sage_fwd_strided: arhip_sage_fwd with element strides {batch, head, token} for v and o
  *   (NULL = dense): v as the projection produced it ([B,N,Hkv,D]), o written as [B,N,Hq*D].
  *   q8, k8 and the scales are this library's own pre-pass outputs and stay dense. */

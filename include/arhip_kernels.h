@@ -118,6 +118,17 @@
 #define ARHIP_KERNEL_FLASH_SAGE_FP8_LONG_LENS "ar_flash_sage_fp8_long_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_FP8_MID_LENS "ar_flash_sage_fp8_mid_lens"
 
+/* The Q quantiser inside the attention kernel, as in the reference (src/runtime/cuda_flash_sage.rs:201-223), for
+ * the pipelined int8 kernel: the argument lists of ar_flash_sage_long / _mid (and their _lens twins) with
+ *     Q    bf16 [b*hq, n, head_dim] instead of int8 codes
+ *     SQ   [b*hq, ceil(n/128)] f32, WRITTEN: the scales the kernel derived (bq must be 128)
+ * K8 / SK as the K quantiser left them, bk = 64 * 2^j.  Bit-identical to ar_sage_quant_blocks_bf16 on Q followed
+ * by ar_flash_sage_long / _mid. */
+#define ARHIP_KERNEL_FLASH_SAGE_QF_LONG "ar_flash_sage_qf_long"
+#define ARHIP_KERNEL_FLASH_SAGE_QF_MID "ar_flash_sage_qf_mid"
+#define ARHIP_KERNEL_FLASH_SAGE_QF_LONG_LENS "ar_flash_sage_qf_long_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_QF_MID_LENS "ar_flash_sage_qf_mid_lens"
+
 /* FP8 E4M3 variant (the reference's `src(fp8 = true)`, src/runtime/cuda_flash_sage.rs:82-84, 92-147):
  * the same argument lists as ar_flash_sage / ar_sage_quant_{blocks,rows}_*, with E4M3 codes
  * (scale = absmax / 448) in place of int8 values. */

@@ -81,7 +81,7 @@ def test_code_object_is_built_and_names_every_entry_point():
     """The named kernels (include/arhip_kernels.h) are all in the code object (no launch here)."""
     text = open(os.path.join(ROOT, "include", "arhip_kernels.h")).read()
     names = re.findall(r'#define ARHIP_KERNEL_\w+ "(\w+)"', text)
-    assert len(names) == 40
+    assert len(names) == 44
     image = open(_lib.KERNELS_PATH, "rb").read()
     for n in names:
         assert n.encode() + b"\0" in image or n.encode() in image, n

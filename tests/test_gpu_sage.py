@@ -10,7 +10,7 @@ import pytest
 import oracle
 from autorust_amd import _lib, synth
 from autorust_amd.device import BF16, F32, selections
-from gpu_util import bf16_ulps, fill_qkv, run_sage
+from gpu_util import Bufs, bf16_ulps, fill_qkv, run_sage
 
 pytestmark = pytest.mark.gpu
 
@@ -240,3 +240,43 @@ def test_token_major_layout(dev, N, Hq, Hkv):
     rows = np.array(sorted({0, 1, 127, 128, 255, 256, N // 2, N - 2, N - 1}), np.int32)
     want = oracle.sage(w_q8, w_k8, w_sq, w_sk, v, bq, bk, causal=True, rows=rows, round_out=True)
     assert bf16_ulps(outs[1][5][:, :, rows], want) <= 3
+
+
+@pytest.mark.parametrize("B,H,Hkv,N,D,causal,use_len,out_dtype", [
+    (1, 32, 32, 2500, 128, False, False, BF16),      # 8 waves per workgroup, ragged last block of queries
+    (2, 8, 4, 1000, 128, True, True, F32),           # 4 waves, grouped heads, key lengths
+    (2, 6, 6, 300, 64, False, False, BF16),
+    (1, 64, 64, 2304, 64, True, False, F32),
+])
+def test_q_quantiser_inside_the_attention_kernel(dev, B, H, Hkv, N, D, causal, use_len, out_dtype):
+    """arhip_sage_fwd_qfused: Q quantised in the prologue of the pipelined kernel (the reference quantises Q inside
+    its attention kernel too, src/runtime/cuda_flash_sage.rs:201-223).  The codes and scales it exports are the
+    oracle's bit for bit, and the output is bit for bit that of quantising first."""
+    q = oracle.bf16_round(synth.normal(901, (B, H, N, D)) * (np.float32(2.0) ** np.linspace(-3, 3, H, dtype=np.float32))[None, :, None, None])
+    k = oracle.bf16_round(synth.normal(902, (B, Hkv, N, D)) + np.float32(1.5) * synth.normal(904, (1, Hkv, 1, D)))
+    v = synth.normal(903, (B, Hkv, N, D))
+    q[0, 0, 128:256] = 0.0                                     # an all-zero block: scale 1
+    kv_len = np.array([N - 77, max(1, N // 3)][:B], np.int32) if use_len else None
+    r = run_sage(dev, q, k, v, 128, 64, smooth=True, in_dtype=BF16, out_dtype=out_dtype, kv_len=kv_len, causal=causal)
+    nqb = (N + 127) // 128
+    with Bufs(dev) as bufs:
+        dq = bufs.put(synth.to_bf16_bits(q))
+        k8, sk = bufs.put(r["k8"]), bufs.put(r["sk"])
+        dv = bufs.put(synth.to_bf16_bits(v))
+        do = bufs.new(q.size * (4 if out_dtype == F32 else 2))
+        sq_out, q8_out = bufs.new(B * H * nqb * 4), bufs.new(q.size)
+        dl = bufs.put(kv_len) if use_len else None
+        dev.sage_fwd_qfused(dq, k8, sk, dv, do, B, H, Hkv, N, D, 64, out_dtype=out_dtype, sq_out=sq_out, q8_out=q8_out,
+                            kv_len=dl, causal=causal)
+        got = do.copyout(np.float32, q.shape) if out_dtype == F32 else synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+        got_sq, got_q8 = sq_out.copyout(np.float32, (B, H, nqb)), q8_out.copyout(np.int8, q.shape)
+        # without the exports, and with a coarser K granularity, the call still runs
+        do2 = bufs.new(q.size * (4 if out_dtype == F32 else 2))
+        dev.sage_fwd_qfused(dq, k8, sk, dv, do2, B, H, Hkv, N, D, 64, out_dtype=out_dtype, kv_len=dl, causal=causal)
+        again = do2.copyout(np.float32, q.shape) if out_dtype == F32 else synth.from_bf16_bits(do2.copyout(np.uint16, q.shape))
+        with pytest.raises(_lib.ArhipError, match="whole 64-key tiles"):
+            dev.sage_fwd_qfused(dq, k8, sk, dv, do2, B, H, Hkv, N, D, 32, out_dtype=out_dtype)
+    w_q8, w_sq = oracle.quant_blocks(q, 128)
+    assert np.array_equal(got_sq, w_sq) and np.array_equal(got_q8, w_q8)
+    assert w_sq[0, 0, 1] == 1.0
+    assert np.array_equal(got, r["out"]) and np.array_equal(again, got)
