@@ -477,7 +477,16 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
                                       {256, 1, 1}, {n, d, blk, nblk, (int64_t)smooth}));
         }
     };
-    quant(q, q8, sq, h, bq, nqb, false);
+    int shift = 0;
+    while (((int64_t)64 << shift) < bk) ++shift;
+    const bool tile_uniform = ((int64_t)64 << shift) == bk;
+    // scales over a power of two of keys below 64 (the reference's bk = 1) are applied per logit
+    const bool key_scales = bk < 64 && (bk & (bk - 1)) == 0;
+    const bool pipelined = !has_mask && (tile_uniform || key_scales) && long_variant(n, d);
+    // bf16 queries with scales over blocks of 128 are quantised by the attention kernel itself (as the reference's
+    // kernel does, cuda_flash_sage.rs:201-223): one launch and one pass over Q fewer
+    const bool q_fused = pipelined && tile_uniform && bf16_in && bq == 128 && !st.sage_fp8;
+    if (!q_fused) quant(q, q8, sq, h, bq, nqb, false);
     if (st.sage_smooth_k) {
         Tensor part = Tensor::empty(dev, {b, hk, nchunk, d}, F);
         const int64_t cpb = 256 / (d / 8);
@@ -496,19 +505,19 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     std::vector<int64_t> svals = vals;
     svals.push_back(bq);
     svals.push_back(bk);
-    int shift = 0;
-    while (((int64_t)64 << shift) < bk) ++shift;
-    const bool tile_uniform = ((int64_t)64 << shift) == bk;
-    // scales over a power of two of keys below 64 (the reference's bk = 1) are applied per logit
-    const bool key_scales = bk < 64 && (bk & (bk - 1)) == 0;
-    if (!has_mask && (tile_uniform || key_scales) && long_variant(n, d)) {
+    if (pipelined) {
         svals.push_back(bf16_in ? 0 : 1);  // out_f32
-        if (mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr))
+        const bool mid = mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr);
+        const std::array<int64_t, 3> grid = {mid ? (n + 127) / 128 : (n + 255) / 256, b * h, 1}, block = {mid ? 256 : 512, 1, 1};
+        if (q_fused)   // Q itself in the first slot; the scales slot is written
+            calls.push_back(attn_call(mid ? "ar_flash_sage_qf_mid" : "ar_flash_sage_qf_long", {q, k8, vb, out, mslot, sq, sk},
+                                      {BF, I8, BF, X, F, F, F}, grid, block, svals));
+        else if (mid)
             calls.push_back(attn_call(st.sage_fp8 ? "ar_flash_sage_fp8_mid" : "ar_flash_sage_mid", {q8, k8, vb, out, mslot, sq, sk},
-                                      {I8, I8, BF, X, F, F, F}, {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));
+                                      {I8, I8, BF, X, F, F, F}, grid, block, svals));
         else
             calls.push_back(attn_call(st.sage_fp8 ? "ar_flash_sage_fp8_long" : "ar_flash_sage_long", {q8, k8, vb, out, mslot, sq, sk},
-                                      {I8, I8, BF, X, F, F, F}, {(n + 255) / 256, b * h, 1}, {512, 1, 1}, svals));
+                                      {I8, I8, BF, X, F, F, F}, grid, block, svals));
     } else if (!bf16_in) {
         calls.push_back(attn_call(general, {q8, k8, vb, out, mslot, sq, sk}, {I8, I8, BF, F, F, F, F},
                                   {(n + 127) / 128, b * h, 1}, {256, 1, 1}, svals));

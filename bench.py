@@ -89,8 +89,10 @@ class SageWorkload:
         self.ws = dev.alloc(dev.sage_quant_workspace(B, H, S, D))
         self.ops = attn_ops(B, H, S, D, causal)
         self.kernel = _lib.K_SAGE
-        # dominant kernel: int8 Q, K (1 B), bf16 V and O (2 B), block scales
-        self.kernel_bytes = n * (1 + 1 + 2 + 2) + 4 * B * H * (S // bq + S // bk)
+        # dominant kernel: int8 K (1 B), Q as int8 codes (1 B) or, quantised in its prologue, bf16 (2 B), bf16 V and O
+        # (2 B), block scales
+        q_bytes = 2 if (not f32_io and bq == 128 and bk % 64 == 0 and not fp8) else 1
+        self.kernel_bytes = n * (q_bytes + 1 + 2 + 2) + 4 * B * H * (S // bq + S // bk)
         self.dtype = "fp8" if fp8 else "int8"
 
     def step(self):
@@ -103,13 +105,21 @@ class SageWorkload:
             d.sage_fwd_fp8(self.q8, self.k8, self.sq, self.sk, self.dv, self.do, B, H, H, S, D, self.bq, self.bk,
                            out_dtype=io, causal=self.causal, wait=False)
             return
-        d.sage_quant(self.dq, self.q8, self.sq, B, H, S, D, self.bq, io, wait=False)
+        # bf16 queries with scales over blocks of 128: the attention kernel quantises Q itself (as the host mirror's
+        # Tensor::sage_attention_with does); otherwise the Q quantiser is a launch of its own
+        q_fused = not self.f32_io and self.bq == 128 and self.bk % 64 == 0 and not self.fp8
+        if not q_fused:
+            d.sage_quant(self.dq, self.q8, self.sq, B, H, S, D, self.bq, io, wait=False)
         d.sage_quant(self.dk, self.k8, self.sk, B, H, S, D, self.bk, io, mean=self.mean, workspace=self.ws,
                      smooth=not self.f32_io, wait=False)
         if self.f32_io:
             d.cast_bf16(self.dvf, self.dv, B * H * S * D, wait=False)
-        d.sage_fwd(self.q8, self.k8, self.sq, self.sk, self.dv, self.do, B, H, H, S, D, self.bq, self.bk,
-                   out_dtype=io, causal=self.causal, wait=False)
+        if q_fused:
+            d.sage_fwd_qfused(self.dq, self.k8, self.sk, self.dv, self.do, B, H, H, S, D, self.bk, out_dtype=io,
+                              sq_out=self.sq, causal=self.causal, wait=False)
+        else:
+            d.sage_fwd(self.q8, self.k8, self.sq, self.sk, self.dv, self.do, B, H, H, S, D, self.bq, self.bk,
+                       out_dtype=io, causal=self.causal, wait=False)
 
     def roofline(self, secs):
         half = self.ops / 2.0
@@ -487,7 +497,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic",
         "config": {"workload": w.name, "B": w.B, "H": w.H, "S": w.S, "D": w.D, "causal": bool(w.causal),
-                   "step": "quantise Q (128-token blocks) + smooth and quantise K (64-token blocks) + %s attention" % w.dtype
+                   "step": "smooth and quantise K (64-token blocks) + %s attention with the Q quantiser (128-token blocks) %s" %
+                           (w.dtype, "as a launch of its own" if w.fp8 else "in its prologue")
                            if w.dtype in ("int8", "fp8") else "attention forward"},
         "roofline": res["roofline"],
         "cpu_baseline": cpu,

@@ -253,7 +253,16 @@ pub fn host_calls_sage(
     let (bq, bk) = (sage.block_q, sage.block_k);
     let (nqb, nkb, nchunk) = ((n + bq - 1) / bq, (n + bk - 1) / bk, (n + 63) / 64);
     let mut calls = Vec::new();
-    calls.push(quant_call(q8fmt, sfx, x, &q, &s.q8, &s.sq, &s.mean, b, h, n, d, bq, nqb, false));
+    let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
+    // scales over a power of two of keys below 64 (the CUDA kernel's bk = 1) are applied per logit
+    let key_scales = bk >= 1 && bk < 64 && bk.count_ones() == 1;
+    let pipelined = !opts.has_mask && (tile_uniform || key_scales) && long_variant(n, d);
+    // bf16 queries with scales over blocks of 128 are quantised by the attention kernel itself (as the CUDA
+    // kernel does): one launch and one pass over Q fewer
+    let q_fused = pipelined && tile_uniform && bf16_in && bq == 128 && !sage.fp8;
+    if !q_fused {
+        calls.push(quant_call(q8fmt, sfx, x, &q, &s.q8, &s.sq, &s.mean, b, h, n, d, bq, nqb, false));
+    }
     if sage.smooth_k {
         let cpb = 256 / (d / 8);
         calls.push(call(&format!("ar_sage_kmean_partial_{sfx}"), vec![k.clone(), s.part.clone()], &[x, f],
@@ -274,17 +283,17 @@ pub fn host_calls_sage(
     let mut sv = vals(n, d, h, opts);
     sv.push(bq);
     sv.push(bk);
-    let tile_uniform = bk >= 64 && bk % 64 == 0 && (bk / 64).count_ones() == 1;
-    // scales over a power of two of keys below 64 (the CUDA kernel's bk = 1) are applied per logit
-    let key_scales = bk >= 1 && bk < 64 && bk.count_ones() == 1;
-    if !opts.has_mask && (tile_uniform || key_scales) && long_variant(n, d) {
+    if pipelined {
         sv.push(!bf16_in as i64); // out_f32
-        if mid_variant(dev, b, h, n, d, opts.causal, lens.is_some()) {
-            calls.push(attn_call(if sage.fp8 { "ar_flash_sage_fp8_mid" } else { "ar_flash_sage_mid" }, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
-                                 [(n + 127) / 128, b * h, 1], [256, 1, 1], sv));
+        let mid = mid_variant(dev, b, h, n, d, opts.causal, lens.is_some());
+        let (grid, block) = if mid { ([(n + 127) / 128, b * h, 1], [256, 1, 1]) } else { ([(n + 255) / 256, b * h, 1], [512, 1, 1]) };
+        if q_fused {
+            // Q itself in the first slot; the scales slot is written
+            let name = if mid { "ar_flash_sage_qf_mid" } else { "ar_flash_sage_qf_long" };
+            calls.push(attn_call(name, vec![q, s.k8, vb, o, mask, s.sq, s.sk], &[bf, i8t, bf, x, f, f, f], lens, grid, block, sv));
         } else {
-            calls.push(attn_call(long, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens,
-                                 [(n + 255) / 256, b * h, 1], [512, 1, 1], sv));
+            let name = if mid { if sage.fp8 { "ar_flash_sage_fp8_mid" } else { "ar_flash_sage_mid" } } else { long };
+            calls.push(attn_call(name, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens, grid, block, sv));
         }
     } else if !bf16_in {
         calls.push(attn_call(general, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, f, f, f, f], lens,

@@ -479,3 +479,34 @@ def test_ar_flash_sage_mid_by_name(dev, kernels, d, causal, out_f32, n):
     # follows the largest Q scale of a workgroup's queries (128 here, 256 there), and P is rounded to
     # bf16 relative to that reference.
     assert np.abs(got - got_long).max() <= tol
+
+
+@pytest.mark.parametrize("form,per_wg,block", [("long", 256, 512), ("mid", 128, 256)])
+@pytest.mark.parametrize("d,causal,out_f32,with_lens", [(128, False, 0, False), (64, True, 1, True)])
+def test_ar_flash_sage_qf_by_name(dev, kernels, form, per_wg, block, d, causal, out_f32, with_lens):
+    """The entries that quantise the bf16 queries in their prologue: the scales they write are the quantiser's,
+    the output is bit for bit that of ar_sage_quant_blocks_bf16 followed by the plain entry of the same form."""
+    b, hq, hkv, n, bq, bk = 2, 4, 2, 700, 128, 64
+    q = oracle.bf16_round(synth.normal(31, (b, hq, n, d)))
+    k = oracle.bf16_round(synth.normal(32, (b, hkv, n, d)) + np.float32(2.0) * synth.normal(34, (1, hkv, 1, d)))
+    v = synth.normal(33, (b, hkv, n, d))
+    lens = np.array([333, n], np.int32) if with_lens else None
+    sfx = "_lens" if with_lens else ""
+    with Bufs(dev) as bufs:
+        q8, sq, _, h_q8, h_sq, _ = _quantise_by_name(dev, kernels, bufs, q, bq, False, BF16)
+        k8, sk, _, h_k8, h_sk, _ = _quantise_by_name(dev, kernels, bufs, k, bk, True, BF16)
+        dq, dv = bufs.put(synth.to_bf16_bits(q)), bufs.put(synth.to_bf16_bits(v))
+        do, dp = bufs.new(q.size * 4), bufs.new(q.size * 4)
+        sq2 = bufs.new(b * hq * ((n + bq - 1) // bq) * 4)
+        dl = [bufs.put(lens)] if with_lens else []
+        vals = [n, d, int(causal), 0, hq, hkv, bq, bk, out_f32]
+        dev.launch(kernels, "ar_flash_sage_qf_" + form + sfx, _grid(n, per_wg, b, hq), (block, 1, 1), [dq, k8, dv, do, do] + dl + [sq2, sk], vals)
+        dev.launch(kernels, "ar_flash_sage_" + form + sfx, _grid(n, per_wg, b, hq), (block, 1, 1), [q8, k8, dv, dp, dp] + dl + [sq, sk], vals)
+        words = q.size if out_f32 else q.size // 2
+        got, plain = do.copyout(np.uint32, (words,)), dp.copyout(np.uint32, (words,))
+        got_sq = sq2.copyout(np.float32, h_sq.shape)
+        with pytest.raises(_lib.ArhipError, match="blocks of 128 queries"):
+            dev.launch(kernels, "ar_flash_sage_qf_" + form + sfx, _grid(n, per_wg, b, hq), (block, 1, 1), [dq, k8, dv, do, do] + dl + [sq2, sk],
+                       [n, d, int(causal), 0, hq, hkv, 64, bk, out_f32])
+    assert np.array_equal(got_sq, h_sq)
+    assert np.array_equal(got, plain)

@@ -323,11 +323,11 @@ def test_capture_and_replay(hdev):
     out = tq.attention_with(tk, tv, None, 0.0, True, sess)
     o2 = tq.sage_attention_with(tk, tv, None, 0.0, True, sess)
     nsteps = sess.end_capture()
-    # one launch for flash; for Sage the pre-pass launches (quantise Q, K mean in two steps, quantise
-    # K) and the attention kernel, which stores bf16 itself, each a HostCall of its own
+    # one launch for flash; for Sage the pre-pass launches (K mean in two steps, quantise K) and the
+    # attention kernel, which quantises the bf16 queries itself and stores bf16, each a HostCall of its own
     names = [sess.step(i)[0] for i in range(nsteps)]
-    assert names == ["ar_flash_bf16_mid", "ar_sage_quant_blocks_bf16", "ar_sage_kmean_partial_bf16", "ar_sage_kmean_final",
-                     "ar_sage_quant_blocks_bf16", "ar_flash_sage_mid"]
+    assert names == ["ar_flash_bf16_mid", "ar_sage_kmean_partial_bf16", "ar_sage_kmean_final",
+                     "ar_sage_quant_blocks_bf16", "ar_flash_sage_qf_mid"]
     name, grid, vals = sess.step(0)
     # grid [query tiles of 128, b*h, 1], vals [n, head_dim, causal, has_mask, hq, hkv] (cuda_flash_bf16.rs:550-599)
     assert grid == [(n + 127) // 128, b * h, 1] and vals == [n, d, 1, 0, h, h]
@@ -335,7 +335,8 @@ def test_capture_and_replay(hdev):
     assert src.endswith("attn_kernels.hsaco") and local == [256, 1, 1] and (nbufs, nvals) == (5, 6)
     BF, F, I32 = 1, 0, 4
     assert sig == [(0, BF), (1, BF), (2, BF), (3, BF), (4, F)] + [(5 + i, I32) for i in range(6)]   # cuda_flash_bf16.rs:563-578
-    assert sess.step(5)[2] == [n, d, 1, 0, h, h] and sess.step_detail(5)[2:4] == (7, 9)   # the six common scalars; then bq, bk, out_f32
+    assert sess.step(4)[2] == [n, d, 1, 0, h, h] and sess.step_detail(4)[2:4] == (7, 9)   # the six common scalars; then bq, bk, out_f32
+    assert sess.step_detail(4)[4][0] == (0, BF)               # the queries themselves, not their codes
     first = out.to_list().copy()
     first2 = o2.to_list().copy()
     allocs = hdev.raw_allocs
