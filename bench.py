@@ -34,7 +34,7 @@ PEAK_HBM = 8000.0    # GB/s, MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # and calibrated against a 1 GiB copy kernel (profiles/attn_pipe_s8192_hbm_traffic.md).
-MEASURED_TRAFFIC = {"sage_int8_b4_h32_s8192_d128": 805.5e6}
+MEASURED_TRAFFIC = {"sage_int8_b4_h32_s8192_d128": 940.0e6}
 
 
 def log(*a):
