@@ -70,15 +70,26 @@ __device__ __forceinline__ void static_for(F &&f)
     }
 }
 
-// LDS bytes attn_pipe_body needs: [piece][64 rows][64 B] K and V tiles, four stages of both (NW = 8), or a
-// ring of two K tiles and one of three V tiles (NW = 4).  PER_KEY (a scale per key, or per block of fewer than
+// The 4-wave form keeps K and V in rings of their own (two and three tiles) so that two workgroups fit a compute
+// unit at D = 128; with 8-bit operands at D = 64 four whole stages fit twice as well (48 KB each), and with them the
+// four-tiles-per-trip loop and one more tile of latency cover: int8 B4 H32 N = 2048 / 8192 -7 / -5 %, causal -4 / -5 %,
+// per-key scales -7 / -5 %, B8 H6 N789 -4 %, same bits (bf16 at D = 64 gains nothing and loses 6 % on short causal shapes).
+template <int D, int MODE, int NW>
+constexpr bool attn_pipe_rings()
+{
+    return NW == 4 && !(D == 64 && MODE != MODE_BF16);
+}
+
+// LDS bytes attn_pipe_body needs: [piece][64 rows][64 B] K and V tiles, four stages of both, or a
+// ring of two K tiles and one of three V tiles (attn_pipe_rings).  PER_KEY (a scale per key, or per block of fewer than
 // 64 keys): behind the tiles, a ring of four times 64 raw key scales and, per wave, two times 64 pairs of
 // derived factors.
 // QFUSE (Q arrives as bf16 and is quantised in the prologue): 256 bytes for the exchange of the waves' maxima.
 template <int D, int MODE, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 constexpr int attn_pipe_lds_bytes()
 {
-    return 4096 * ((NW == 8 ? 4 : 2) * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64) + (NW == 8 ? 4 : 3) * (D * 2 / 64)) +
+    constexpr bool R = attn_pipe_rings<D, MODE, NW>();
+    return 4096 * ((R ? 2 : 4) * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64) + (R ? 3 : 4) * (D * 2 / 64)) +
            (PER_KEY ? 1024 + NW * 1024 : 0) + (QFUSE ? 256 : 0);
 }
 
@@ -111,7 +122,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
     static_assert(!PER_KEY || BIAS || MODE == MODE_FP8, "per-key scales: int8 (on the biased accumulators) and FP8");
     static_assert(NW == 8 || NW == 4, "8 waves (one workgroup per CU) or 4 (two)");
-    constexpr bool RINGS = NW == 4;  // K and V in rings of their own, two and three tiles deep
+    constexpr bool RINGS = attn_pipe_rings<D, MODE, NW>();  // K and V in rings of their own, two and three tiles deep
     constexpr int BQ = NW * 32;
     constexpr int QK_BYTES = (MODE != MODE_BF16) ? 1 : 2;
     constexpr int KP = D * QK_BYTES / 64;  // 64-byte pieces per K row
