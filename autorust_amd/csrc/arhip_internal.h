@@ -12,9 +12,10 @@
 
 #include "../../include/arhip.h"
 
+// A loaded code object, or several of them loaded from one image (a container: see arhip_module_load)
 struct arhip_module_entry {
-    hipModule_t mod = nullptr;
-    std::vector<char> image;
+    std::vector<hipModule_t> mods;
+    std::vector<std::vector<char>> images;  // private copies, alive as long as the modules are loaded
     std::unordered_map<std::string, hipFunction_t> fns;
 };
 

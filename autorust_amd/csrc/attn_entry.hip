@@ -49,6 +49,14 @@
 // last: it switches floating-point contraction off for the rest of the file
 #include "sage_quant_kernels.h"
 
+// The entry points compile as eleven code objects side by side (-DARHIP_ENTRY_PART=1 ... 11; the build packs them into
+// one file that arhip_module_load takes as a whole): the pipelined kernels are several thousand instructions per
+// variant, minutes of compilation per entry.  Without the macro this file is one code object with all of them.
+#ifndef ARHIP_ENTRY_PART
+#define ARHIP_ENTRY_PART 0
+#endif
+#define ARHIP_PART(k) (ARHIP_ENTRY_PART == 0 || ARHIP_ENTRY_PART == (k))
+
 using namespace arhip;
 
 namespace {
@@ -111,6 +119,7 @@ __device__ __forceinline__ void flash_f32_entry(float *lds, const float *Q, cons
 }
 }  // namespace
 
+#if ARHIP_PART(1)
 extern "C" __global__ void __launch_bounds__(256) ar_flash_f32(const float *Q, const float *K, const float *V, float *O,
                                                                 const float *M, int N, int head_dim, int causal,
                                                                 int has_mask, int hq, int hkv)
@@ -151,6 +160,7 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_fwd(const float *Q, cons
     }
 }
 
+#endif
 // Short shapes (few workgroups of 128 queries would leave most of the chip idle): 32 queries per
 // workgroup, grid [ceil(N/32), B*hq, 1], the key tiles dealt out between the four waves.  head_dim 64
 // only (the reference's own head size); any other returns without writing.  LSE may be null.
@@ -173,6 +183,7 @@ __device__ __forceinline__ void flash_f32_short(const float *Q, const float *K, 
 }
 }  // namespace
 
+#if ARHIP_PART(1)
 extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_f32_short(const float *Q, const float *K, const float *V, float *O,
                                                                          const float *M, int N, int head_dim, int causal,
                                                                          int has_mask, int hq, int hkv)
@@ -198,6 +209,7 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_prep(const float *O, con
     else if (head_dim == 128) bwd_prep_body<128>(O, dO, D, rows, row0);
 }
 
+#endif
 namespace {
 __device__ __forceinline__ FlashBwdParams bwd_params(const float *Q, const float *K, const float *V, const float *dO,
                                                      const float *LSE, const float *D, const float *M, int N,
@@ -213,6 +225,7 @@ __device__ __forceinline__ FlashBwdParams bwd_params(const float *Q, const float
 }
 }  // namespace
 
+#if ARHIP_PART(1)
 extern "C" __global__ void __launch_bounds__(256) ar_fl_bwd_dq(const float *Q, const float *K, const float *V,
                                                                 const float *dO, const float *LSE, const float *D,
                                                                 const float *M, float *dQ, int N, int head_dim, int causal,
@@ -249,8 +262,10 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_bwd_dkv(const float *Q, 
     }
 }
 
+#endif
 // The same for short shapes: 32 queries (dQ) / 32 keys (dK, dV) per workgroup, grid [ceil(N/32), B*hq, 1] /
 // [ceil(N/32), B*hkv, 1], the tiles of the other side dealt out between the four waves.  head_dim 64 only.
+#if ARHIP_PART(1)
 extern "C" __global__ void __launch_bounds__(256, 2) ar_fl_bwd_dq_short(const float *Q, const float *K, const float *V,
                                                                          const float *dO, const float *LSE, const float *D,
                                                                          const float *M, float *dQ, int N, int head_dim,
@@ -279,6 +294,7 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_bwd_dkv_short(const floa
     else bwd_dkv_body<64, 4, false, true>(p, lds, wg);
 }
 
+#endif
 namespace {
 __device__ __forceinline__ void flash_bf16_entry(unsigned char *lds, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                                                  uint16_t *O, const float *M, const int *L, int N, int head_dim, int causal,
@@ -302,6 +318,7 @@ __device__ __forceinline__ void flash_bf16_entry(unsigned char *lds, const uint1
 }
 }  // namespace
 
+#if ARHIP_PART(1)
 extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                                                                  uint16_t *O, const float *M, int N, int head_dim, int causal,
                                                                  int has_mask, int hq, int hkv)
@@ -318,6 +335,7 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_bf16_lens(const uint1
     flash_bf16_entry(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
 }
 
+#endif
 namespace {
 template <int NW>
 __device__ __forceinline__ void flash_bf16_long_entry(unsigned char *lds, const uint16_t *Q, const uint16_t *K, const uint16_t *V,
@@ -337,6 +355,7 @@ __device__ __forceinline__ void flash_bf16_long_entry(unsigned char *lds, const 
 }
 }  // namespace
 
+#if ARHIP_PART(2)
 extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                                                                       uint16_t *O, const float *M, int N, int head_dim,
                                                                       int causal, int has_mask, int hq, int hkv)
@@ -353,7 +372,9 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_bf16_long_lens(const 
     flash_bf16_long_entry<8>(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
 }
 
+#endif
 // the 4-wave form of the pipelined kernel: 128 queries per workgroup, two workgroups per compute unit
+#if ARHIP_PART(3)
 extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_bf16_mid(const uint16_t *Q, const uint16_t *K, const uint16_t *V,
                                                                         uint16_t *O, const float *M, int N, int head_dim,
                                                                         int causal, int has_mask, int hq, int hkv)
@@ -370,6 +391,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_bf16_mid_lens(cons
     flash_bf16_long_entry<4>(lds, Q, K, V, O, M, L, N, head_dim, causal, has_mask, hq, hkv);
 }
 
+#endif
 namespace {
 // ar_flash_sage / ar_flash_sage_fp8: the general kernel on pre-quantised operands, QMODE = MODE_I8 or MODE_FP8
 template <int QMODE>
@@ -408,6 +430,7 @@ __device__ __forceinline__ void flash_sage_entry(unsigned char *lds, const void 
 }
 }  // namespace
 
+#if ARHIP_PART(4)
 extern "C" __global__ void __launch_bounds__(256) ar_flash_sage(const int8_t *Q8, const int8_t *K8, const uint16_t *V, float *O,
                                                                  const float *M, const float *SQ, const float *SK, int N,
                                                                  int head_dim, int causal, int has_mask, int hq, int hkv,
@@ -426,8 +449,10 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_lens(const int8_
     flash_sage_entry<MODE_I8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
 }
 
+#endif
 // the FP8 E4M3 variant (the reference's AR_FP8 = 1 source, src/runtime/cuda_flash_sage.rs:82-84): same
 // arguments, Q8 / K8 hold E4M3 codes
+#if ARHIP_PART(5)
 extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_fp8(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
                                                                      float *O, const float *M, const float *SQ, const float *SK,
                                                                      int N, int head_dim, int causal, int has_mask, int hq,
@@ -446,6 +471,7 @@ extern "C" __global__ void __launch_bounds__(256) ar_flash_sage_fp8_lens(const u
     flash_sage_entry<MODE_FP8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk);
 }
 
+#endif
 // ar_flash_sage_long / ar_flash_sage_fp8_long: the pipelined kernel on pre-quantised operands
 template <int QMODE, int NW = 8>
 __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const void *Q8, const void *K8, const uint16_t *V, void *O,
@@ -464,16 +490,12 @@ __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const 
     p.bq = bq; p.bk = bk;
     p.bk_tile_shift = shift;
     p.bk_key_shift = keys ? key_shift : -1;
+    p.out_f32 = out_f32;
     const int wg = linear_wg();
 #define AR_SAGE_LONG(DD, PK)                                                              \
     do {                                                                                  \
-        if (out_f32) {                                                                    \
-            if (causal) attn_pipe_body<DD, true, QMODE, true, NW, PK>(p, lds, wg);        \
-            else attn_pipe_body<DD, false, QMODE, true, NW, PK>(p, lds, wg);              \
-        } else {                                                                          \
-            if (causal) attn_pipe_body<DD, true, QMODE, false, NW, PK>(p, lds, wg);       \
-            else attn_pipe_body<DD, false, QMODE, false, NW, PK>(p, lds, wg);             \
-        }                                                                                 \
+        if (causal) attn_pipe_body<DD, true, QMODE, false, NW, PK>(p, lds, wg);           \
+        else attn_pipe_body<DD, false, QMODE, false, NW, PK>(p, lds, wg);                 \
     } while (0)
     if (keys) {
         if (head_dim == 64) AR_SAGE_LONG(64, true);
@@ -485,6 +507,7 @@ __device__ __forceinline__ void flash_sage_long_entry(unsigned char *lds, const 
 #undef AR_SAGE_LONG
 }
 
+#if ARHIP_PART(6)
 extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
                                                                       void *O, const float *M, const float *SQ, const float *SK,
                                                                       int N, int head_dim, int causal, int has_mask, int hq,
@@ -503,7 +526,9 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_long_lens(const 
     flash_sage_long_entry<MODE_I8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
+#endif
 // the 4-wave form: 128 queries per workgroup, two workgroups per compute unit
+#if ARHIP_PART(7)
 extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_mid(const int8_t *Q8, const int8_t *K8, const uint16_t *V,
                                                                         void *O, const float *M, const float *SQ, const float *SK,
                                                                         int N, int head_dim, int causal, int has_mask, int hq,
@@ -522,6 +547,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_mid_lens(cons
     flash_sage_long_entry<MODE_I8, 4>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
+#endif
 // ar_flash_sage_qf_long / _mid: the pipelined int8 kernel with the Q quantiser in its prologue.  Q holds bf16
 // values; SQ [b*hq, ceil(n/128)] RECEIVES the scales (bq must be 128); K8 / SK as from the K quantiser with
 // bk = 64 * 2^j.  Same grid and block as ar_flash_sage_long / _mid.
@@ -539,22 +565,19 @@ __device__ __forceinline__ void flash_sage_qf_entry(unsigned char *lds, const ui
     p.bq = bq; p.bk = bk;
     p.bk_tile_shift = shift;
     p.bk_key_shift = -1;
+    p.out_f32 = out_f32;
     const int wg = linear_wg();
 #define AR_SAGE_QF(DD)                                                                        \
     do {                                                                                      \
-        if (out_f32) {                                                                        \
-            if (causal) attn_pipe_body<DD, true, MODE_I8, true, NW, false, true>(p, lds, wg); \
-            else attn_pipe_body<DD, false, MODE_I8, true, NW, false, true>(p, lds, wg);       \
-        } else {                                                                              \
-            if (causal) attn_pipe_body<DD, true, MODE_I8, false, NW, false, true>(p, lds, wg);\
-            else attn_pipe_body<DD, false, MODE_I8, false, NW, false, true>(p, lds, wg);      \
-        }                                                                                     \
+        if (causal) attn_pipe_body<DD, true, MODE_I8, false, NW, false, true>(p, lds, wg);    \
+        else attn_pipe_body<DD, false, MODE_I8, false, NW, false, true>(p, lds, wg);          \
     } while (0)
     if (head_dim == 64) AR_SAGE_QF(64);
     else if (head_dim == 128) AR_SAGE_QF(128);
 #undef AR_SAGE_QF
 }
 
+#if ARHIP_PART(8)
 extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_qf_long(const uint16_t *Q, const int8_t *K8, const uint16_t *V,
                                                                          void *O, const float *M, float *SQ, const float *SK,
                                                                          int N, int head_dim, int causal, int has_mask, int hq,
@@ -574,6 +597,8 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_qf_long_lens(con
     flash_sage_qf_entry<8>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
+#endif
+#if ARHIP_PART(9)
 extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_qf_mid(const uint16_t *Q, const int8_t *K8, const uint16_t *V,
                                                                            void *O, const float *M, float *SQ, const float *SK,
                                                                            int N, int head_dim, int causal, int has_mask, int hq,
@@ -593,6 +618,8 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_qf_mid_lens(c
     flash_sage_qf_entry<4>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
+#endif
+#if ARHIP_PART(10)
 extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
                                                                           void *O, const float *M, const float *SQ, const float *SK,
                                                                           int N, int head_dim, int causal, int has_mask, int hq,
@@ -612,6 +639,8 @@ extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long_lens(co
     flash_sage_long_entry<MODE_FP8>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
+#endif
+#if ARHIP_PART(11)
 extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_mid(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
                                                                             void *O, const float *M, const float *SQ, const float *SK,
                                                                             int N, int head_dim, int causal, int has_mask, int hq,
@@ -631,6 +660,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_mid_lens(
     flash_sage_long_entry<MODE_FP8, 4>(lds, Q8, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
+#endif
 // ---- Sage pre-pass (the quantiser the reference runs inside its attention kernel,
 // src/runtime/cuda_flash_sage.rs:201-223,248-278, hoisted into passes of its own) ----
 // x [B*H, N, D] f32 or bf16; block [256,1,1] for all of them.
@@ -640,6 +670,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_mid_lens(
 //   ar_sage_quant_rows_*     grid [ceil(B*H*N / (256/(D/8))), 1, 1]          x8, scales [B*H*N]
 //   ar_cast_bf16             grid [min(ceil(n/256), 16384), 1, 1]            y bf16
 // smooth != 0 subtracts mean[bh][d] first (K smoothing).
+#if ARHIP_PART(1)
 extern "C" __global__ void __launch_bounds__(256) ar_sage_kmean_partial_f32(const float *x, float *part, int N, int D, int nchunk)
 {
     k_mean_partial_body<float>(x, part, N, D, nchunk, XLayout::dense(1, N, D), blockIdx);
@@ -680,6 +711,7 @@ extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_bf16(const 
     if (smooth) quant_rows_body<uint16_t, true>(x, x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);
     else quant_rows_body<uint16_t, false>(x, x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);
 }
+#endif
 // FP8 E4M3 quantiser entries: same arguments, x8 receives E4M3 codes, scale = absmax / 448
 #define AR_QUANT_FP8(SUFFIX, T)                                                                                              \
     extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_blocks_fp8_##SUFFIX(                                     \
@@ -694,11 +726,16 @@ extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_bf16(const 
         if (smooth) quant_rows_body<T, true, true>(x, (int8_t *)x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);   \
         else quant_rows_body<T, false, true>(x, (int8_t *)x8, scales, mean, N, D, rows_total, XLayout::dense(1, N, D), blockIdx);         \
     }
+#if ARHIP_PART(1)
 AR_QUANT_FP8(f32, float)
 AR_QUANT_FP8(bf16, uint16_t)
+#endif
 #undef AR_QUANT_FP8
 
+#if ARHIP_PART(1)
 extern "C" __global__ void __launch_bounds__(256) ar_cast_bf16(const float *x, uint16_t *y, long n)
 {
     cast_bf16_body(x, y, (size_t)n, blockIdx);
 }
+
+#endif

@@ -83,6 +83,7 @@ struct AttnParams {
     int bq, bk;
     int bk_tile_shift;  // log2(bk / 64) when the K scales are tile-uniform
     int bk_key_shift;   // log2(bk) for the pipelined kernel's per-key form (bk a power of two below 64)
+    int out_f32;        // pipelined 8-bit kernels: store f32 instead of bf16
     int nq;        // query tiles per head
     int total;     // workgroups
     int lpt;       // causal: order the whole grid longest-tile-first (small grids)

@@ -880,7 +880,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     if (p.lse != nullptr && h == 0 && q_row < N) {
         p.lse[(size_t)bh * N + q_row] = (l_tot > 0.f) ? (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : NEG_SENTINEL;
     }
-    if constexpr (OUT_F32) {
+    // (f32 or bf16 output is the launch's choice, not a variant of the kernel: the two stores are a few lines at the
+    // end, and every variant of the kernel is minutes of compilation)
+    if (OUT_F32 || (MODE != MODE_BF16 && p.out_f32)) {
         if (q_row < N) {
             const size_t obase = (size_t)b * p.os[0] + (size_t)head * p.os[1] + (size_t)q_row * p.os[2];
 #pragma unroll

@@ -142,7 +142,7 @@ extern "C" int arhip_close(arhip_device *dev)
     (void)hipSetDevice(dev->ordinal);
     (void)hipStreamSynchronize(dev->stream);
     for (auto &kv : dev->modules) {
-        (void)hipModuleUnload(kv.second->mod);
+        for (hipModule_t m : kv.second->mods) (void)hipModuleUnload(m);
         delete kv.second;
     }
     for (auto &e : dev->prof_log) {
@@ -397,13 +397,40 @@ extern "C" int arhip_module_load(arhip_device *dev, const void *image, size_t le
         *module = it->second;
         return ARHIP_OK;
     }
-    // Keep a private copy of the image alive for as long as the module is loaded.
+    // An image is one code object (an ELF file), or a container of several that the build compiles side by side
+    // and that are looked up as one: "ARHIPKO1", uint32 count, uint32 0, then per part uint64 size and the part's
+    // bytes padded to a multiple of 16.
+    std::vector<std::pair<const char *, size_t>> parts;
+    const char *bytes = (const char *)image;
+    if (len >= 16 && memcmp(bytes, "ARHIPKO1", 8) == 0) {
+        uint32_t count;
+        memcpy(&count, bytes + 8, 4);
+        size_t at = 16;
+        for (uint32_t i = 0; i < count; ++i) {
+            uint64_t sz = 0;
+            ARHIP_REQUIRE(at + 8 <= len, "arhip_module_load: truncated container (part %u of %u)", i, count);
+            memcpy(&sz, bytes + at, 8);
+            at += 8;
+            ARHIP_REQUIRE(sz > 0 && sz <= len - at, "arhip_module_load: truncated container (part %u of %u)", i, count);
+            parts.emplace_back(bytes + at, (size_t)sz);
+            at += (size_t)((sz + 15) & ~(uint64_t)15);
+        }
+        ARHIP_REQUIRE(!parts.empty(), "arhip_module_load: empty container");
+    } else {
+        parts.emplace_back(bytes, len);
+    }
+    // Keep a private copy of every part alive for as long as its module is loaded.
     arhip_module_entry *e = new arhip_module_entry();
-    e->image.assign((const char *)image, (const char *)image + len);
-    hipError_t err = hipModuleLoadData(&e->mod, e->image.data());
-    if (err != hipSuccess) {
-        delete e;
-        return arhip_fail(ARHIP_EHIP, "hipModuleLoadData failed: %s", hipGetErrorString(err));
+    for (auto &pt : parts) {
+        e->images.emplace_back(pt.first, pt.first + pt.second);
+        hipModule_t mod = nullptr;
+        hipError_t err = hipModuleLoadData(&mod, e->images.back().data());
+        if (err != hipSuccess) {
+            for (hipModule_t m : e->mods) (void)hipModuleUnload(m);
+            delete e;
+            return arhip_fail(ARHIP_EHIP, "hipModuleLoadData failed: %s", hipGetErrorString(err));
+        }
+        e->mods.push_back(mod);
     }
     dev->modules[key] = e;
     *module = e;
@@ -517,7 +544,15 @@ extern "C" int arhip_launch(arhip_device *dev, void *module, const char *name,
     hipFunction_t fn;
     auto it = m->fns.find(name);
     if (it == m->fns.end()) {
-        ARHIP_HIP(hipModuleGetFunction(&fn, m->mod, name));
+        hipError_t err = hipErrorNotFound;
+        for (hipModule_t mod : m->mods) {
+            err = hipModuleGetFunction(&fn, mod, name);
+            if (err == hipSuccess) break;
+        }
+        (void)hipGetLastError();  // a miss in an earlier part of a container is not an error of this launch
+        if (err != hipSuccess) {
+            return arhip_fail(ARHIP_EHIP, "arhip_launch: no kernel named %s in the module: %s", name, hipGetErrorString(err));
+        }
         m->fns[name] = fn;
     } else {
         fn = it->second;

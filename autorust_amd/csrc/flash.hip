@@ -6,7 +6,7 @@
 // (src/runtime/cuda_flash_sage.rs:452-485).
 #include "arhip_internal.h"
 #include "attn_fwd.h"
-#include "attn_pipe.h"
+#include "pipe_launch.h"
 #include "flash_bwd_f32.h"
 #include "flash_f32.h"
 
@@ -64,16 +64,9 @@ static void launch_attn(hipStream_t stream, const AttnParams &p, bool causal, bo
         hipLaunchKernelGGL((attn_fwd_kernel<D, NW, false, false, MODE, PER_KEY, OUT_F32, DBG>), grid, block, 0, stream, p);
 }
 
-// The software-pipelined kernel (no additive mask, tile-uniform K scales): 8 waves per workgroup, or 4
-// (two workgroups per compute unit) where a workgroup sees few tiles.
-template <int D, int MODE, bool OUT_F32, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
-static void launch_pipe(hipStream_t stream, const AttnParams &p, bool causal)
-{
-    const dim3 grid((unsigned)p.total), block(NW * 64);
-    if (causal) hipLaunchKernelGGL((attn_pipe_kernel<D, true, MODE, OUT_F32, NW, PER_KEY, QFUSE>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((attn_pipe_kernel<D, false, MODE, OUT_F32, NW, PER_KEY, QFUSE>), grid, block, 0, stream, p);
-}
-
+// The software-pipelined kernel (no additive mask): 8 waves per workgroup, or 4 (two workgroups per compute
+// unit) where a workgroup sees few tiles.  Its variants are compiled in translation units of their own
+// (pipe_launch.h).
 // Which of the two: 128 queries per workgroup hide a workgroup's prologue and epilogue under its
 // neighbour's tiles and fill the chip with fewer heads, but request every K/V tile twice as often and
 // keep only one tile in flight.  Two workgroups of equal length that start together stay in step and
@@ -232,15 +225,13 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
     p.total = (int)(p.nq * B * Hq);
     p.lpt = p.total <= 16 * dev->cus;  // few workgroups per CU: balance them globally
     if (int rc = t.begin()) return rc;
-    if (D == 64) {
-        if (pipe && nw == 4) launch_pipe<64, MODE_BF16, false, 4>(dev->stream, p, c);
-        else if (pipe) launch_pipe<64, MODE_BF16, false>(dev->stream, p, c);
-        else if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
+    if (pipe) {
+        launch_pipe_bf16(dev->stream, p, (int)D, c, nw);
+    } else if (D == 64) {
+        if (nw == 1) launch_attn<64, 1, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
         else launch_attn<64, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
     } else {
-        if (pipe && nw == 4) launch_pipe<128, MODE_BF16, false, 4>(dev->stream, p, c);
-        else if (pipe) launch_pipe<128, MODE_BF16, false>(dev->stream, p, c);
-        else launch_attn<128, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
+        launch_attn<128, 4, MODE_BF16, false, false, false, true>(dev->stream, p, c, hm);
     }
     arhip_note_selected(ARHIP_K_FLASH_BF16);
     return t.end();
@@ -300,6 +291,7 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
     const bool dbg = dbg_logits != nullptr;
     ARHIP_REQUIRE(!(fp8 && dbg), "arhip_sage_fwd_fp8: the logits export is an int8 facility");
     const bool c = causal != 0, hm = mask != nullptr, f32o = out_dtype == ARHIP_F32;
+    p.out_f32 = f32o;
     // K scales that are uniform over a 64-key tile (bk = 64 * 2^n) take the fast kernel; anything
     // else, including the reference's per-key scales (bk == 1), stages the tile's scales in LDS
     int shift = 0;
@@ -341,45 +333,24 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
         if (dbg) {                                                                                     \
             if (per_key) SAGE_V(DD, 4, true, true, false);                                             \
             else SAGE_V(DD, 4, false, true, false);                                                    \
-        } else if (pipe && pipe_keys) {                                                                \
-            if (pipe4 && f32o) launch_pipe<DD, MODE_I8, true, 4, true>(dev->stream, p, c);             \
-            else if (pipe4) launch_pipe<DD, MODE_I8, false, 4, true>(dev->stream, p, c);               \
-            else if (f32o) launch_pipe<DD, MODE_I8, true, 8, true>(dev->stream, p, c);                 \
-            else launch_pipe<DD, MODE_I8, false, 8, true>(dev->stream, p, c);                          \
-        } else if (per_key) SAGE_V(DD, 4, true, false, true);                                          \
-        else if (pipe4 && f32o) launch_pipe<DD, MODE_I8, true, 4>(dev->stream, p, c);                  \
-        else if (pipe4) launch_pipe<DD, MODE_I8, false, 4>(dev->stream, p, c);                         \
-        else if (nw == 4) SAGE_V(DD, 4, false, false, true);                                           \
-        else if (f32o) launch_pipe<DD, MODE_I8, true>(dev->stream, p, c);                              \
-        else launch_pipe<DD, MODE_I8, false>(dev->stream, p, c);                                       \
+        } else if (pipe && pipe_keys) launch_pipe_i8_keys(dev->stream, p, DD, c, nw);                  \
+        else if (per_key) SAGE_V(DD, 4, true, false, true);                                            \
+        else if (pipe) launch_pipe_i8(dev->stream, p, DD, c, nw);                                      \
+        else SAGE_V(DD, 4, false, false, true);                                                        \
     } while (0)
 #define SAGE_F(DD, PK)                                                                                 \
     do {                                                                                               \
         if (f32o) launch_attn<DD, 4, MODE_FP8, PK, true, false, true>(dev->stream, p, c, hm);          \
         else launch_attn<DD, 4, MODE_FP8, PK, false, false, true>(dev->stream, p, c, hm);              \
     } while (0)
-#define SAGE_FP(DD, NWW, PK)                                                                          \
-    do {                                                                                               \
-        if (f32o) launch_pipe<DD, MODE_FP8, true, NWW, PK>(dev->stream, p, c);                         \
-        else launch_pipe<DD, MODE_FP8, false, NWW, PK>(dev->stream, p, c);                             \
-    } while (0)
-#define SAGE_FPD(NWW, PK)                                                                              \
-    do {                                                                                               \
-        if (D == 64) SAGE_FP(64, NWW, PK);                                                             \
-        else SAGE_FP(128, NWW, PK);                                                                    \
-    } while (0)
     if (fp8 && pipe) {
-        if (pipe4 && pipe_keys) SAGE_FPD(4, true);
-        else if (pipe4) SAGE_FPD(4, false);
-        else if (pipe_keys) SAGE_FPD(8, true);
-        else SAGE_FPD(8, false);
+        if (pipe_keys) launch_pipe_fp8_keys(dev->stream, p, (int)D, c, nw);
+        else launch_pipe_fp8(dev->stream, p, (int)D, c, nw);
     } else if (fp8) {
         if (D == 64) { if (per_key) SAGE_F(64, true); else SAGE_F(64, false); }
         else { if (per_key) SAGE_F(128, true); else SAGE_F(128, false); }
     } else if (D == 64) SAGE_D(64);
     else SAGE_D(128);
-#undef SAGE_FPD
-#undef SAGE_FP
 #undef SAGE_F
 #undef SAGE_D
 #undef SAGE_V
@@ -418,7 +389,8 @@ extern "C" int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const
     p.bk_tile_shift = shift;
     p.bk_key_shift = -1;
     p.scale = scale;
-    const bool c = causal != 0, f32o = out_dtype == ARHIP_F32;
+    const bool c = causal != 0;
+    p.out_f32 = out_dtype == ARHIP_F32;
     const int nw = pipe_wants_4_waves(dev, B * Hq, N, D, c, kv_len != nullptr) ? 4 : 8;
     p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
     p.total = (int)(p.nq * B * Hq);
@@ -426,14 +398,7 @@ extern "C" int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const
     arhip_call_timer t{dev, wait, secs};
     t.kernel = ARHIP_K_SAGE;
     if (int rc = t.begin()) return rc;
-#define SAGE_QF(DD, NWW)                                                                               \
-    do {                                                                                               \
-        if (f32o) launch_pipe<DD, MODE_I8, true, NWW, false, true>(dev->stream, p, c);                 \
-        else launch_pipe<DD, MODE_I8, false, NWW, false, true>(dev->stream, p, c);                     \
-    } while (0)
-    if (D == 64) { if (nw == 4) SAGE_QF(64, 4); else SAGE_QF(64, 8); }
-    else { if (nw == 4) SAGE_QF(128, 4); else SAGE_QF(128, 8); }
-#undef SAGE_QF
+    launch_pipe_i8_qf(dev->stream, p, (int)D, c, nw);
     arhip_note_selected(ARHIP_K_SAGE);
     return t.end();
 }

@@ -1,0 +1,6 @@
+// The pipelined int8 attention kernel that quantises its bf16 queries in its prologue.
+#define PIPE_FN launch_pipe_i8_qf
+#define PIPE_MODE MODE_I8
+#define PIPE_KEYS false
+#define PIPE_QF true
+#include "pipe_tu.h"

@@ -106,8 +106,10 @@ int arhip_graph_destroy(arhip_device *dev, void *graph_exec);
 /* ---- generic host-kernel launch: `Compiled::run_host_kernel`,
  *      src/runtime/device.rs:383-402; argument encoding of
  *      src/runtime/ops_cuda.rs:930-1019 (`CudaProgram::call`) ----
- * image: a gfx950 code object (hipcc --genco).  Modules are cached per device
- * by content hash.  args: nbufs device pointers followed by nvals scalars;
+ * image: a gfx950 code object (hipcc --genco), or a container of several that are looked up as
+ * one: "ARHIPKO1", uint32 count, uint32 0, then per code object uint64 size and its bytes padded
+ * to a multiple of 16 (autorust_amd/attn_kernels.hsaco is such a file: its entry points compile as
+ * eleven code objects side by side).  Modules are cached per device by content hash.  args: nbufs device pointers followed by nvals scalars;
  * val_bits[i] in {32, 64} narrows vals[i] like the reference's signature
  * dtype does.  grid is in blocks. */
 int arhip_module_load(arhip_device *dev, const void *image, size_t len, void **module);

@@ -5,8 +5,10 @@
  * This is the second face of the boundary: hosts that launch kernels by name, the way the
  * reference's `HostCall{src, name, signature, bufs, global, local, vals}` ->
  * `Compiled::run_host_kernel` -> `Prog::call` does (src/engine/session.rs:210-256,
- * src/runtime/device.rs:383-402), load the code object with arhip_module_load (or
- * hipModuleLoadData) and launch these with arhip_launch (or hipModuleLaunchKernel).
+ * src/runtime/device.rs:383-402), load the file with arhip_module_load and launch these with
+ * arhip_launch.  (The file is a container of eleven code objects, see arhip_module_load in
+ * arhip.h; a host that wants hipModuleLoadData / hipModuleLaunchKernel itself loads each part,
+ * or builds csrc/attn_entry.hip without -DARHIP_ENTRY_PART as one plain code object.)
  * Arguments are device pointers followed by scalars, in the reference's order
  * (src/runtime/cuda_flash_bf16.rs:226-231, 550-599):
  *
