@@ -225,6 +225,9 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // reloaded from a spill lane) and a memory instruction reading it: the compiler pads neither
     // for inline assembly, so the assembly carries the wait states itself (s_mov + s_nop 3).
     auto issue_tile = [&](int tile) __attribute__((always_inline)) {
+        // RINGS waits for everything in flight at the end of every tile: a transfer past the last tile (which would
+        // deliver zeros) is a memory round trip the last two tiles of a workgroup would wait for
+        if (RINGS && tile >= ntiles) return;
         const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
         const uint32_t dst_k = lds0 + k_base(tile), dst_v = lds0 + v_base(tile);
         if constexpr (PER_KEY) {
