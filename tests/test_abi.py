@@ -85,3 +85,27 @@ def test_code_object_is_built_and_names_every_entry_point():
     image = open(_lib.KERNELS_PATH, "rb").read()
     for n in names:
         assert n.encode() + b"\0" in image or n.encode() in image, n
+
+
+def test_code_object_file_is_a_container_of_elf_parts():
+    """attn_kernels.hsaco holds the entry points as several code objects (they compile side by side): "ARHIPKO1",
+    count, then per part its size and bytes padded to 16; arhip_module_load takes the file as a whole.  Every part
+    is a gfx950 code object and every named kernel lives in exactly one of them."""
+    import struct
+    image = open(_lib.KERNELS_PATH, "rb").read()
+    assert image[:8] == b"ARHIPKO1"
+    count, zero = struct.unpack_from("<II", image, 8)
+    assert count == 11 and zero == 0
+    at, parts = 16, []
+    for _ in range(count):
+        (size,) = struct.unpack_from("<Q", image, at)
+        at += 8
+        parts.append(image[at:at + size])
+        # hipcc --genco writes an offload bundle around the ELF image; hipModuleLoadData takes either
+        assert parts[-1].startswith((b"\x7fELF", b"__CLANG_OFFLOAD_BUNDLE__")) and len(parts[-1]) == size
+        at += (size + 15) & ~15
+    assert at == len(image)
+    text = open(os.path.join(ROOT, "include", "arhip_kernels.h")).read()
+    for n in re.findall(r'#define ARHIP_KERNEL_\w+ "(\w+)"', text):
+        homes = [i for i, part in enumerate(parts) if n.encode() + b".kd\0" in part]
+        assert len(homes) == 1, (n, homes)
