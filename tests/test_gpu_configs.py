@@ -124,6 +124,14 @@ def _sage_config(dev, B, H, N, D, causal, sigma, outliers, seed, rows_per_head_e
         do = bufs.new(q.size * 2, zero=False)
         dev.sage_fwd(q8, k8, sq, sk, dv, do, B, H, H, N, D, bq, bk, out_dtype=BF16, causal=causal)
         got = synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+        if bq == 128 and bk % 64 == 0:
+            # the same launch with the Q quantiser in the attention kernel's prologue (what the host mirror and
+            # bench.py run for bf16 tensors): its scales and its output are those of the two launches above, bit for bit
+            do2, sq2 = bufs.new(q.size * 2, zero=False), bufs.new(B * H * nqb * 4)
+            dev.sage_fwd_qfused(dq, k8, sk, dv, do2, B, H, H, N, D, bk, out_dtype=BF16, sq_out=sq2, causal=causal)
+            assert np.array_equal(sq2.copyout(np.float32, (B, H, nqb)), sq.copyout(np.float32, (B, H, nqb)))
+            assert np.array_equal(do2.copyout(np.uint16, q.shape), do.copyout(np.uint16, q.shape))
+            do2.free()
         g_q8, g_k8 = q8.copyout(np.int8, q.shape), k8.copyout(np.int8, k.shape)
         g_sq, g_sk = sq.copyout(np.float32, (B, H, nqb)), sk.copyout(np.float32, (B, H, nkb))
         g_mean = mean.copyout(np.float32, (B, H, D))
