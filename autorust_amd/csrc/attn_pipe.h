@@ -1,7 +1,8 @@
-// Fused attention forward for long sequences on gfx950: the software-pipelined variant of
-// attn_fwd_kernel (attn_fwd.h) for launches without an additive mask, per-key scales or the
-// logits export.  Same arithmetic, same MFMA decomposition (S^T = K . Q^T, one query per lane,
-// O^T += V^T . P^T), different plumbing:
+// Fused attention forward on gfx950: the software-pipelined kernel, which serves every launch without an
+// additive mask or the logits export (attn_fwd_kernel, attn_fwd.h, keeps those), bf16, int8 and FP8 E4M3
+// operands, K scales over whole 64-key tiles or per key (PER_KEY), the Q quantiser of the int8 path inside its
+// prologue on request (QFUSE).  Same arithmetic and MFMA decomposition as attn_fwd_kernel (S^T = K . Q^T, one
+// query per lane, O^T += V^T . P^T), different plumbing:
 //
 //   HBM -> LDS   K and V tiles of 64 keys go straight to LDS (buffer_load ... lds, 16 bytes per
 //                lane, no registers in between), four stages deep, so a tile is requested three
@@ -36,7 +37,7 @@
 // NW = 4 is the variant for launches whose workgroups see few tiles (short or causal sequences): 128
 // queries per workgroup and at most 80 KB of LDS, so that a compute unit holds two workgroups and one's
 // prologue and epilogue (first transfers, output store, the gap to the next workgroup) run under the
-// other's tiles.  K and V then live in rings of their own, K two tiles deep and V three: while tile t is
+// other's tiles.  K and V then live in rings of their own (attn_pipe_rings), K two tiles deep and V three: while tile t is
 // computed the wave reads K(t+1), V(t) and V(t+1) from LDS (K(t) went into registers during tile t-1),
 // and tile t+2 is on its way.  The rare reference move takes the block's logits from their registers
 // instead of recomputing them from K(t), which this ring no longer holds.
