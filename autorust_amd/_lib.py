@@ -72,10 +72,12 @@ SIGNATURES = {
     "arhip_sage_quant_static": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),
     "arhip_cast_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, _pd]),
+    "arhip_sage_prep_kv_rows": (c_int, [c_void_p] * 6 + [c_int64] * 4 + [c_int, _pd]),
     "arhip_sage_quant_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),
     "arhip_sage_fwd_fp8": (c_int, [c_void_p] * 9 + [c_int64] * 7 + [c_int, c_int, c_float, c_int, _pd]),
     "arhip_sage_fwd_qfused": (c_int, [c_void_p] * 9 + [c_int64] * 6 + [c_int, c_int, c_float, c_int, _pd]),
+    "arhip_sage_fwd_qfused_rows": (c_int, [c_void_p] * 9 + [c_int64] * 6 + [c_int, c_int, c_float, c_int, _pd]),
     "arhip_sage_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_float,
                                c_void_p, ctypes.POINTER(ctypes.c_int32), c_int, _pd]),

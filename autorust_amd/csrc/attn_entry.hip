@@ -49,7 +49,7 @@
 // last: it switches floating-point contraction off for the rest of the file
 #include "sage_quant_kernels.h"
 
-// The entry points compile as eleven code objects side by side (-DARHIP_ENTRY_PART=1 ... 11; the build packs them into
+// The entry points compile as thirteen code objects side by side (-DARHIP_ENTRY_PART=1 ... 13; the build packs them into
 // one file that arhip_module_load takes as a whole): the pipelined kernels are several thousand instructions per
 // variant, minutes of compilation per entry.  Without the macro this file is one code object with all of them.
 #ifndef ARHIP_ENTRY_PART
@@ -619,6 +619,77 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_qf_mid_lens(c
 }
 
 #endif
+// ar_flash_sage_qr_long / _mid: the reference's convention in one launch.  Q holds f32 values and is quantised row by
+// row in the prologue; SQ [b*hq, n] RECEIVES the scales (bq must be 1); K8 / SK as from the K quantiser with bk a
+// power of two below 64 (bk = 1: a scale per key).  Same grid and block as ar_flash_sage_long / _mid.
+template <int NW>
+__device__ __forceinline__ void flash_sage_qr_entry(unsigned char *lds, const float *Q, const void *K8, const uint16_t *V, void *O,
+                                                    const float *M, const int *L, float *SQ, const float *SK, int N, int head_dim,
+                                                    int causal, int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
+{
+    int key_shift = 0;
+    while ((1 << key_shift) < bk) ++key_shift;
+    if (has_mask || bk >= 64 || (1 << key_shift) != bk || bq != 1) return;  // refused on the host
+    AttnParams p = dense_params(Q, K8, V, O, M, N, head_dim, 0, hq, hkv, L);
+    p.sk = SK;
+    p.sq_out = SQ;
+    p.bq = bq; p.bk = bk;
+    p.bk_tile_shift = 0;
+    p.bk_key_shift = key_shift;
+    p.out_f32 = out_f32;
+    const int wg = linear_wg();
+#define AR_SAGE_QR(DD)                                                                       \
+    do {                                                                                     \
+        if (causal) attn_pipe_body<DD, true, MODE_I8, false, NW, true, true>(p, lds, wg);    \
+        else attn_pipe_body<DD, false, MODE_I8, false, NW, true, true>(p, lds, wg);          \
+    } while (0)
+    if (head_dim == 64) AR_SAGE_QR(64);
+    else if (head_dim == 128) AR_SAGE_QR(128);
+#undef AR_SAGE_QR
+}
+
+#if ARHIP_PART(12)
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_qr_long(const float *Q, const int8_t *K8, const uint16_t *V,
+                                                                         void *O, const float *M, float *SQ, const float *SK,
+                                                                         int N, int head_dim, int causal, int has_mask, int hq,
+                                                                         int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 8, true, true>()];
+    flash_sage_qr_entry<8>(lds, Q, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_qr_long_lens(const float *Q, const int8_t *K8, const uint16_t *V,
+                                                                              void *O, const float *M, const int *L, float *SQ,
+                                                                              const float *SK, int N, int head_dim, int causal,
+                                                                              int has_mask, int hq, int hkv, int bq, int bk,
+                                                                              int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 8, true, true>()];
+    flash_sage_qr_entry<8>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+#endif
+#if ARHIP_PART(13)
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_qr_mid(const float *Q, const int8_t *K8, const uint16_t *V,
+                                                                           void *O, const float *M, float *SQ, const float *SK,
+                                                                           int N, int head_dim, int causal, int has_mask, int hq,
+                                                                           int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4, true, true>()];
+    flash_sage_qr_entry<4>(lds, Q, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_qr_mid_lens(const float *Q, const int8_t *K8, const uint16_t *V,
+                                                                                void *O, const float *M, const int *L, float *SQ,
+                                                                                const float *SK, int N, int head_dim, int causal,
+                                                                                int has_mask, int hq, int hkv, int bq, int bk,
+                                                                                int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4, true, true>()];
+    flash_sage_qr_entry<4>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+#endif
 #if ARHIP_PART(10)
 extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_long(const uint8_t *Q8, const uint8_t *K8, const uint16_t *V,
                                                                           void *O, const float *M, const float *SQ, const float *SK,
@@ -736,6 +807,15 @@ AR_QUANT_FP8(bf16, uint16_t)
 extern "C" __global__ void __launch_bounds__(256) ar_cast_bf16(const float *x, uint16_t *y, long n)
 {
     cast_bf16_body(x, y, (size_t)n, blockIdx);
+}
+
+// ar_sage_quant_rows_cast_f32: ar_sage_quant_rows_f32 (smooth = 0) on K and ar_cast_bf16 on V in one launch.
+//   grid [row_blocks + cast_blocks, 1, 1] with row_blocks = ceil(B*Hkv*N / (256/(D/8))), cast_blocks = min(ceil(nv/256), 16384)
+extern "C" __global__ void __launch_bounds__(256) ar_sage_quant_rows_cast_f32(const float *k, int8_t *k8, float *scales,
+                                                                               const float *v, uint16_t *vb, int N, int D,
+                                                                               long rows_total, long nv, int row_blocks)
+{
+    quant_rows_cast_body(k, k8, scales, v, vb, N, D, rows_total, nv, row_blocks, blockIdx);
 }
 
 #endif

@@ -85,13 +85,14 @@ constexpr bool attn_pipe_rings()
 // ring of two K tiles and one of three V tiles (attn_pipe_rings).  PER_KEY (a scale per key, or per block of fewer than
 // 64 keys): behind the tiles, a ring of four times 64 raw key scales and, per wave, two times 64 pairs of
 // derived factors.
-// QFUSE (Q arrives as bf16 and is quantised in the prologue): 256 bytes for the exchange of the waves' maxima.
+// QFUSE (Q is quantised in the prologue): with scales over blocks of 128 queries, 256 bytes for the exchange of the
+// waves' maxima.
 template <int D, int MODE, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 constexpr int attn_pipe_lds_bytes()
 {
     constexpr bool R = attn_pipe_rings<D, MODE, NW>();
     return 4096 * ((R ? 2 : 4) * (D * ((MODE != MODE_BF16) ? 1 : 2) / 64) + (R ? 3 : 4) * (D * 2 / 64)) +
-           (PER_KEY ? 1024 + NW * 1024 : 0) + (QFUSE ? 256 : 0);
+           (PER_KEY ? 1024 + NW * 1024 : 0) + ((QFUSE && !PER_KEY) ? 256 : 0);
 }
 
 // workgroup index -> (batch * heads + head, query tile of 256), as in attn_fwd_kernel
@@ -112,14 +113,16 @@ __device__ __forceinline__ void pipe_work_item(const AttnParams &p, int wg, int 
 
 // The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
 // aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below.
-// QFUSE (int8, Q scales over blocks of 128 queries, K scales over whole tiles): p.q holds bf16 values and the
-// prologue is the quantiser of sage_quant_kernels.h for this workgroup's queries, operation for operation
-// (absmax over the block, scale = absmax / 127 or 1, x8 = clamp(rint(x * (1 / scale)), +-127)), so the result is
-// bit for bit that of quantising first; p.sq_out / p.q8_out, where not null, receive the scales and the codes.
+// QFUSE (int8): the prologue is the quantiser of sage_quant_kernels.h for this workgroup's queries, operation for
+// operation (absmax, scale = absmax / 127 or 1, x8 = clamp(rint(x * (1 / scale)), +-127)), so the result is bit for bit
+// that of quantising first; p.sq_out / p.q8_out, where not null, receive the scales and the codes.  Two forms: with K
+// scales over whole tiles, p.q holds bf16 values and a scale covers a block of 128 queries; with PER_KEY, p.q holds
+// f32 values and every query has its own scale (the reference's convention, src/runtime/cuda_flash_sage.rs:201-223).
 template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
-    static_assert(!QFUSE || (BIAS && !PER_KEY), "the fused Q quantiser: int8, K scales over whole tiles");
+    static_assert(!QFUSE || BIAS, "the fused Q quantiser is an int8 device");
+    constexpr bool QROWS = QFUSE && PER_KEY;  // f32 queries, a scale per query
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
     static_assert(!PER_KEY || BIAS || MODE == MODE_FP8, "per-key scales: int8 (on the biased accumulators) and FP8");
     static_assert(NW == 8 || NW == 4, "8 waves (one workgroup per CU) or 4 (two)");
@@ -343,7 +346,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     // exponent factor of the keys of tile t (in the group of tile `it` or the next one): scale log2(e),
     // times sq sk for int8 (s = (float)acc * ((sq * sk) * scale), src/runtime/cuda_flash_sage.rs:315-322)
     // PER_KEY: the keys' own scales are applied per logit (see convert_sk); what is left is the lane's factor
-    const float sq_c = (sq_lane * p.scale) * LOG2E;
+    float sq_c = (sq_lane * p.scale) * LOG2E;  // (QFUSE: set again once the prologue has the scale)
     auto tile_c = [&](int t, int it) __attribute__((always_inline)) -> float {
         if constexpr (PER_KEY) {
             return sq_c;
@@ -694,8 +697,15 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     static_for<0, AHEAD>([&](auto ti) __attribute__((always_inline)) { issue_tile(decltype(ti)::value); });
     // Q operand, resident in registers.  Everything in flight is awaited here once, Q included, so
     // that no wait for a global load is left inside the loops.
-    uint4 qraw[QFUSE ? KSTEPS : 1][2];  // QFUSE: the 16 bf16 values behind each 16-byte piece of the operand
-    if constexpr (QFUSE) {
+    // QFUSE: the 16 values (bf16: 2 x 16 bytes, f32: 4 x 16 bytes) behind each 16-byte piece of the operand
+    uint4 qraw[QFUSE ? KSTEPS : 1][QROWS ? 4 : 2];
+    if constexpr (QROWS) {
+        const float *qb = (const float *)p.q + (size_t)b * p.qs[0] + (size_t)head * p.qs[1] + (size_t)min(q_row, N - 1) * p.qs[2];
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) qraw[s][c] = *(const uint4 *)(qb + s * 32 + h * 16 + c * 4);
+    } else if constexpr (QFUSE) {
         const uint16_t *qb = (const uint16_t *)p.q + (size_t)b * p.qs[0] + (size_t)head * p.qs[1] + (size_t)min(q_row, N - 1) * p.qs[2];
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
@@ -728,9 +738,14 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     if constexpr (QFUSE) {
         // bf16 -> f32 is a shift; the quantiser's own operations from there on
         auto val = [&](int s, int e) __attribute__((always_inline)) -> float {
-            const uint4 w = qraw[s][e >> 3];
-            const uint32_t u = (e & 7) < 2 ? w.x : (e & 7) < 4 ? w.y : (e & 7) < 6 ? w.z : w.w;
-            return __uint_as_float((e & 1) ? (u & 0xffff0000u) : (u << 16));
+            if constexpr (QROWS) {
+                const uint4 w = qraw[s][e >> 2];
+                return __uint_as_float((e & 3) == 0 ? w.x : (e & 3) == 1 ? w.y : (e & 3) == 2 ? w.z : w.w);
+            } else {
+                const uint4 w = qraw[s][e >> 3];
+                const uint32_t u = (e & 7) < 2 ? w.x : (e & 7) < 4 ? w.y : (e & 7) < 6 ? w.z : w.w;
+                return __uint_as_float((e & 1) ? (u & 0xffff0000u) : (u << 16));
+            }
         };
         float mx = 0.f;
 #pragma unroll
@@ -738,15 +753,17 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmaxf(mx, fabsf(val(s, e)));
         mx = xhalf_max(mx);  // the two lanes of a query
-#pragma unroll
-        for (int o = 16; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
         float *red = (float *)(lds + QF_RED);
-        if (lane == 0) red[wave] = mx;
-        __syncthreads();
-        // a block of 128 queries is four waves (a block past the last query holds copies of the last row and is
-        // neither used nor written back)
-        const int w0 = wave & ~3;
-        mx = fmaxf(fmaxf(red[w0], red[w0 + 1]), fmaxf(red[w0 + 2], red[w0 + 3]));
+        if constexpr (!QROWS) {
+#pragma unroll
+            for (int o = 16; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            if (lane == 0) red[wave] = mx;
+            __syncthreads();
+            // a block of 128 queries is four waves (a block past the last query holds copies of the last row and is
+            // neither used nor written back)
+            const int w0 = wave & ~3;
+            mx = fmaxf(fmaxf(red[w0], red[w0 + 1]), fmaxf(red[w0 + 2], red[w0 + 3]));
+        }
         const float scale = (mx > 0.f) ? mx / 127.0f : 1.f;
         const float inv = 1.f / scale;
 #pragma unroll
@@ -761,13 +778,18 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             qreg[s] = make_uint4(w[0], w[1], w[2], w[3]);
         }
         sq_lane = scale;
-        // the workgroup's largest Q scale, for the grid below: every wave reads every wave's maximum
-        float wg_mx = red[0];
+        sq_c = (sq_lane * p.scale) * LOG2E;
+        if constexpr (QROWS) {
+            if (p.sq_out != nullptr && h == 0 && q_row < N) p.sq_out[(size_t)bh * N + q_row] = scale;
+        } else {
+            // the workgroup's largest Q scale, for the grid below: every wave reads every wave's maximum
+            float wg_mx = red[0];
 #pragma unroll
-        for (int w = 1; w < NW; ++w) wg_mx = fmaxf(wg_mx, red[w]);
-        mq = (wg_mx > 0.f) ? wg_mx / 127.0f : 1.f;
-        const int blk = q_row >> 7, nqb = (N + 127) >> 7;
-        if (p.sq_out != nullptr && lane == 0 && (wave & 3) == 0 && blk < nqb) p.sq_out[(size_t)bh * nqb + blk] = scale;
+            for (int w = 1; w < NW; ++w) wg_mx = fmaxf(wg_mx, red[w]);
+            mq = (wg_mx > 0.f) ? wg_mx / 127.0f : 1.f;
+            const int blk = q_row >> 7, nqb = (N + 127) >> 7;
+            if (p.sq_out != nullptr && lane == 0 && (wave & 3) == 0 && blk < nqb) p.sq_out[(size_t)bh * nqb + blk] = scale;
+        }
         if (p.q8_out != nullptr && q_row < N) {
             int8_t *dst = p.q8_out + ((size_t)bh * N + q_row) * D;
 #pragma unroll

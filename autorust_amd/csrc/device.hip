@@ -476,6 +476,10 @@ const named_entry NAMED[] = {
     {"ar_flash_sage_qf_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
     {"ar_flash_sage_qf_mid", 7, 9, 256, 128, false, true, true, 0, false},
     {"ar_flash_sage_qf_mid_lens", 8, 9, 256, 128, false, true, true, 0, false},
+    {"ar_flash_sage_qr_long", 7, 9, 512, 256, false, true, true, 0, false},
+    {"ar_flash_sage_qr_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
+    {"ar_flash_sage_qr_mid", 7, 9, 256, 128, false, true, true, 0, false},
+    {"ar_flash_sage_qr_mid_lens", 8, 9, 256, 128, false, true, true, 0, false},
     {"ar_flash_sage_fp8_mid", 7, 9, 256, 128, false, true, true, 0, false},
     {"ar_flash_sage_fp8_mid_lens", 8, 9, 256, 128, false, true, true, 0, false},
     {"ar_flash_sage_fp8_long", 7, 9, 512, 256, false, true, true, 0, false},
@@ -521,6 +525,9 @@ int check_named_entry(const char *name, const unsigned grid[3], const unsigned b
             const int64_t bk = vals[7];
             ARHIP_REQUIRE((bk & (bk - 1)) == 0, "arhip_launch: %s needs K scales over a power of two of keys (bk = 2^j), got bk = %lld",
                           name, (long long)bk);
+            if (strstr(name, "_qr_") != nullptr)
+                ARHIP_REQUIRE(vals[6] == 1 && bk < 64, "arhip_launch: %s quantises Q row by row and takes K scales over "
+                              "a power of two of keys below 64, got bq = %lld, bk = %lld", name, (long long)vals[6], (long long)bk);
             if (strstr(name, "_qf_") != nullptr)
                 ARHIP_REQUIRE(vals[6] == 128 && bk >= 64, "arhip_launch: %s quantises Q over blocks of 128 queries and takes K scales "
                               "over whole 64-key tiles, got bq = %lld, bk = %lld", name, (long long)vals[6], (long long)bk);

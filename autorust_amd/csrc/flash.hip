@@ -403,6 +403,51 @@ extern "C" int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const
     return t.end();
 }
 
+// The reference's own convention in one attention launch: f32 queries quantised row by row inside the kernel
+// (src/runtime/cuda_flash_sage.rs:201-223), K scales per key (or per power of two of keys below 64).
+extern "C" int arhip_sage_fwd_qfused_rows(arhip_device *dev, const float *q, const int8_t *k8, const float *sk,
+                                          const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
+                                          int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
+                                          int causal, int out_dtype, float scale, int wait, double *secs)
+{
+    if (int rc = check_common("arhip_sage_fwd_qfused_rows", dev, q, k8, v, o, nullptr, B, Hq, Hkv, N, D)) return rc;
+    ARHIP_REQUIRE(sk, "arhip_sage_fwd_qfused_rows: null scale pointer");
+    ARHIP_REQUIRE(out_dtype == ARHIP_F32 || out_dtype == ARHIP_BF16, "arhip_sage_fwd_qfused_rows: out_dtype %d", out_dtype);
+    int key_shift = 0;
+    while (((int64_t)1 << key_shift) < bk) ++key_shift;
+    ARHIP_REQUIRE(bk >= 1 && bk < 64 && ((int64_t)1 << key_shift) == bk,
+                  "arhip_sage_fwd_qfused_rows: K scales over a power of two of keys below 64 (bk = 1 ... 32), got bk = %lld", (long long)bk);
+    ARHIP_REQUIRE(pipe_addressable(N, D, 2), "arhip_sage_fwd_qfused_rows: (N + 320) * D * 2 must stay below 2^31 (N = %lld)", (long long)N);
+    ARHIP_REQUIRE(q8_out == nullptr || arhip_aligned16(q8_out), "arhip_sage_fwd_qfused_rows: q8_out must be 16-byte aligned");
+    ARHIP_HIP(hipSetDevice(dev->ordinal));
+    AttnParams p = {};
+    p.q = q; p.k = k8; p.v = v; p.o = o;
+    p.kv_len = kv_len;
+    p.sk = sk;
+    p.sq_out = sq_out; p.q8_out = q8_out;
+    p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.N = (int)N;
+    dense_strides(p.qs, Hq, N, D);
+    dense_strides(p.ks, Hkv, N, D);
+    dense_strides(p.vs, Hkv, N, D);
+    dense_strides(p.os, Hq, N, D);
+    p.bq = 1; p.bk = (int)bk;
+    p.bk_tile_shift = 0;
+    p.bk_key_shift = key_shift;
+    p.scale = scale;
+    const bool c = causal != 0;
+    p.out_f32 = out_dtype == ARHIP_F32;
+    const int nw = pipe_wants_4_waves(dev, B * Hq, N, D, c, kv_len != nullptr) ? 4 : 8;
+    p.nq = (int)((N + nw * 32 - 1) / (nw * 32));
+    p.total = (int)(p.nq * B * Hq);
+    p.lpt = p.total <= 16 * dev->cus;
+    arhip_call_timer t{dev, wait, secs};
+    t.kernel = ARHIP_K_SAGE;
+    if (int rc = t.begin()) return rc;
+    launch_pipe_i8_keys_qf(dev->stream, p, (int)D, c, nw);
+    arhip_note_selected(ARHIP_K_SAGE);
+    return t.end();
+}
+
 extern "C" int arhip_sage_fwd_strided(arhip_device *dev, const int8_t *q8, const int8_t *k8,
                                       const float *sq, const float *sk, const uint16_t *v, void *o,
                                       const int64_t v_strides[3], const int64_t o_strides[3],

@@ -486,7 +486,9 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     // bf16 queries with scales over blocks of 128 are quantised by the attention kernel itself (as the reference's
     // kernel does, cuda_flash_sage.rs:201-223): one launch and one pass over Q fewer
     const bool q_fused = pipelined && tile_uniform && bf16_in && bq == 128 && !st.sage_fp8;
-    if (!q_fused) quant(q, q8, sq, h, bq, nqb, false);
+    // f32 queries with a scale each and K scales per key (the reference's own convention): the same, row by row
+    const bool q_rows = pipelined && key_scales && !bf16_in && bq == 1 && !st.sage_fp8;
+    if (!q_fused && !q_rows) quant(q, q8, sq, h, bq, nqb, false);
     if (st.sage_smooth_k) {
         Tensor part = Tensor::empty(dev, {b, hk, nchunk, d}, F);
         const int64_t cpb = 256 / (d / 8);
@@ -494,9 +496,19 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
                                   {n, d, nchunk}));
         calls.push_back(make_call(dev, "ar_sage_kmean_final", {part, mean}, {F, F}, {b * hk, 1, 1}, {d, 1, 1}, {n, d, nchunk}));
     }
-    quant(k, k8, sk, hk, bk, nkb, st.sage_smooth_k);
     Tensor vb = v;
-    if (!bf16_in) {
+    // unsmoothed f32 K with a scale per key and the cast of V are one launch (ar_sage_quant_rows_cast_f32)
+    const bool kv_one_launch = !bf16_in && bk == 1 && !st.sage_smooth_k && !st.sage_fp8;
+    if (kv_one_launch) {
+        vb = Tensor::empty(dev, {b, hk, n, d}, BF);
+        const int64_t rows = b * hk * n, rpb = 256 / (d / 8), row_blocks = (rows + rpb - 1) / rpb, nv = rows * d;
+        calls.push_back(make_call(dev, "ar_sage_quant_rows_cast_f32", {k, k8, sk, v, vb}, {F, I8, F, F, BF},
+                                  {row_blocks + std::min<int64_t>((nv + 255) / 256, 16384), 1, 1}, {256, 1, 1},
+                                  {n, d, rows, nv, row_blocks}, {2, 3}));
+    } else {
+        quant(k, k8, sk, hk, bk, nkb, st.sage_smooth_k);
+    }
+    if (!bf16_in && !kv_one_launch) {
         vb = Tensor::empty(dev, {b, hk, n, d}, BF);
         const int64_t nv = b * hk * n * d;
         calls.push_back(make_call(dev, "ar_cast_bf16", {v, vb}, {F, BF}, {std::min<int64_t>((nv + 255) / 256, 16384), 1, 1},
@@ -512,6 +524,9 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
         if (q_fused)   // Q itself in the first slot; the scales slot is written
             calls.push_back(attn_call(mid ? "ar_flash_sage_qf_mid" : "ar_flash_sage_qf_long", {q, k8, vb, out, mslot, sq, sk},
                                       {BF, I8, BF, X, F, F, F}, grid, block, svals));
+        else if (q_rows)
+            calls.push_back(attn_call(mid ? "ar_flash_sage_qr_mid" : "ar_flash_sage_qr_long", {q, k8, vb, out, mslot, sq, sk},
+                                      {F, I8, BF, X, F, F, F}, grid, block, svals));
         else if (mid)
             calls.push_back(attn_call(st.sage_fp8 ? "ar_flash_sage_fp8_mid" : "ar_flash_sage_mid", {q8, k8, vb, out, mslot, sq, sk},
                                       {I8, I8, BF, X, F, F, F}, grid, block, svals));

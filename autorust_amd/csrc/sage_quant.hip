@@ -3,6 +3,7 @@
 #include "arhip_internal.h"
 #include "sage_quant_kernels.h"
 
+#include <algorithm>
 #include <mutex>
 
 // Scratch of arhip_sage_quant_static, resident on the device: the partial channel sums of the K
@@ -160,6 +161,29 @@ extern "C" int arhip_sage_quant_static(arhip_device *dev, const void *x, int8_t 
         ws = g_scratch_ptr[dev->ordinal];
     }
     return sage_quant_impl(dev, x, nullptr, x8, scales, mean, ws, B, H, N, D, block, dtype, smooth, wait, secs, -1);
+}
+
+extern "C" int arhip_sage_prep_kv_rows(arhip_device *dev, const float *k, int8_t *k8, float *sk, const float *v, uint16_t *vb,
+                                       int64_t B, int64_t Hkv, int64_t N, int64_t D, int wait, double *secs)
+{
+    ARHIP_REQUIRE(dev != nullptr, "arhip_sage_prep_kv_rows: null device");
+    ARHIP_REQUIRE(k && k8 && sk && v && vb, "arhip_sage_prep_kv_rows: null pointer");
+    ARHIP_REQUIRE(B > 0 && Hkv > 0 && N > 0 && (D == 64 || D == 128), "arhip_sage_prep_kv_rows: shape B=%lld Hkv=%lld N=%lld D=%lld",
+                  (long long)B, (long long)Hkv, (long long)N, (long long)D);
+    ARHIP_REQUIRE(arhip_aligned16(k) && arhip_aligned16(k8) && arhip_aligned16(v) && arhip_aligned16(vb),
+                  "arhip_sage_prep_kv_rows: tensors must be 16-byte aligned");
+    ARHIP_HIP(hipSetDevice(dev->ordinal));
+    const long rows = (long)(B * Hkv * N), nv = rows * (long)D;
+    const int rpb = 256 / (int)(D / 8);
+    const long row_blocks = (rows + rpb - 1) / rpb;
+    const long cast_blocks = std::min<long>((nv + 255) / 256, 16384);
+    ARHIP_REQUIRE(row_blocks + cast_blocks < ((long)1 << 31), "arhip_sage_prep_kv_rows: too many rows");
+    arhip_call_timer t{dev, wait, secs};
+    t.kernel = ARHIP_K_SAGE_QUANT;
+    if (int rc = t.begin()) return rc;
+    hipLaunchKernelGGL(quant_rows_cast_kernel, dim3((unsigned)(row_blocks + cast_blocks)), dim3(256), 0, dev->stream, k, k8, sk, v, vb,
+                       (int)N, (int)D, rows, nv, (int)row_blocks);
+    return t.end();
 }
 
 extern "C" int arhip_cast_bf16(arhip_device *dev, const float *x, uint16_t *y, int64_t n, int wait, double *secs)

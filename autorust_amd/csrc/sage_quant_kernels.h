@@ -287,5 +287,28 @@ __global__ void __launch_bounds__(256) cast_bf16_kernel(const float *x, uint16_t
     cast_bf16_body(x, y, n, blockIdx);
 }
 
+// The reference's pre-pass for K and V in one launch (f32 tensors, a scale per key, no smoothing): workgroups
+// [0, row_blocks) quantise rows of K as quant_rows does, the rest cast V to bf16 as cast_bf16 does.  Two launches of a
+// few microseconds each become one; results are those of the two kernels bit for bit.
+__device__ __forceinline__ void quant_rows_cast_body(const float *k, int8_t *k8, float *scales, const float *v, uint16_t *vb,
+                                                     int N, int D, long rows_total, long nv, int row_blocks, const dim3 bid)
+{
+    if ((int)bid.x < row_blocks) {
+        quant_rows_body<float, false>(k, k8, scales, nullptr, N, D, rows_total, XLayout::dense(1, N, D), bid);
+    } else {
+        const size_t stride = (size_t)(gridDim.x - row_blocks) * blockDim.x;
+        for (size_t i = (size_t)(bid.x - row_blocks) * blockDim.x + threadIdx.x; i < (size_t)nv; i += stride) {
+            const __bf16 b = (__bf16)v[i];  // round-to-nearest-even
+            vb[i] = __builtin_bit_cast(uint16_t, b);
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) quant_rows_cast_kernel(const float *k, int8_t *k8, float *scales, const float *v,
+                                                              uint16_t *vb, int N, int D, long rows_total, long nv, int row_blocks)
+{
+    quant_rows_cast_body(k, k8, scales, v, vb, N, D, rows_total, nv, row_blocks, blockIdx);
+}
+
 
 }  // namespace arhip

@@ -246,6 +246,24 @@ class Device:
                                              int(causal), out_dtype, scale, int(wait), ctypes.byref(s)))
         return s.value if wait else None
 
+    def sage_prep_kv_rows(self, k, k8, sk, v, vb, B, Hkv, N, D, wait=True):
+        """K quantised row by row (no smoothing) and V cast to bf16 in one launch (f32 tensors)."""
+        s = ctypes.c_double()
+        check(self.lib.arhip_sage_prep_kv_rows(self.handle, self._ptr(k), self._ptr(k8), self._ptr(sk), self._ptr(v), self._ptr(vb),
+                                               B, Hkv, N, D, int(wait), ctypes.byref(s)))
+        return s.value if wait else None
+
+    def sage_fwd_qfused_rows(self, q, k8, sk, v, o, B, Hq, Hkv, N, D, bk, out_dtype=F32, sq_out=None, q8_out=None, kv_len=None,
+                             causal=False, scale=None, wait=True):
+        """The reference's convention in one attention launch: f32 q quantised row by row inside the kernel, K scales
+        per key (bk a power of two below 64)."""
+        scale = float(1.0 / np.sqrt(np.float32(D))) if scale is None else float(scale)
+        s = ctypes.c_double()
+        check(self.lib.arhip_sage_fwd_qfused_rows(self.handle, self._ptr(q), self._ptr(k8), self._ptr(sk), self._ptr(v),
+                                                  self._ptr(o), self._ptr(sq_out), self._ptr(q8_out), self._ptr(kv_len),
+                                                  B, Hq, Hkv, N, D, bk, int(causal), out_dtype, scale, int(wait), ctypes.byref(s)))
+        return s.value if wait else None
+
     def sage_quant_static(self, x, x8, scales, B, H, N, D, block, dtype, mean=None, smooth=False, wait=True):
         """sage_quant with the partial sums in the library's own device array (no allocation)."""
         s = ctypes.c_double()

@@ -91,7 +91,7 @@ class SageWorkload:
         self.kernel = _lib.K_SAGE
         # dominant kernel: int8 K (1 B), Q as int8 codes (1 B) or, quantised in its prologue, bf16 (2 B), bf16 V and O
         # (2 B), block scales
-        q_bytes = 2 if (not f32_io and bq == 128 and bk % 64 == 0 and not fp8) else 1
+        q_bytes = 2 if (not f32_io and bq == 128 and bk % 64 == 0 and not fp8) else 4 if (f32_io and bq == 1 and bk == 1) else 1
         self.kernel_bytes = n * (q_bytes + 1 + 2 + 2) + 4 * B * H * (S // bq + S // bk)
         self.dtype = "fp8" if fp8 else "int8"
 
@@ -108,6 +108,13 @@ class SageWorkload:
         # bf16 queries with scales over blocks of 128: the attention kernel quantises Q itself (as the host mirror's
         # Tensor::sage_attention_with does); otherwise the Q quantiser is a launch of its own
         q_fused = not self.f32_io and self.bq == 128 and self.bk % 64 == 0 and not self.fp8
+        if self.f32_io and self.bq == 1 and self.bk == 1:
+            # the reference's convention in two launches: K's per-key quantiser together with V's cast, then the
+            # attention kernel, which quantises the f32 queries row by row in its prologue
+            d.sage_prep_kv_rows(self.dk, self.k8, self.sk, self.dvf, self.dv, B, H, S, D, wait=False)
+            d.sage_fwd_qfused_rows(self.dq, self.k8, self.sk, self.dv, self.do, B, H, H, S, D, self.bk, out_dtype=io,
+                                   sq_out=self.sq, causal=self.causal, wait=False)
+            return
         if not q_fused:
             d.sage_quant(self.dq, self.q8, self.sq, B, H, S, D, self.bq, io, wait=False)
         d.sage_quant(self.dk, self.k8, self.sk, B, H, S, D, self.bk, io, mean=self.mean, workspace=self.ws,

@@ -109,7 +109,7 @@ int arhip_graph_destroy(arhip_device *dev, void *graph_exec);
  * image: a gfx950 code object (hipcc --genco), or a container of several that are looked up as
  * one: "ARHIPKO1", uint32 count, uint32 0, then per code object uint64 size and its bytes padded
  * to a multiple of 16 (autorust_amd/attn_kernels.hsaco is such a file: its entry points compile as
- * eleven code objects side by side).  Modules are cached per device by content hash.  args: nbufs device pointers followed by nvals scalars;
+ * thirteen code objects side by side).  Modules are cached per device by content hash.  args: nbufs device pointers followed by nvals scalars;
  * val_bits[i] in {32, 64} narrows vals[i] like the reference's signature
  * dtype does.  grid is in blocks. */
 int arhip_module_load(arhip_device *dev, const void *image, size_t len, void **module);
@@ -236,6 +236,12 @@ int arhip_sage_fwd_fp8(arhip_device *dev, const uint8_t *q8, const uint8_t *k8,
                        int64_t bq, int64_t bk, int causal, int out_dtype, float scale,
                        int wait, double *secs);
 
+/* arhip_sage_prep_kv_rows: the reference's K and V preparation (cuda_flash_sage.rs:209-222, 257-262: a scale per
+ *   key, no smoothing, V to bf16) for f32 tensors in ONE launch: k8 / sk as arhip_sage_quant(block 1, smooth 0)
+ *   writes them, vb as arhip_cast_bf16 writes it, bit for bit.  k, v [B,Hkv,N,D] f32. */
+int arhip_sage_prep_kv_rows(arhip_device *dev, const float *k, int8_t *k8, float *sk, const float *v, uint16_t *vb,
+                            int64_t B, int64_t Hkv, int64_t N, int64_t D, int wait, double *secs);
+
 /* arhip_cast_bf16: f32 -> bf16 round-to-nearest-even of n elements (the V
  *   operand of the Sage kernel: cuda_flash_sage.rs:99-103, 257-262). */
 int arhip_cast_bf16(arhip_device *dev, const float *x, uint16_t *y, int64_t n, int wait, double *secs);
@@ -267,6 +273,14 @@ int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const int8_t *k8
                           const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
                           int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
                           int causal, int out_dtype, float scale, int wait, double *secs);
+
+/* arhip_sage_fwd_qfused_rows: the same for the reference's own convention: q f32 [B,Hq,N,D], a scale
+ *   per query (sq_out [B,Hq,N]), k8 / sk from arhip_sage_quant with bk = 1 (or a power of two below
+ *   64); bit for bit arhip_sage_quant(block 1) on q followed by arhip_sage_fwd. */
+int arhip_sage_fwd_qfused_rows(arhip_device *dev, const float *q, const int8_t *k8, const float *sk,
+                               const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
+                               int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
+                               int causal, int out_dtype, float scale, int wait, double *secs);
 
 /* arhip_sage_fwd_strided: arhip_sage_fwd with element strides {batch, head, token} for v and o
  *   (NULL = dense): v as the projection produced it ([B,N,Hkv,D]), o written as [B,N,Hq*D].

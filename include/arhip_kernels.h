@@ -6,7 +6,7 @@
  * reference's `HostCall{src, name, signature, bufs, global, local, vals}` ->
  * `Compiled::run_host_kernel` -> `Prog::call` does (src/engine/session.rs:210-256,
  * src/runtime/device.rs:383-402), load the file with arhip_module_load and launch these with
- * arhip_launch.  (The file is a container of eleven code objects, see arhip_module_load in
+ * arhip_launch.  (The file is a container of thirteen code objects, see arhip_module_load in
  * arhip.h; a host that wants hipModuleLoadData / hipModuleLaunchKernel itself loads each part,
  * or builds csrc/attn_entry.hip without -DARHIP_ENTRY_PART as one plain code object.)
  * Arguments are device pointers followed by scalars, in the reference's order
@@ -99,6 +99,10 @@
 #define ARHIP_KERNEL_SAGE_QUANT_ROWS_F32 "ar_sage_quant_rows_f32"
 #define ARHIP_KERNEL_SAGE_QUANT_ROWS_BF16 "ar_sage_quant_rows_bf16"
 #define ARHIP_KERNEL_CAST_BF16 "ar_cast_bf16"
+/* ar_sage_quant_rows_f32 (smooth = 0) on K and ar_cast_bf16 on V in one launch, for the reference's convention:
+ *   (K f32, K8, SK, V f32, Vb bf16, int N, int D, long rows_total, long nv, int row_blocks),
+ *   grid [row_blocks + min(ceil(nv/256), 16384), 1, 1], row_blocks = ceil(rows_total / (256/(D/8))), block [256,1,1] */
+#define ARHIP_KERNEL_SAGE_QUANT_ROWS_CAST_F32 "ar_sage_quant_rows_cast_f32"
 
 /* Key-padding masks on the named-kernel seam.  The reference's fused kernels admit a dense [n, n] mask
  * only (src/models/flash_attention.rs:389-396) and leave per-batch key lengths to its general path
@@ -126,6 +130,15 @@
  *     SQ   [b*hq, ceil(n/128)] f32, WRITTEN: the scales the kernel derived (bq must be 128)
  * K8 / SK as the K quantiser left them, bk = 64 * 2^j.  Bit-identical to ar_sage_quant_blocks_bf16 on Q followed
  * by ar_flash_sage_long / _mid. */
+/* The reference's own convention in one launch: the argument lists of ar_flash_sage_long / _mid (and _lens) with
+ *     Q    f32 [b*hq, n, head_dim], quantised row by row in the kernel's prologue
+ *     SQ   [b*hq, n] f32, WRITTEN: one scale per query (bq must be 1)
+ * K8 / SK as the K quantiser left them, bk a power of two below 64 (1: a scale per key).  Bit-identical to
+ * ar_sage_quant_rows_f32 on Q followed by ar_flash_sage_long / _mid. */
+#define ARHIP_KERNEL_FLASH_SAGE_QR_LONG "ar_flash_sage_qr_long"
+#define ARHIP_KERNEL_FLASH_SAGE_QR_MID "ar_flash_sage_qr_mid"
+#define ARHIP_KERNEL_FLASH_SAGE_QR_LONG_LENS "ar_flash_sage_qr_long_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_QR_MID_LENS "ar_flash_sage_qr_mid_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_QF_LONG "ar_flash_sage_qf_long"
 #define ARHIP_KERNEL_FLASH_SAGE_QF_MID "ar_flash_sage_qf_mid"
 #define ARHIP_KERNEL_FLASH_SAGE_QF_LONG_LENS "ar_flash_sage_qf_long_lens"

@@ -260,7 +260,9 @@ pub fn host_calls_sage(
     // bf16 queries with scales over blocks of 128 are quantised by the attention kernel itself (as the CUDA
     // kernel does): one launch and one pass over Q fewer
     let q_fused = pipelined && tile_uniform && bf16_in && bq == 128 && !sage.fp8;
-    if !q_fused {
+    // f32 queries with a scale each and K scales per key (the CUDA kernel's own convention): the same, row by row
+    let q_rows = pipelined && key_scales && !bf16_in && bq == 1 && !sage.fp8;
+    if !q_fused && !q_rows {
         calls.push(quant_call(q8fmt, sfx, x, &q, &s.q8, &s.sq, &s.mean, b, h, n, d, bq, nqb, false));
     }
     if sage.smooth_k {
@@ -270,8 +272,21 @@ pub fn host_calls_sage(
         calls.push(call("ar_sage_kmean_final", vec![s.part.clone(), s.mean.clone()], &[f, f], [b * hk, 1, 1], [d, 1, 1],
                         vec![n, d, nchunk], &[]));
     }
-    calls.push(quant_call(q8fmt, sfx, x, &k, &s.k8, &s.sk, &s.mean, b, hk, n, d, bk, nkb, sage.smooth_k));
+    // unsmoothed f32 K with a scale per key and the cast of V are one launch (ar_sage_quant_rows_cast_f32)
+    let kv_one_launch = !bf16_in && bk == 1 && !sage.smooth_k && !sage.fp8 && s.vb.is_some();
+    if !kv_one_launch {
+        calls.push(quant_call(q8fmt, sfx, x, &k, &s.k8, &s.sk, &s.mean, b, hk, n, d, bk, nkb, sage.smooth_k));
+    }
     let vb = match &s.vb {
+        Some(vb) if kv_one_launch => {
+            let rows = b * hk * n;
+            let rpb = 256 / (d / 8);
+            let (row_blocks, nv) = ((rows + rpb - 1) / rpb, rows * d);
+            calls.push(call("ar_sage_quant_rows_cast_f32", vec![k.clone(), s.k8.clone(), s.sk.clone(), v.clone(), vb.clone()],
+                            &[f, i8t, f, f, bf], [row_blocks + ((nv + 255) / 256).min(16384), 1, 1], [256, 1, 1],
+                            vec![n, d, rows, nv, row_blocks], &[2, 3]));
+            vb.clone()
+        }
         Some(vb) => {
             let nv = b * hk * n * d;
             calls.push(call("ar_cast_bf16", vec![v.clone(), vb.clone()], &[f, bf], [((nv + 255) / 256).min(16384), 1, 1], [256, 1, 1],
@@ -291,6 +306,9 @@ pub fn host_calls_sage(
             // Q itself in the first slot; the scales slot is written
             let name = if mid { "ar_flash_sage_qf_mid" } else { "ar_flash_sage_qf_long" };
             calls.push(attn_call(name, vec![q, s.k8, vb, o, mask, s.sq, s.sk], &[bf, i8t, bf, x, f, f, f], lens, grid, block, sv));
+        } else if q_rows {
+            let name = if mid { "ar_flash_sage_qr_mid" } else { "ar_flash_sage_qr_long" };
+            calls.push(attn_call(name, vec![q, s.k8, vb, o, mask, s.sq, s.sk], &[f, i8t, bf, x, f, f, f], lens, grid, block, sv));
         } else {
             let name = if mid { if sage.fp8 { "ar_flash_sage_fp8_mid" } else { "ar_flash_sage_mid" } } else { long };
             calls.push(attn_call(name, vec![s.q8, s.k8, vb, o, mask, s.sq, s.sk], &[i8t, i8t, bf, x, f, f, f], lens, grid, block, sv));

@@ -280,3 +280,37 @@ def test_q_quantiser_inside_the_attention_kernel(dev, B, H, Hkv, N, D, causal, u
     assert np.array_equal(got_sq, w_sq) and np.array_equal(got_q8, w_q8)
     assert w_sq[0, 0, 1] == 1.0
     assert np.array_equal(got, r["out"]) and np.array_equal(again, got)
+
+
+@pytest.mark.parametrize("B,H,Hkv,N,D,bk,causal,use_len,out_dtype", [
+    (1, 6, 6, 789, 64, 1, False, False, F32),          # the reference's shape and convention (tests/sage_int8.rs)
+    (2, 8, 4, 1000, 128, 1, True, True, F32),
+    (1, 32, 32, 2304, 128, 16, False, False, BF16),    # 8 waves per workgroup, a K scale per 16 keys
+    (2, 6, 3, 300, 64, 1, True, False, BF16),
+])
+def test_row_quantiser_inside_the_attention_kernel(dev, B, H, Hkv, N, D, bk, causal, use_len, out_dtype):
+    """arhip_sage_fwd_qfused_rows: f32 queries quantised row by row in the prologue of the per-key pipelined kernel,
+    as the reference's kernel does (src/runtime/cuda_flash_sage.rs:201-223).  Exported codes and scales are the
+    oracle's bit for bit, and the output is bit for bit that of quantising first."""
+    q, k, v = fill_qkv(B, H, Hkv, N, D)
+    q = q * (np.float32(2.0) ** np.linspace(-2, 2, H, dtype=np.float32))[None, :, None, None]
+    q[0, 0, 5] = 0.0                                           # an all-zero row: scale 1
+    kv_len = np.array([N - 77, max(1, N // 3)][:B], np.int32) if use_len else None
+    r = run_sage(dev, q, k, v, 1, bk, smooth=False, out_dtype=out_dtype, kv_len=kv_len, causal=causal)
+    with Bufs(dev) as bufs:
+        dq = bufs.put(q)
+        k8, sk = bufs.put(r["k8"]), bufs.put(r["sk"])
+        dv = bufs.put(synth.to_bf16_bits(v))
+        do = bufs.new(q.size * (4 if out_dtype == F32 else 2))
+        sq_out, q8_out = bufs.new(B * H * N * 4), bufs.new(q.size)
+        dl = bufs.put(kv_len) if use_len else None
+        dev.sage_fwd_qfused_rows(dq, k8, sk, dv, do, B, H, Hkv, N, D, bk, out_dtype=out_dtype, sq_out=sq_out, q8_out=q8_out,
+                                 kv_len=dl, causal=causal)
+        got = do.copyout(np.float32, q.shape) if out_dtype == F32 else synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+        got_sq, got_q8 = sq_out.copyout(np.float32, (B, H, N)), q8_out.copyout(np.int8, q.shape)
+        with pytest.raises(_lib.ArhipError, match="power of two of keys below 64"):
+            dev.sage_fwd_qfused_rows(dq, k8, sk, dv, do, B, H, Hkv, N, D, 64, out_dtype=out_dtype)
+    w_q8, w_sq = oracle.quant_blocks(q, 1)
+    assert np.array_equal(got_sq, w_sq) and np.array_equal(got_q8, w_q8)
+    assert w_sq[0, 0, 5] == 1.0
+    assert np.array_equal(got, r["out"])

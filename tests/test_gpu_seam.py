@@ -510,3 +510,64 @@ def test_ar_flash_sage_qf_by_name(dev, kernels, form, per_wg, block, d, causal, 
                        [n, d, int(causal), 0, hq, hkv, 64, bk, out_f32])
     assert np.array_equal(got_sq, h_sq)
     assert np.array_equal(got, plain)
+
+
+@pytest.mark.parametrize("form,per_wg,block", [("long", 256, 512), ("mid", 128, 256)])
+@pytest.mark.parametrize("d,bk,causal,out_f32,with_lens", [(64, 1, False, 1, False), (128, 16, True, 0, True)])
+def test_ar_flash_sage_qr_by_name(dev, kernels, form, per_wg, block, d, bk, causal, out_f32, with_lens):
+    """The entries that quantise f32 queries row by row in their prologue (the reference's convention,
+    src/runtime/cuda_flash_sage.rs:201-223): the scales they write are ar_sage_quant_rows_f32's, the output is bit
+    for bit that of that quantiser followed by the plain entry of the same form."""
+    b, hq, hkv, n, bq = 2, 4, 2, 700, 1
+    q = synth.normal(41, (b, hq, n, d))
+    k = synth.normal(42, (b, hkv, n, d))
+    v = synth.normal(43, (b, hkv, n, d))
+    lens = np.array([333, n], np.int32) if with_lens else None
+    sfx = "_lens" if with_lens else ""
+    with Bufs(dev) as bufs:
+        q8, sq, _, h_q8, h_sq, _ = _quantise_by_name(dev, kernels, bufs, q, bq, False, F32)
+        k8, sk, _, h_k8, h_sk, _ = _quantise_by_name(dev, kernels, bufs, k, bk, False, F32)
+        dq, dv = bufs.put(q), bufs.put(synth.to_bf16_bits(v))
+        do, dp = bufs.new(q.size * 4), bufs.new(q.size * 4)
+        sq2 = bufs.new(b * hq * n * 4)
+        dl = [bufs.put(lens)] if with_lens else []
+        vals = [n, d, int(causal), 0, hq, hkv, bq, bk, out_f32]
+        name = "ar_flash_sage_qr_" + form + sfx
+        dev.launch(kernels, name, _grid(n, per_wg, b, hq), (block, 1, 1), [dq, k8, dv, do, do] + dl + [sq2, sk], vals)
+        dev.launch(kernels, "ar_flash_sage_" + form + sfx, _grid(n, per_wg, b, hq), (block, 1, 1), [q8, k8, dv, dp, dp] + dl + [sq, sk], vals)
+        words = q.size if out_f32 else q.size // 2
+        got, plain = do.copyout(np.uint32, (words,)), dp.copyout(np.uint32, (words,))
+        got_sq = sq2.copyout(np.float32, h_sq.shape)
+        for bad_bq, bad_bk in [(128, bk), (1, 64)]:
+            with pytest.raises(_lib.ArhipError, match="quantises Q row by row"):
+                dev.launch(kernels, name, _grid(n, per_wg, b, hq), (block, 1, 1), [dq, k8, dv, do, do] + dl + [sq2, sk],
+                           [n, d, int(causal), 0, hq, hkv, bad_bq, bad_bk, out_f32])
+    assert np.array_equal(got_sq, h_sq)
+    assert np.array_equal(got, plain)
+
+
+@pytest.mark.parametrize("b,hkv,n,d", [(1, 6, 789, 64), (2, 3, 1000, 128), (1, 1, 5, 64)])
+def test_ar_sage_quant_rows_cast_by_name(dev, kernels, b, hkv, n, d):
+    """One launch for the reference's K and V preparation (a scale per key, no smoothing; V to bf16,
+    src/runtime/cuda_flash_sage.rs:209-222, 257-262): the same bytes as ar_sage_quant_rows_f32 and ar_cast_bf16, and
+    the typed entry point arhip_sage_prep_kv_rows gives them too."""
+    k = synth.normal(51, (b, hkv, n, d)) * np.float32(3.0)
+    k[0, 0, min(3, n - 1)] = 0.0
+    v = synth.normal(52, (b, hkv, n, d))
+    rows = b * hkv * n
+    rpb = 256 // (d // 8)
+    row_blocks = (rows + rpb - 1) // rpb
+    cast_blocks = min((v.size + 255) // 256, 16384)
+    with Bufs(dev) as bufs:
+        dk, dvf = bufs.put(k), bufs.put(v)
+        k8, sk, vb = bufs.new(k.size), bufs.new(rows * 4), bufs.new(v.size * 2)
+        dev.launch(kernels, "ar_sage_quant_rows_cast_f32", (row_blocks + cast_blocks, 1, 1), (256, 1, 1), [dk, k8, sk, dvf, vb],
+                   [n, d, rows, v.size, row_blocks], [32, 32, 64, 64, 32])
+        got = k8.copyout(np.int8, k.shape), sk.copyout(np.float32, (b, hkv, n)), vb.copyout(np.uint16, v.shape)
+        k8b, skb, vbb = bufs.new(k.size), bufs.new(rows * 4), bufs.new(v.size * 2)
+        dev.sage_prep_kv_rows(dk, k8b, skb, dvf, vbb, b, hkv, n, d)
+        typed = k8b.copyout(np.int8, k.shape), skb.copyout(np.float32, (b, hkv, n)), vbb.copyout(np.uint16, v.shape)
+    w8, ws = oracle.quant_blocks(k, 1)
+    for g in (got, typed):
+        assert np.array_equal(g[0], w8) and np.array_equal(g[1], ws)
+        assert np.array_equal(g[2], synth.to_bf16_bits(v))

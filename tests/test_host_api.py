@@ -146,6 +146,15 @@ def test_sage_attention_with_selects_the_quantised_kernel(hdev):
     k8, sk = oracle.quant_blocks(k, 1)
     err = float(np.abs(out.to_list() - oracle.sage(q8, k8, sq, sk, v, 1, 1)).max())
     assert err < 2e-3                                        # tests/sage_int8.rs:148
+    # that convention is two launches: K's per-key quantiser together with V's cast, then the attention kernel,
+    # which quantises the f32 queries row by row itself (as the reference's kernel does, cuda_flash_sage.rs:201-223)
+    sess.begin_capture()
+    again = tq.sage_attention_with(tk, tv, None, 0.0, False, sess, ref)
+    ncalls = sess.end_capture()
+    assert [sess.step(i)[0] for i in range(ncalls)] == ["ar_sage_quant_rows_cast_f32", "ar_flash_sage_qr_mid"]
+    assert sess.step_detail(1)[4][0] == (0, FLOAT32) and np.array_equal(again.to_list(), out.to_list())
+    sess.replay()
+    assert np.array_equal(again.to_list(), out.to_list())
     out2 = tq.sage_attention_with(tk, tv, None, 0.0, False, sess)
     err2 = float(np.abs(out2.to_list() - oracle.sdpa_f64(q, k, v)).max())
     assert err2 < 2e-2
