@@ -287,6 +287,8 @@ def test_q_quantiser_inside_the_attention_kernel(dev, B, H, Hkv, N, D, causal, u
     (2, 8, 4, 1000, 128, 1, True, True, F32),
     (1, 32, 32, 2304, 128, 16, False, False, BF16),    # 8 waves per workgroup, a K scale per 16 keys
     (2, 6, 3, 300, 64, 1, True, False, BF16),
+    (1, 2, 2, 1, 64, 1, False, False, F32),            # a single token
+    (2, 2, 1, 129, 128, 4, True, True, F32),           # one query past a workgroup's 128
 ])
 def test_row_quantiser_inside_the_attention_kernel(dev, B, H, Hkv, N, D, bk, causal, use_len, out_dtype):
     """arhip_sage_fwd_qfused_rows: f32 queries quantised row by row in the prologue of the per-key pipelined kernel,
@@ -294,7 +296,8 @@ def test_row_quantiser_inside_the_attention_kernel(dev, B, H, Hkv, N, D, bk, cau
     oracle's bit for bit, and the output is bit for bit that of quantising first."""
     q, k, v = fill_qkv(B, H, Hkv, N, D)
     q = q * (np.float32(2.0) ** np.linspace(-2, 2, H, dtype=np.float32))[None, :, None, None]
-    q[0, 0, 5] = 0.0                                           # an all-zero row: scale 1
+    zr = min(5, N - 1)
+    q[0, 0, zr] = 0.0                                          # an all-zero row: scale 1
     kv_len = np.array([N - 77, max(1, N // 3)][:B], np.int32) if use_len else None
     r = run_sage(dev, q, k, v, 1, bk, smooth=False, out_dtype=out_dtype, kv_len=kv_len, causal=causal)
     with Bufs(dev) as bufs:
@@ -312,5 +315,5 @@ def test_row_quantiser_inside_the_attention_kernel(dev, B, H, Hkv, N, D, bk, cau
             dev.sage_fwd_qfused_rows(dq, k8, sk, dv, do, B, H, Hkv, N, D, 64, out_dtype=out_dtype)
     w_q8, w_sq = oracle.quant_blocks(q, 1)
     assert np.array_equal(got_sq, w_sq) and np.array_equal(got_q8, w_q8)
-    assert w_sq[0, 0, 5] == 1.0
+    assert w_sq[0, 0, zr] == 1.0
     assert np.array_equal(got, r["out"])
