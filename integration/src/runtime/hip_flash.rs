@@ -17,6 +17,8 @@
 //! | `ar_flash_sage`      | 256   | `[ceil(n/128), b*h, 1]` | same `+ bq, bk`; buffers `+ SQ, SK`; O is f32|
 //! | `ar_flash_sage_long` | 512   | `[ceil(n/256), b*h, 1]` | same `+ bq, bk, out_f32`                     |
 //! | `ar_flash_sage_mid`  | 256   | `[ceil(n/128), b*h, 1]` | same; the pipelined kernel with 4 waves      |
+//! | `ar_flash_sage_qf_long`, `ar_flash_sage_qf_mid` | as `_long` / `_mid` | first buffer: the bf16 queries themselves; `SQ` is written (`bq` 128, `bk` 64·2^j) |
+//! | `ar_flash_sage_qr_long`, `ar_flash_sage_qr_mid` | as `_long` / `_mid` | first buffer: the f32 queries themselves; `SQ` `[b*h, n]` is written (`bq` 1, `bk` a power of two below 64) |
 //! | `ar_flash_sage_fp8`, `ar_flash_sage_fp8_long`, `ar_flash_sage_fp8_mid` | as the int8 entries, on E4M3 codes (`SageOptions::fp8`) |
 //! | `<entry>_lens`       | as `<entry>` | as `<entry>`     | one more buffer after the mask slot: `L`, int32 `[b]` key lengths |
 //!
@@ -27,8 +29,11 @@
 //! builder falls through to `ar_flash_f32_lens` then.
 //!
 //! Unlike the CUDA Sage kernel, which quantises inside the attention kernel (K once per query
-//! block, `cuda_flash_sage.rs:248-278`), the quantiser is a pre-pass of its own here, with K
-//! smoothing and per-block scales (128 query tokens / 64 key tokens by default).  A Sage call is
+//! block, `cuda_flash_sage.rs:248-278`), the K quantiser is a pre-pass of its own here, with K
+//! smoothing and per-block scales (128 query tokens / 64 key tokens by default); the queries are
+//! quantised by the attention kernel itself where an entry for it exists (`_qf_`: bf16 tensors with
+//! `block_q` 128; `_qr_`: f32 tensors with a scale per query, the CUDA kernel's convention, whose K
+//! quantiser and V cast are the one launch `ar_sage_quant_rows_cast_f32`).  A Sage call is
 //! therefore a short sequence of `HostCall`s; their scratch buffers ride in `bufs`, so a JIT
 //! replay finds them again.
 
