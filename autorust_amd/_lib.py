@@ -77,6 +77,7 @@ SIGNATURES = {
                                      c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, _pd]),
     "arhip_sage_fwd_fp8": (c_int, [c_void_p] * 9 + [c_int64] * 7 + [c_int, c_int, c_float, c_int, _pd]),
     "arhip_sage_fwd_qfused": (c_int, [c_void_p] * 9 + [c_int64] * 6 + [c_int, c_int, c_float, c_int, _pd]),
+    "arhip_sage_fwd_fp8_qfused": (c_int, [c_void_p] * 9 + [c_int64] * 6 + [c_int, c_int, c_float, c_int, _pd]),
     "arhip_sage_fwd_qfused_rows": (c_int, [c_void_p] * 9 + [c_int64] * 6 + [c_int, c_int, c_float, c_int, _pd]),
     "arhip_sage_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_float,

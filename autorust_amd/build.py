@@ -22,10 +22,10 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # the pipelined kernel's variants compile in translation units of their own (pipe_launch.h), side by side
 SOURCES = ["device.hip", "flash.hip", "sage_quant.hip", "pipe_bf16.hip", "pipe_i8.hip", "pipe_i8_keys.hip", "pipe_i8_qf.hip",
-           "pipe_i8_keys_qf.hip", "pipe_fp8.hip", "pipe_fp8_keys.hip"]
+           "pipe_i8_keys_qf.hip", "pipe_fp8.hip", "pipe_fp8_qf.hip", "pipe_fp8_keys.hip"]
 HEADERS = ["arhip_internal.h", "attn_fwd.h", "attn_pipe.h", "pipe_launch.h", "pipe_tu.h", "flash_f32.h", "flash_bwd_f32.h",
            "sage_quant_kernels.h", os.path.join("..", "..", "include", "arhip.h")]
-ENTRY_PARTS = 13  # code objects csrc/attn_entry.hip compiles as (-DARHIP_ENTRY_PART=k), packed into KERNELS
+ENTRY_PARTS = 15  # code objects csrc/attn_entry.hip compiles as (-DARHIP_ENTRY_PART=k), packed into KERNELS
 
 # -packed-fp32-ops off: packed fp32 VALU instructions are not used by this build.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

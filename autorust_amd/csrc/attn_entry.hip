@@ -49,7 +49,7 @@
 // last: it switches floating-point contraction off for the rest of the file
 #include "sage_quant_kernels.h"
 
-// The entry points compile as thirteen code objects side by side (-DARHIP_ENTRY_PART=1 ... 13; the build packs them into
+// The entry points compile as fifteen code objects side by side (-DARHIP_ENTRY_PART=1 ... 15; the build packs them into
 // one file that arhip_module_load takes as a whole): the pipelined kernels are several thousand instructions per
 // variant, minutes of compilation per entry.  Without the macro this file is one code object with all of them.
 #ifndef ARHIP_ENTRY_PART
@@ -548,10 +548,11 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_mid_lens(cons
 }
 
 #endif
-// ar_flash_sage_qf_long / _mid: the pipelined int8 kernel with the Q quantiser in its prologue.  Q holds bf16
+// ar_flash_sage_qf_long / _mid (and ar_flash_sage_fp8_qf_long / _mid on E4M3 codes): the pipelined 8-bit kernel with the
+// Q quantiser in its prologue.  Q holds bf16
 // values; SQ [b*hq, ceil(n/128)] RECEIVES the scales (bq must be 128); K8 / SK as from the K quantiser with
 // bk = 64 * 2^j.  Same grid and block as ar_flash_sage_long / _mid.
-template <int NW>
+template <int NW, int MODE = MODE_I8>
 __device__ __forceinline__ void flash_sage_qf_entry(unsigned char *lds, const uint16_t *Q, const void *K8, const uint16_t *V, void *O,
                                                     const float *M, const int *L, float *SQ, const float *SK, int N, int head_dim,
                                                     int causal, int has_mask, int hq, int hkv, int bq, int bk, int out_f32)
@@ -569,8 +570,8 @@ __device__ __forceinline__ void flash_sage_qf_entry(unsigned char *lds, const ui
     const int wg = linear_wg();
 #define AR_SAGE_QF(DD)                                                                        \
     do {                                                                                      \
-        if (causal) attn_pipe_body<DD, true, MODE_I8, false, NW, false, true>(p, lds, wg);    \
-        else attn_pipe_body<DD, false, MODE_I8, false, NW, false, true>(p, lds, wg);          \
+        if (causal) attn_pipe_body<DD, true, MODE, false, NW, false, true>(p, lds, wg);       \
+        else attn_pipe_body<DD, false, MODE, false, NW, false, true>(p, lds, wg);             \
     } while (0)
     if (head_dim == 64) AR_SAGE_QF(64);
     else if (head_dim == 128) AR_SAGE_QF(128);
@@ -616,6 +617,48 @@ extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_qf_mid_lens(c
 {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_I8, 4, false, true>()];
     flash_sage_qf_entry<4>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+#endif
+#if ARHIP_PART(14)
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_qf_long(const uint16_t *Q, const uint8_t *K8, const uint16_t *V,
+                                                                             void *O, const float *M, float *SQ, const float *SK,
+                                                                             int N, int head_dim, int causal, int has_mask, int hq,
+                                                                             int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 8, false, true>()];
+    flash_sage_qf_entry<8, MODE_FP8>(lds, Q, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(512) ar_flash_sage_fp8_qf_long_lens(const uint16_t *Q, const uint8_t *K8, const uint16_t *V,
+                                                                                  void *O, const float *M, const int *L, float *SQ,
+                                                                                  const float *SK, int N, int head_dim, int causal,
+                                                                                  int has_mask, int hq, int hkv, int bq, int bk,
+                                                                                  int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 8, false, true>()];
+    flash_sage_qf_entry<8, MODE_FP8>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+#endif
+#if ARHIP_PART(15)
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_qf_mid(const uint16_t *Q, const uint8_t *K8, const uint16_t *V,
+                                                                               void *O, const float *M, float *SQ, const float *SK,
+                                                                               int N, int head_dim, int causal, int has_mask, int hq,
+                                                                               int hkv, int bq, int bk, int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 4, false, true>()];
+    flash_sage_qf_entry<4, MODE_FP8>(lds, Q, K8, V, O, M, nullptr, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) ar_flash_sage_fp8_qf_mid_lens(const uint16_t *Q, const uint8_t *K8, const uint16_t *V,
+                                                                                    void *O, const float *M, const int *L, float *SQ,
+                                                                                    const float *SK, int N, int head_dim, int causal,
+                                                                                    int has_mask, int hq, int hkv, int bq, int bk,
+                                                                                    int out_f32)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[attn_pipe_lds_bytes<128, MODE_FP8, 4, false, true>()];
+    flash_sage_qf_entry<4, MODE_FP8>(lds, Q, K8, V, O, M, L, SQ, SK, N, head_dim, causal, has_mask, hq, hkv, bq, bk, out_f32);
 }
 
 #endif

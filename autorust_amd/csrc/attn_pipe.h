@@ -113,15 +113,18 @@ __device__ __forceinline__ void pipe_work_item(const AttnParams &p, int wg, int 
 
 // The kernel body.  lds: attn_pipe_lds_bytes<D, MODE>() bytes of workgroup memory, 1024-byte
 // aligned; wg_linear: this workgroup's index in [0, p.total).  BIAS (int8 only): see s_init below.
-// QFUSE (int8): the prologue is the quantiser of sage_quant_kernels.h for this workgroup's queries, operation for
-// operation (absmax, scale = absmax / 127 or 1, x8 = clamp(rint(x * (1 / scale)), +-127)), so the result is bit for bit
+// QFUSE (int8, FP8): the prologue is the quantiser of sage_quant_kernels.h for this workgroup's queries, operation for
+// operation (absmax, scale = absmax / 127 or 1, x8 = clamp(rint(x * (1 / scale)), +-127); FP8: absmax / 448 and the
+// saturating E4M3 conversion of x * (1 / scale)), so the result is bit for bit
 // that of quantising first; p.sq_out / p.q8_out, where not null, receive the scales and the codes.  Two forms: with K
 // scales over whole tiles, p.q holds bf16 values and a scale covers a block of 128 queries; with PER_KEY, p.q holds
 // f32 values and every query has its own scale (the reference's convention, src/runtime/cuda_flash_sage.rs:201-223).
 template <int D, bool CAUSAL, int MODE, bool OUT_F32, bool BIAS, int NW = 8, bool PER_KEY = false, bool QFUSE = false>
 __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned char *lds, int wg_linear)
 {
-    static_assert(!QFUSE || BIAS, "the fused Q quantiser is an int8 device");
+    static_assert(!QFUSE || MODE != MODE_BF16, "the fused Q quantiser produces 8-bit operands");
+    static_assert(!QFUSE || BIAS || MODE == MODE_FP8, "int8 with the fused Q quantiser runs on biased logits");
+    static_assert(!(QFUSE && PER_KEY && MODE == MODE_FP8), "rows form: int8 only");
     constexpr bool QROWS = QFUSE && PER_KEY;  // f32 queries, a scale per query
     static_assert(!BIAS || MODE == MODE_I8, "biased accumulators are an int8 device");
     static_assert(!PER_KEY || BIAS || MODE == MODE_FP8, "per-key scales: int8 (on the biased accumulators) and FP8");
@@ -764,16 +767,31 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             const int w0 = wave & ~3;
             mx = fmaxf(fmaxf(red[w0], red[w0 + 1]), fmaxf(red[w0 + 2], red[w0 + 3]));
         }
-        const float scale = (mx > 0.f) ? mx / 127.0f : 1.f;
+        constexpr float QMAX = (MODE == MODE_FP8) ? 448.0f : 127.0f;
+        const float scale = (mx > 0.f) ? mx / QMAX : 1.f;
         const float inv = 1.f / scale;
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
             uint32_t w[4] = {0u, 0u, 0u, 0u};
+            if constexpr (MODE == MODE_FP8) {
+                // E4M3, round to nearest even, saturating: the clamp first, as the pre-pass quantiser does
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                int iv = (int)rintf(val(s, e) * inv);
-                iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
-                w[e >> 2] |= ((uint32_t)iv & 0xffu) << ((e & 3) * 8);
+                for (int j = 0; j < 4; ++j) {
+                    float c[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) c[i] = fminf(fmaxf(val(s, 4 * j + i) * inv, -448.0f), 448.0f);
+                    int r = 0;
+                    r = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], r, false);
+                    r = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], r, true);
+                    w[j] = (uint32_t)r;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    int iv = (int)rintf(val(s, e) * inv);
+                    iv = iv < -127 ? -127 : (iv > 127 ? 127 : iv);
+                    w[e >> 2] |= ((uint32_t)iv & 0xffu) << ((e & 3) * 8);
+                }
             }
             qreg[s] = make_uint4(w[0], w[1], w[2], w[3]);
         }
@@ -786,7 +804,7 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
             float wg_mx = red[0];
 #pragma unroll
             for (int w = 1; w < NW; ++w) wg_mx = fmaxf(wg_mx, red[w]);
-            mq = (wg_mx > 0.f) ? wg_mx / 127.0f : 1.f;
+            mq = (wg_mx > 0.f) ? wg_mx / QMAX : 1.f;
             const int blk = q_row >> 7, nqb = (N + 127) >> 7;
             if (p.sq_out != nullptr && lane == 0 && (wave & 3) == 0 && blk < nqb) p.sq_out[(size_t)bh * nqb + blk] = scale;
         }

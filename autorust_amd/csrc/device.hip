@@ -476,6 +476,10 @@ const named_entry NAMED[] = {
     {"ar_flash_sage_qf_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
     {"ar_flash_sage_qf_mid", 7, 9, 256, 128, false, true, true, 0, false},
     {"ar_flash_sage_qf_mid_lens", 8, 9, 256, 128, false, true, true, 0, false},
+    {"ar_flash_sage_fp8_qf_long", 7, 9, 512, 256, false, true, true, 0, false},
+    {"ar_flash_sage_fp8_qf_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
+    {"ar_flash_sage_fp8_qf_mid", 7, 9, 256, 128, false, true, true, 0, false},
+    {"ar_flash_sage_fp8_qf_mid_lens", 8, 9, 256, 128, false, true, true, 0, false},
     {"ar_flash_sage_qr_long", 7, 9, 512, 256, false, true, true, 0, false},
     {"ar_flash_sage_qr_long_lens", 8, 9, 512, 256, false, true, true, 0, false},
     {"ar_flash_sage_qr_mid", 7, 9, 256, 128, false, true, true, 0, false},

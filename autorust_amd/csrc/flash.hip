@@ -359,21 +359,21 @@ static int sage_fwd_impl(arhip_device *dev, const int8_t *q8, const int8_t *k8,
 }
 
 // Q quantised inside the attention kernel (as the reference does, src/runtime/cuda_flash_sage.rs:201-223): the
-// pipelined int8 kernel with bf16 queries, scales over blocks of 128 queries.
-extern "C" int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const int8_t *k8, const float *sk,
-                                     const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
-                                     int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
-                                     int causal, int out_dtype, float scale, int wait, double *secs)
+// pipelined int8 (FP8) kernel with bf16 queries, scales over blocks of 128 queries.
+static int sage_fwd_qfused_impl(const char *who, bool fp8, arhip_device *dev, const uint16_t *q, const int8_t *k8, const float *sk,
+                               const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
+                               int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
+                               int causal, int out_dtype, float scale, int wait, double *secs)
 {
-    if (int rc = check_common("arhip_sage_fwd_qfused", dev, q, k8, v, o, nullptr, B, Hq, Hkv, N, D)) return rc;
-    ARHIP_REQUIRE(sk, "arhip_sage_fwd_qfused: null scale pointer");
-    ARHIP_REQUIRE(out_dtype == ARHIP_F32 || out_dtype == ARHIP_BF16, "arhip_sage_fwd_qfused: out_dtype %d", out_dtype);
+    if (int rc = check_common(who, dev, q, k8, v, o, nullptr, B, Hq, Hkv, N, D)) return rc;
+    ARHIP_REQUIRE(sk, "%s: null scale pointer", who);
+    ARHIP_REQUIRE(out_dtype == ARHIP_F32 || out_dtype == ARHIP_BF16, "%s: out_dtype %d", who, out_dtype);
     int shift = 0;
     while (((int64_t)64 << shift) < bk) ++shift;
-    ARHIP_REQUIRE(((int64_t)64 << shift) == bk, "arhip_sage_fwd_qfused: K scales over whole 64-key tiles (bk = 64 * 2^j), got bk = %lld",
+    ARHIP_REQUIRE(((int64_t)64 << shift) == bk, "%s: K scales over whole 64-key tiles (bk = 64 * 2^j), got bk = %lld", who,
                   (long long)bk);
-    ARHIP_REQUIRE(pipe_addressable(N, D, 2), "arhip_sage_fwd_qfused: (N + 320) * D * 2 must stay below 2^31 (N = %lld)", (long long)N);
-    ARHIP_REQUIRE(q8_out == nullptr || arhip_aligned16(q8_out), "arhip_sage_fwd_qfused: q8_out must be 16-byte aligned");
+    ARHIP_REQUIRE(pipe_addressable(N, D, 2), "%s: (N + 320) * D * 2 must stay below 2^31 (N = %lld)", who, (long long)N);
+    ARHIP_REQUIRE(q8_out == nullptr || arhip_aligned16(q8_out), "%s: q8_out must be 16-byte aligned", who);
     ARHIP_HIP(hipSetDevice(dev->ordinal));
     AttnParams p = {};
     p.q = q; p.k = k8; p.v = v; p.o = o;
@@ -398,9 +398,29 @@ extern "C" int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const
     arhip_call_timer t{dev, wait, secs};
     t.kernel = ARHIP_K_SAGE;
     if (int rc = t.begin()) return rc;
-    launch_pipe_i8_qf(dev->stream, p, (int)D, c, nw);
+    if (fp8) launch_pipe_fp8_qf(dev->stream, p, (int)D, c, nw);
+    else launch_pipe_i8_qf(dev->stream, p, (int)D, c, nw);
     arhip_note_selected(ARHIP_K_SAGE);
     return t.end();
+}
+
+extern "C" int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const int8_t *k8, const float *sk,
+                                     const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
+                                     int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
+                                     int causal, int out_dtype, float scale, int wait, double *secs)
+{
+    return sage_fwd_qfused_impl("arhip_sage_fwd_qfused", false, dev, q, k8, sk, v, o, sq_out, q8_out, kv_len, B, Hq, Hkv, N, D, bk,
+                                causal, out_dtype, scale, wait, secs);
+}
+
+// The same on E4M3 codes (k8 from arhip_sage_quant_fp8; the kernel derives E4M3 codes of Q with scale = absmax / 448).
+extern "C" int arhip_sage_fwd_fp8_qfused(arhip_device *dev, const uint16_t *q, const uint8_t *k8, const float *sk,
+                                         const uint16_t *v, void *o, float *sq_out, uint8_t *q8_out, const int32_t *kv_len,
+                                         int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
+                                         int causal, int out_dtype, float scale, int wait, double *secs)
+{
+    return sage_fwd_qfused_impl("arhip_sage_fwd_fp8_qfused", true, dev, q, (const int8_t *)k8, sk, v, o, sq_out, (int8_t *)q8_out,
+                                kv_len, B, Hq, Hkv, N, D, bk, causal, out_dtype, scale, wait, secs);
 }
 
 // The reference's own convention in one attention launch: f32 queries quantised row by row inside the kernel

@@ -485,7 +485,7 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
     const bool pipelined = !has_mask && (tile_uniform || key_scales) && long_variant(n, d);
     // bf16 queries with scales over blocks of 128 are quantised by the attention kernel itself (as the reference's
     // kernel does, cuda_flash_sage.rs:201-223): one launch and one pass over Q fewer
-    const bool q_fused = pipelined && tile_uniform && bf16_in && bq == 128 && !st.sage_fp8;
+    const bool q_fused = pipelined && tile_uniform && bf16_in && bq == 128;
     // f32 queries with a scale each and K scales per key (the reference's own convention): the same, row by row
     const bool q_rows = pipelined && key_scales && !bf16_in && bq == 1 && !st.sage_fp8;
     if (!q_fused && !q_rows) quant(q, q8, sq, h, bq, nqb, false);
@@ -522,7 +522,9 @@ std::vector<HostCall> attention_host_calls(const Tensor &q, const Tensor &k, con
         const bool mid = mid_variant(dev, b, h, n, d, is_causal, key_lengths != nullptr);
         const std::array<int64_t, 3> grid = {mid ? (n + 127) / 128 : (n + 255) / 256, b * h, 1}, block = {mid ? 256 : 512, 1, 1};
         if (q_fused)   // Q itself in the first slot; the scales slot is written
-            calls.push_back(attn_call(mid ? "ar_flash_sage_qf_mid" : "ar_flash_sage_qf_long", {q, k8, vb, out, mslot, sq, sk},
+            calls.push_back(attn_call(st.sage_fp8 ? (mid ? "ar_flash_sage_fp8_qf_mid" : "ar_flash_sage_fp8_qf_long")
+                                                  : (mid ? "ar_flash_sage_qf_mid" : "ar_flash_sage_qf_long"),
+                                      {q, k8, vb, out, mslot, sq, sk},
                                       {BF, I8, BF, X, F, F, F}, grid, block, svals));
         else if (q_rows)
             calls.push_back(attn_call(mid ? "ar_flash_sage_qr_mid" : "ar_flash_sage_qr_long", {q, k8, vb, out, mslot, sq, sk},

@@ -16,6 +16,7 @@ void launch_pipe_i8_keys(hipStream_t stream, const AttnParams &p, int D, bool ca
 void launch_pipe_i8_qf(hipStream_t stream, const AttnParams &p, int D, bool causal, int nw);    // bf16 queries, quantised in the prologue
 void launch_pipe_i8_keys_qf(hipStream_t stream, const AttnParams &p, int D, bool causal, int nw);  // f32 queries, a scale per query and per key
 void launch_pipe_fp8(hipStream_t stream, const AttnParams &p, int D, bool causal, int nw);
+void launch_pipe_fp8_qf(hipStream_t stream, const AttnParams &p, int D, bool causal, int nw);   // bf16 queries, quantised in the prologue
 void launch_pipe_fp8_keys(hipStream_t stream, const AttnParams &p, int D, bool causal, int nw);
 
 }  // namespace arhip

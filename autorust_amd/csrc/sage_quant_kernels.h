@@ -96,6 +96,14 @@ __device__ __forceinline__ void k_mean_final_body(const float *part, float *mean
     const float *p = part + (size_t)bh * nchunk * D + d;
     float tot = 0.f;
     int c = 0;
+    // few waves run this kernel (one per 64 channels of a head), so its time is the number of load round trips
+    for (; c + 32 <= nchunk; c += 32) {
+        float v[32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) v[i] = p[(size_t)(c + i) * D];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) tot += v[i];
+    }
     for (; c + 8 <= nchunk; c += 8) {
         float v[8];
 #pragma unroll

@@ -236,14 +236,15 @@ class Device:
         return s.value if wait else None
 
     def sage_fwd_qfused(self, q, k8, sk, v, o, B, Hq, Hkv, N, D, bk, out_dtype=BF16, sq_out=None, q8_out=None, kv_len=None,
-                        causal=False, scale=None, wait=True):
+                        causal=False, scale=None, wait=True, fp8=False):
         """sage_quant of Q (bf16, blocks of 128 queries) inside the attention kernel; sq_out / q8_out receive the
-        scales and codes it derived."""
+        scales and codes it derived.  fp8: E4M3 codes (k8 from sage_quant_fp8)."""
         scale = float(1.0 / np.sqrt(np.float32(D))) if scale is None else float(scale)
         s = ctypes.c_double()
-        check(self.lib.arhip_sage_fwd_qfused(self.handle, self._ptr(q), self._ptr(k8), self._ptr(sk), self._ptr(v), self._ptr(o),
-                                             self._ptr(sq_out), self._ptr(q8_out), self._ptr(kv_len), B, Hq, Hkv, N, D, bk,
-                                             int(causal), out_dtype, scale, int(wait), ctypes.byref(s)))
+        fn = self.lib.arhip_sage_fwd_fp8_qfused if fp8 else self.lib.arhip_sage_fwd_qfused
+        check(fn(self.handle, self._ptr(q), self._ptr(k8), self._ptr(sk), self._ptr(v), self._ptr(o),
+                 self._ptr(sq_out), self._ptr(q8_out), self._ptr(kv_len), B, Hq, Hkv, N, D, bk,
+                 int(causal), out_dtype, scale, int(wait), ctypes.byref(s)))
         return s.value if wait else None
 
     def sage_prep_kv_rows(self, k, k8, sk, v, vb, B, Hkv, N, D, wait=True):

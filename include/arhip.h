@@ -109,7 +109,7 @@ int arhip_graph_destroy(arhip_device *dev, void *graph_exec);
  * image: a gfx950 code object (hipcc --genco), or a container of several that are looked up as
  * one: "ARHIPKO1", uint32 count, uint32 0, then per code object uint64 size and its bytes padded
  * to a multiple of 16 (autorust_amd/attn_kernels.hsaco is such a file: its entry points compile as
- * thirteen code objects side by side).  Modules are cached per device by content hash.  args: nbufs device pointers followed by nvals scalars;
+ * fifteen code objects side by side).  Modules are cached per device by content hash.  args: nbufs device pointers followed by nvals scalars;
  * val_bits[i] in {32, 64} narrows vals[i] like the reference's signature
  * dtype does.  grid is in blocks. */
 int arhip_module_load(arhip_device *dev, const void *image, size_t len, void **module);
@@ -273,6 +273,14 @@ int arhip_sage_fwd_qfused(arhip_device *dev, const uint16_t *q, const int8_t *k8
                           const uint16_t *v, void *o, float *sq_out, int8_t *q8_out, const int32_t *kv_len,
                           int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
                           int causal, int out_dtype, float scale, int wait, double *secs);
+
+/* arhip_sage_fwd_fp8_qfused: the same on E4M3 codes (the reference's AR_FP8 branch, src/runtime/cuda_flash_sage.rs:125-128):
+ *   k8 / sk from arhip_sage_quant_fp8; the kernel derives the codes of q with scale = absmax / 448; bit for bit
+ *   arhip_sage_quant_fp8 on q followed by arhip_sage_fwd_fp8. */
+int arhip_sage_fwd_fp8_qfused(arhip_device *dev, const uint16_t *q, const uint8_t *k8, const float *sk,
+                              const uint16_t *v, void *o, float *sq_out, uint8_t *q8_out, const int32_t *kv_len,
+                              int64_t B, int64_t Hq, int64_t Hkv, int64_t N, int64_t D, int64_t bk,
+                              int causal, int out_dtype, float scale, int wait, double *secs);
 
 /* arhip_sage_fwd_qfused_rows: the same for the reference's own convention: q f32 [B,Hq,N,D], a scale
  *   per query (sq_out [B,Hq,N]), k8 / sk from arhip_sage_quant with bk = 1 (or a power of two below

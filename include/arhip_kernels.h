@@ -6,7 +6,7 @@
  * reference's `HostCall{src, name, signature, bufs, global, local, vals}` ->
  * `Compiled::run_host_kernel` -> `Prog::call` does (src/engine/session.rs:210-256,
  * src/runtime/device.rs:383-402), load the file with arhip_module_load and launch these with
- * arhip_launch.  (The file is a container of thirteen code objects, see arhip_module_load in
+ * arhip_launch.  (The file is a container of fifteen code objects, see arhip_module_load in
  * arhip.h; a host that wants hipModuleLoadData / hipModuleLaunchKernel itself loads each part,
  * or builds csrc/attn_entry.hip without -DARHIP_ENTRY_PART as one plain code object.)
  * Arguments are device pointers followed by scalars, in the reference's order
@@ -129,7 +129,16 @@
  *     Q    bf16 [b*hq, n, head_dim] instead of int8 codes
  *     SQ   [b*hq, ceil(n/128)] f32, WRITTEN: the scales the kernel derived (bq must be 128)
  * K8 / SK as the K quantiser left them, bk = 64 * 2^j.  Bit-identical to ar_sage_quant_blocks_bf16 on Q followed
- * by ar_flash_sage_long / _mid. */
+ * by ar_flash_sage_long / _mid.  The _fp8_ entries do the same on E4M3 codes (scale = absmax / 448): bit-identical to
+ * ar_sage_quant_blocks_fp8_bf16 on Q followed by ar_flash_sage_fp8_long / _mid. */
+#define ARHIP_KERNEL_FLASH_SAGE_QF_LONG "ar_flash_sage_qf_long"
+#define ARHIP_KERNEL_FLASH_SAGE_QF_MID "ar_flash_sage_qf_mid"
+#define ARHIP_KERNEL_FLASH_SAGE_QF_LONG_LENS "ar_flash_sage_qf_long_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_QF_MID_LENS "ar_flash_sage_qf_mid_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_QF_LONG "ar_flash_sage_fp8_qf_long"
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_QF_MID "ar_flash_sage_fp8_qf_mid"
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_QF_LONG_LENS "ar_flash_sage_fp8_qf_long_lens"
+#define ARHIP_KERNEL_FLASH_SAGE_FP8_QF_MID_LENS "ar_flash_sage_fp8_qf_mid_lens"
 /* The reference's own convention in one launch: the argument lists of ar_flash_sage_long / _mid (and _lens) with
  *     Q    f32 [b*hq, n, head_dim], quantised row by row in the kernel's prologue
  *     SQ   [b*hq, n] f32, WRITTEN: one scale per query (bq must be 1)
@@ -139,10 +148,6 @@
 #define ARHIP_KERNEL_FLASH_SAGE_QR_MID "ar_flash_sage_qr_mid"
 #define ARHIP_KERNEL_FLASH_SAGE_QR_LONG_LENS "ar_flash_sage_qr_long_lens"
 #define ARHIP_KERNEL_FLASH_SAGE_QR_MID_LENS "ar_flash_sage_qr_mid_lens"
-#define ARHIP_KERNEL_FLASH_SAGE_QF_LONG "ar_flash_sage_qf_long"
-#define ARHIP_KERNEL_FLASH_SAGE_QF_MID "ar_flash_sage_qf_mid"
-#define ARHIP_KERNEL_FLASH_SAGE_QF_LONG_LENS "ar_flash_sage_qf_long_lens"
-#define ARHIP_KERNEL_FLASH_SAGE_QF_MID_LENS "ar_flash_sage_qf_mid_lens"
 
 /* FP8 E4M3 variant (the reference's `src(fp8 = true)`, src/runtime/cuda_flash_sage.rs:82-84, 92-147):
  * the same argument lists as ar_flash_sage / ar_sage_quant_{blocks,rows}_*, with E4M3 codes

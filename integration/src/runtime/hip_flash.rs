@@ -17,7 +17,7 @@
 //! | `ar_flash_sage`      | 256   | `[ceil(n/128), b*h, 1]` | same `+ bq, bk`; buffers `+ SQ, SK`; O is f32|
 //! | `ar_flash_sage_long` | 512   | `[ceil(n/256), b*h, 1]` | same `+ bq, bk, out_f32`                     |
 //! | `ar_flash_sage_mid`  | 256   | `[ceil(n/128), b*h, 1]` | same; the pipelined kernel with 4 waves      |
-//! | `ar_flash_sage_qf_long`, `ar_flash_sage_qf_mid` | as `_long` / `_mid` | first buffer: the bf16 queries themselves; `SQ` is written (`bq` 128, `bk` 64·2^j) |
+//! | `ar_flash_sage_qf_long`, `ar_flash_sage_qf_mid`, `ar_flash_sage_fp8_qf_long`, `ar_flash_sage_fp8_qf_mid` | as `_long` / `_mid` | first buffer: the bf16 queries themselves; `SQ` is written (`bq` 128, `bk` 64·2^j) |
 //! | `ar_flash_sage_qr_long`, `ar_flash_sage_qr_mid` | as `_long` / `_mid` | first buffer: the f32 queries themselves; `SQ` `[b*h, n]` is written (`bq` 1, `bk` a power of two below 64) |
 //! | `ar_flash_sage_fp8`, `ar_flash_sage_fp8_long`, `ar_flash_sage_fp8_mid` | as the int8 entries, on E4M3 codes (`SageOptions::fp8`) |
 //! | `<entry>_lens`       | as `<entry>` | as `<entry>`     | one more buffer after the mask slot: `L`, int32 `[b]` key lengths |
@@ -264,7 +264,7 @@ pub fn host_calls_sage(
     let pipelined = !opts.has_mask && (tile_uniform || key_scales) && long_variant(n, d);
     // bf16 queries with scales over blocks of 128 are quantised by the attention kernel itself (as the CUDA
     // kernel does): one launch and one pass over Q fewer
-    let q_fused = pipelined && tile_uniform && bf16_in && bq == 128 && !sage.fp8;
+    let q_fused = pipelined && tile_uniform && bf16_in && bq == 128;
     // f32 queries with a scale each and K scales per key (the CUDA kernel's own convention): the same, row by row
     let q_rows = pipelined && key_scales && !bf16_in && bq == 1 && !sage.fp8;
     if !q_fused && !q_rows {
@@ -309,7 +309,12 @@ pub fn host_calls_sage(
         let (grid, block) = if mid { ([(n + 127) / 128, b * h, 1], [256, 1, 1]) } else { ([(n + 255) / 256, b * h, 1], [512, 1, 1]) };
         if q_fused {
             // Q itself in the first slot; the scales slot is written
-            let name = if mid { "ar_flash_sage_qf_mid" } else { "ar_flash_sage_qf_long" };
+            let name = match (sage.fp8, mid) {
+                (false, true) => "ar_flash_sage_qf_mid",
+                (false, false) => "ar_flash_sage_qf_long",
+                (true, true) => "ar_flash_sage_fp8_qf_mid",
+                (true, false) => "ar_flash_sage_fp8_qf_long",
+            };
             calls.push(attn_call(name, vec![q, s.k8, vb, o, mask, s.sq, s.sk], &[bf, i8t, bf, x, f, f, f], lens, grid, block, sv));
         } else if q_rows {
             let name = if mid { "ar_flash_sage_qr_mid" } else { "ar_flash_sage_qr_long" };

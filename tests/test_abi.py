@@ -81,7 +81,7 @@ def test_code_object_is_built_and_names_every_entry_point():
     """The named kernels (include/arhip_kernels.h) are all in the code object (no launch here)."""
     text = open(os.path.join(ROOT, "include", "arhip_kernels.h")).read()
     names = re.findall(r'#define ARHIP_KERNEL_\w+ "(\w+)"', text)
-    assert len(names) == 49
+    assert len(names) == 53
     image = open(_lib.KERNELS_PATH, "rb").read()
     for n in names:
         assert n.encode() + b"\0" in image or n.encode() in image, n
@@ -95,7 +95,7 @@ def test_code_object_file_is_a_container_of_elf_parts():
     image = open(_lib.KERNELS_PATH, "rb").read()
     assert image[:8] == b"ARHIPKO1"
     count, zero = struct.unpack_from("<II", image, 8)
-    assert count == 13 and zero == 0
+    assert count == 15 and zero == 0
     at, parts = 16, []
     for _ in range(count):
         (size,) = struct.unpack_from("<Q", image, at)

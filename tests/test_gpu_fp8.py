@@ -129,3 +129,42 @@ def test_fp8_attention_against_exact(dev):
 def test_fp8_has_no_logits_export(dev):
     from autorust_amd import _lib
     assert "arhip_sage_fwd_fp8" in _lib.SIGNATURES and len(_lib.SIGNATURES["arhip_sage_fwd_fp8"][1]) == 21
+
+
+@pytest.mark.parametrize("B,H,Hkv,N,D,causal,use_len,out_dtype", [
+    (1, 32, 32, 2304, 128, False, False, BF16),        # 8 waves per workgroup
+    (2, 8, 4, 1000, 128, True, True, F32),
+    (2, 6, 3, 300, 64, True, False, BF16),
+    (1, 2, 2, 1, 64, False, False, F32),
+])
+def test_fp8_q_quantiser_inside_the_attention_kernel(dev, B, H, Hkv, N, D, causal, use_len, out_dtype):
+    """arhip_sage_fwd_fp8_qfused: the E4M3 quantiser of Q (scale = absmax / 448 over blocks of 128 queries,
+    src/runtime/cuda_flash_sage.rs:9, 125-128) in the prologue of the pipelined kernel.  The codes and scales it
+    exports are the oracle's bit for bit, and the output is bit for bit that of quantising first."""
+    from autorust_amd import _lib
+    q = oracle.bf16_round(synth.normal(911, (B, H, N, D)) * (np.float32(2.0) ** np.linspace(-3, 3, H, dtype=np.float32))[None, :, None, None])
+    k = oracle.bf16_round(synth.normal(912, (B, Hkv, N, D)) + np.float32(1.5) * synth.normal(914, (1, Hkv, 1, D)))
+    v = synth.normal(913, (B, Hkv, N, D))
+    if N > 256:
+        q[0, 0, 128:256] = 0.0                                 # an all-zero block: scale 1
+    kv_len = np.array([N - 77, max(1, N // 3)][:B], np.int32) if use_len else None
+    _, k8h, _, skh, want = run_fp8(dev, q, k, v, 128, 64, True, in_dtype=BF16, out_dtype=out_dtype, kv_len=kv_len, causal=causal)
+    nqb = (N + 127) // 128
+    with Bufs(dev) as bufs:
+        dq = bufs.put(synth.to_bf16_bits(q))
+        k8, sk = bufs.put(k8h), bufs.put(skh)
+        dv = bufs.put(synth.to_bf16_bits(v))
+        do = bufs.new(q.size * (4 if out_dtype == F32 else 2))
+        sq_out, q8_out = bufs.new(B * H * nqb * 4), bufs.new(q.size)
+        dl = bufs.put(kv_len) if use_len else None
+        dev.sage_fwd_qfused(dq, k8, sk, dv, do, B, H, Hkv, N, D, 64, out_dtype=out_dtype, sq_out=sq_out, q8_out=q8_out,
+                            kv_len=dl, causal=causal, fp8=True)
+        got = do.copyout(np.float32, q.shape) if out_dtype == F32 else synth.from_bf16_bits(do.copyout(np.uint16, q.shape))
+        got_sq, got_q8 = sq_out.copyout(np.float32, (B, H, nqb)), q8_out.copyout(np.uint8, q.shape)
+        with pytest.raises(_lib.ArhipError, match="whole 64-key tiles"):
+            dev.sage_fwd_qfused(dq, k8, sk, dv, do, B, H, Hkv, N, D, 32, out_dtype=out_dtype, fp8=True)
+    w_q8, w_sq = oracle.quant_blocks_fp8(q, 128)
+    assert np.array_equal(got_sq, w_sq) and np.array_equal(got_q8, w_q8)
+    if N > 256:
+        assert w_sq[0, 0, 1] == 1.0
+    assert np.array_equal(got, want)

@@ -571,3 +571,43 @@ def test_ar_sage_quant_rows_cast_by_name(dev, kernels, b, hkv, n, d):
     for g in (got, typed):
         assert np.array_equal(g[0], w8) and np.array_equal(g[1], ws)
         assert np.array_equal(g[2], synth.to_bf16_bits(v))
+
+
+@pytest.mark.parametrize("form,per_wg,block", [("long", 256, 512), ("mid", 128, 256)])
+@pytest.mark.parametrize("d,causal,out_f32,with_lens", [(128, False, 0, False), (64, True, 1, True)])
+def test_ar_flash_sage_fp8_qf_by_name(dev, kernels, form, per_wg, block, d, causal, out_f32, with_lens):
+    """The FP8 entries that quantise the bf16 queries in their prologue: the scales they write are
+    ar_sage_quant_blocks_fp8_bf16's, the output is bit for bit that of that quantiser followed by the plain FP8 entry
+    of the same form."""
+    b, hq, hkv, n, bq, bk = 2, 4, 2, 700, 128, 64
+    q = oracle.bf16_round(synth.normal(61, (b, hq, n, d)))
+    k = oracle.bf16_round(synth.normal(62, (b, hkv, n, d)))
+    v = synth.normal(63, (b, hkv, n, d))
+    lens = np.array([333, n], np.int32) if with_lens else None
+    sfx = "_lens" if with_lens else ""
+    with Bufs(dev) as bufs:
+        def quant(x, blk, heads):
+            dx, x8 = bufs.put(synth.to_bf16_bits(x)), bufs.new(x.size)
+            nblk = (n + blk - 1) // blk
+            sc, mean = bufs.new(b * heads * nblk * 4), bufs.new(b * heads * d * 4)
+            dev.launch(kernels, "ar_sage_quant_blocks_fp8_bf16", (nblk, b * heads, 1), (256, 1, 1), [dx, x8, sc, mean],
+                       [n, d, blk, nblk, 0])
+            return dx, x8, sc
+        dq, q8, sq = quant(q, bq, hq)
+        _, k8, sk = quant(k, bk, hkv)
+        dv = bufs.put(synth.to_bf16_bits(v))
+        do, dp = bufs.new(q.size * 4), bufs.new(q.size * 4)
+        sq2 = bufs.new(b * hq * ((n + bq - 1) // bq) * 4)
+        dl = [bufs.put(lens)] if with_lens else []
+        vals = [n, d, int(causal), 0, hq, hkv, bq, bk, out_f32]
+        name = "ar_flash_sage_fp8_qf_" + form + sfx
+        dev.launch(kernels, name, _grid(n, per_wg, b, hq), (block, 1, 1), [dq, k8, dv, do, do] + dl + [sq2, sk], vals)
+        dev.launch(kernels, "ar_flash_sage_fp8_" + form + sfx, _grid(n, per_wg, b, hq), (block, 1, 1), [q8, k8, dv, dp, dp] + dl + [sq, sk], vals)
+        words = q.size if out_f32 else q.size // 2
+        got, plain = do.copyout(np.uint32, (words,)), dp.copyout(np.uint32, (words,))
+        got_sq, h_sq = sq2.copyout(np.float32, (b, hq, (n + bq - 1) // bq)), sq.copyout(np.float32, (b, hq, (n + bq - 1) // bq))
+        with pytest.raises(_lib.ArhipError, match="blocks of 128 queries"):
+            dev.launch(kernels, name, _grid(n, per_wg, b, hq), (block, 1, 1), [dq, k8, dv, do, do] + dl + [sq2, sk],
+                       [n, d, int(causal), 0, hq, hkv, 64, bk, out_f32])
+    assert np.array_equal(got_sq, h_sq) and np.array_equal(h_sq, oracle.quant_blocks_fp8(q, bq)[1])
+    assert np.array_equal(got, plain)

@@ -218,6 +218,14 @@ def test_sage_fp8_setting(hdev):
     names = [sess.step(i)[0] for i in range(n_calls)]
     assert names[0] == "ar_sage_quant_blocks_fp8_f32" and "ar_flash_sage_fp8_mid" in names
     assert float(np.abs(out.to_list() - oracle.sdpa_f64(q, k, v, causal=True)).max()) < 6e-2
+    # bf16 tensors: the FP8 attention kernel quantises the queries itself, as the int8 one does
+    bq_, bk_, bv_ = (Tensor.from_slice(hdev, a, a.shape, BFLOAT16) for a in (q, k, v))
+    sess.begin_capture()
+    outb = bq_.sage_attention_with(bk_, bv_, None, 0.0, True, sess, st)
+    n_calls = sess.end_capture()
+    names = [sess.step(i)[0] for i in range(n_calls)]
+    assert names == ["ar_sage_kmean_partial_bf16", "ar_sage_kmean_final", "ar_sage_quant_blocks_fp8_bf16", "ar_flash_sage_fp8_qf_mid"]
+    assert float(np.abs(outb.to_list() - oracle.sdpa_f64(q, k, v, causal=True)).max()) < 6e-2
     # enough long 256-query workgroups: the 8-wave pipelined FP8 entry, as for int8
     b, h, n = 2, 32, 2048
     q, k, v = _fill((b, h, n, d), 3), _fill((b, h, n, d), 11), _fill((b, h, n, d), 19)
