@@ -104,6 +104,8 @@ __device__ __forceinline__ void flash_f32_entry(float *lds, const float *Q, cons
     p.kv_len = L;
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nq = (int)gridDim.x;
+    p.total = (int)(gridDim.x * gridDim.y);
+    p.lpt_heads = (p.total <= 16 * 256) ? (int)gridDim.y : 0;  // few workgroups per compute unit: longest first over all heads
     dense(p.qs, hq, N, head_dim);
     dense(p.ks, hkv, N, head_dim);
     dense(p.os, hq, N, head_dim);
@@ -146,6 +148,8 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_fwd(const float *Q, cons
     p.mask = has_mask ? M : nullptr;
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nq = (int)gridDim.x;
+    p.total = (int)(gridDim.x * gridDim.y);
+    p.lpt_heads = (p.total <= 16 * 256) ? (int)gridDim.y : 0;  // few workgroups per compute unit: longest first over all heads
     dense(p.qs, hq, N, head_dim);
     dense(p.ks, hkv, N, head_dim);
     dense(p.os, hq, N, head_dim);
@@ -173,6 +177,8 @@ __device__ __forceinline__ void flash_f32_short(const float *Q, const float *K, 
     p.mask = has_mask ? M : nullptr;
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nq = (int)gridDim.x;
+    p.total = (int)(gridDim.x * gridDim.y);
+    p.lpt_heads = (p.total <= 16 * 256) ? (int)gridDim.y : 0;  // few workgroups per compute unit: longest first over all heads
     dense(p.qs, hq, N, 64);
     dense(p.ks, hkv, N, 64);
     dense(p.os, hq, N, 64);
@@ -220,6 +226,8 @@ __device__ __forceinline__ FlashBwdParams bwd_params(const float *Q, const float
     p.mask = has_mask ? M : nullptr;
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nt = (int)gridDim.x;
+    p.total_q = p.total_kv = (int)(gridDim.x * gridDim.y);
+    p.lpt_q = p.lpt_kv = (p.total_q <= 16 * 256) ? (int)gridDim.y : 0;  // few workgroups per compute unit: longest first over all heads
     p.scale = 1.0f / __builtin_sqrtf((float)head_dim);
     return p;
 }

@@ -32,6 +32,8 @@ struct FlashBwdParams {
     float *dq, *dk, *dv;
     int Hq, Hkv, N;
     int nt;  // tiles per head: query tiles (dQ kernel) or key tiles (dK/dV kernel)
+    int total_q, total_kv;  // workgroups in the dQ grid (nt * B * Hq) and in the dK/dV grid (nt * B * Hkv)
+    int lpt_q, lpt_kv;  // causal, few workgroups per compute unit: B * Hq / B * Hkv, and the grids run longest tile first over all heads; else 0
     float scale;
 };
 
@@ -86,9 +88,15 @@ __device__ __forceinline__ void bwd_dq_body(const FlashBwdParams &p, float *lds,
     float *vs = ks + F32_BK * ROW;
     const int stid = SPLIT ? lane : tid;      // index among the threads staging a tile
     const int i32 = lane & 31, h = lane >> 5;
-    const int bh = wg_linear / p.nt;
-    int qt = wg_linear - bh * p.nt;
-    if (CAUSAL) qt = p.nt - 1 - qt;
+    // every XCD (consecutive workgroups go to different ones) gets a contiguous range of heads
+    const int wg_x = (p.total_q > 0 && (p.total_q & 7) == 0) ? (wg_linear & 7) * (p.total_q >> 3) + (wg_linear >> 3) : wg_linear;
+    int bh = wg_x / p.nt;
+    int qt = wg_x - bh * p.nt;
+    if (CAUSAL) qt = p.nt - 1 - qt;  // the longest query tiles first, within a head ...
+    if (CAUSAL && p.lpt_q > 0) {     // ... or over the whole grid
+        qt = p.nt - 1 - wg_linear / p.lpt_q;
+        bh = wg_linear % p.lpt_q;
+    }
     const int b = bh / p.Hq, head = bh - b * p.Hq;
     const int N = p.N;
     const int qblk = qt * BQ;
@@ -272,8 +280,13 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
     float *stat = qs + 2 * F32_BK * ROW;  // lse[32], D[32] of the staged queries
     const int stid = SPLIT ? lane : tid;      // index among the threads staging a tile
     const int i32 = lane & 31, h = lane >> 5;
-    const int kv_bh = wg_linear / p.nt;
-    const int kt = wg_linear - kv_bh * p.nt;
+    const int wg_x = (p.total_kv > 0 && (p.total_kv & 7) == 0) ? (wg_linear & 7) * (p.total_kv >> 3) + (wg_linear >> 3) : wg_linear;
+    int kv_bh = wg_x / p.nt;
+    int kt = wg_x - kv_bh * p.nt;  // causal: the first key tiles see the most queries
+    if (CAUSAL && p.lpt_kv > 0) {       // the longest over the whole grid first
+        kt = wg_linear / p.lpt_kv;
+        kv_bh = wg_linear % p.lpt_kv;
+    }
     const int b = kv_bh / p.Hkv, kvh = kv_bh - b * p.Hkv;
     const int group = p.Hq / p.Hkv;
     const int N = p.N;
@@ -348,9 +361,8 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
     constexpr int STEP = SPLIT ? NW : 1;
     const int first = SPLIT ? wave : 0;
     if (first < steps) fetch(first);
-    for (int step = first; step < steps; step += STEP) {
-        const int g = step / (qtiles - qt0);
-        const int q0 = (qt0 + step - g * (qtiles - qt0)) * F32_BK;
+    // the staged tile of the previous step goes to LDS, the next one is requested
+    auto stage = [&](int step) __attribute__((always_inline)) {
         if (!SPLIT) __syncthreads();
 #pragma unroll
         for (int j = 0; j < PER_THREAD; ++j) {
@@ -365,7 +377,10 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
         }
         if (step + STEP < steps) fetch(step + STEP);
         if (!SPLIT) __syncthreads();
-        if (CAUSAL && q0 + F32_BK - 1 < wk0) continue;  // every query of the tile precedes this wave's keys
+    };
+    auto compute = [&](int step) __attribute__((always_inline)) {
+        const int g = step / (qtiles - qt0);
+        const int q0 = (qt0 + step - g * (qtiles - qt0)) * F32_BK;
 
         // S = Q K^T and dP = dO V^T: lane = key, register r = query 8 (r / 4) + 4 h + r % 4 of the tile
         f32x16_t s, dp;
@@ -387,6 +402,7 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
             dp = __builtin_amdgcn_mfma_f32_32x32x2f32(c.w, vr[st + 3], dp, 0, 0, 0);
         }
         float pr[16], ds[16];
+        const int kq = key - q0 - 4 * h;  // causal: query 8 gq + 4 h + t of the tile sees this lane's key iff kq <= 8 gq + t
 #pragma unroll
         for (int gq = 0; gq < 4; ++gq) {
             const float4 l4 = *(const float4 *)&stat[8 * gq + 4 * h];
@@ -398,7 +414,7 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
                 const int qi = q0 + 8 * gq + 4 * h + t;
                 float xv = fmaf(s[r], c2, -lv[t]);
                 if (p.mask != nullptr && qi < N) xv = fmaf(p.mask[(size_t)qi * N + jj], BWD_LOG2E, xv);
-                const bool dead = qi >= N || !key_live || (CAUSAL && key > qi) || !(lv[t] > BWD_LSE_FLOOR);
+                const bool dead = qi >= N || !key_live || (CAUSAL && kq > 8 * gq + t) || !(lv[t] > BWD_LSE_FLOOR);
                 pr[r] = dead ? 0.f : __builtin_amdgcn_exp2f(xv);
                 ds[r] = pr[r] * (dp[r] - dvv[t]) * p.scale;
             }
@@ -414,6 +430,25 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
                 dv[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(dcol[db * 32], pr[r], dv[db], 0, 0, 0);
                 dk[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(qcol[db * 32], ds[r], dk[db], 0, 0, 0);
             }
+        }
+    };
+    if constexpr (CAUSAL && !SPLIT) {
+        // Every query of the first `wave` tiles of a head precedes this wave's keys: those tiles are staged (all
+        // waves pass the same barriers) and not computed.  Two plain loops instead of a branch around the matrix
+        // work, which costs the register allocator the accumulators twice.
+        const int tiles = qtiles - qt0, nskip = min(wave, tiles);
+        for (int g = 0; g < group; ++g) {
+            for (int t = 0; t < nskip; ++t) stage(g * tiles + t);
+            for (int t = nskip; t < tiles; ++t) {
+                stage(g * tiles + t);
+                compute(g * tiles + t);
+            }
+        }
+    } else {
+        // (SPLIT: the tiles start at the workgroup's first key, so none lies wholly before its keys)
+        for (int step = first; step < steps; step += STEP) {
+            stage(step);
+            compute(step);
         }
     }
     if constexpr (SPLIT) {

@@ -35,6 +35,8 @@ struct FlashF32Params {
     const int32_t *kv_len;  // [B] or null
     float *lse;             // optional [B,Hq,N]: m + log(l), src/runtime/cuda_flash_train.rs:141
     int Hq, Hkv, N, nq;
+    int lpt_heads;  // causal, few workgroups per compute unit: B * Hq, and the grid runs longest query tile first over all heads; else 0
+    int total;      // workgroups in the grid (nq * B * Hq)
     long qs[3], ks[3], os[3];  // element strides [batch, head, token] of q / k,v / o (channel stride 1)
     float scale;
 };
@@ -73,9 +75,19 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     float *vs = ks + F32_BK * KROW;                // [F32_BK][D]
     const int stid = SPLITK ? lane : tid;          // index among the threads staging a tile
     const int i32 = lane & 31, h = lane >> 5;
-    const int bh = wg_linear / p.nq;
-    int qt = wg_linear - bh * p.nq;
+    // causal: the longest query tiles first, within a head or (few, very unequal workgroups per compute unit) over
+    // the whole grid, so that no head's long tiles are left for the end
+    // Consecutive workgroups go to different XCDs (8, each with its own L2): every XCD gets a contiguous range of
+    // heads, so that the query tiles sharing a head's K/V meet in one L2 and, under the causal mask, every XCD gets
+    // tiles of every length.
+    const int wg_x = (p.total > 0 && (p.total & 7) == 0) ? (wg_linear & 7) * (p.total >> 3) + (wg_linear >> 3) : wg_linear;
+    int bh = wg_x / p.nq;
+    int qt = wg_x - bh * p.nq;
     if (CAUSAL) qt = p.nq - 1 - qt;
+    if (CAUSAL && p.lpt_heads > 0) {
+        qt = p.nq - 1 - wg_linear / p.lpt_heads;
+        bh = wg_linear % p.lpt_heads;
+    }
     const int b = bh / p.Hq, head = bh - b * p.Hq;
     const int N = p.N;
     const int qblk = qt * BQ;

@@ -103,3 +103,23 @@ def test_backward_rejects_what_it_does_not_cover(dev):
     with pytest.raises(_lib.ArhipError):
         dev.flash_bwd(x, x, x, x, None, x, x, x, x, x, 1, 1, 1, 8, 64)   # no lse
     x.free()
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_forward_and_backward_on_a_grid_of_many_workgroups(dev, causal):
+    """More than 16 workgroups per compute unit (5120 in the query grids, 2560 in the dK/dV grid with two query heads
+    per K/V head): the grids then run head by head with every eighth of them (one XCD's share) a contiguous range of
+    heads, instead of longest tile first over all heads.  Heads are independent, so a sample of them is checked
+    against the float64 oracle on their own slices."""
+    B, Hq, Hkv, N, D = 8, 80, 40, 1024, 64
+    q, k, v, do = (synth.normal(s, (B, H, N, D)) for s, H in ((81, Hq), (82, Hkv), (83, Hkv), (84, Hq)))
+    kv_len = np.array([N, 1000, 513, N, 77, N, 900, 1], np.int32)
+    got = run_fwd_bwd(dev, q, k, v, do, kv_len=kv_len, causal=causal)
+    for b, hk in ((0, 0), (1, 39), (2, 17), (4, 5), (7, 39), (7, 0)):
+        sl = (slice(b, b + 1), slice(2 * hk, 2 * hk + 2))
+        slk = (slice(b, b + 1), slice(hk, hk + 1))
+        want = oracle.attention_backward_f64(q[sl], k[slk], v[slk], do[sl], kv_len=kv_len[b:b + 1], causal=causal)
+        mine = (got[0][sl], got[1][sl], got[2][sl], got[3][slk], got[4][slk])
+        for name, g, w in zip(("o", "lse", "dq", "dk", "dv"), mine, want):
+            err = np.abs(g - w).max()
+            assert err <= 3e-5 * max(1.0, np.abs(w).max()), (b, hk, name, err)
