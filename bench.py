@@ -413,6 +413,8 @@ def build_workload(dev, name):
     # the shape the reference publishes its own kernel times on (B8 H6 N789 D64, PERFORMANCE.md:314-317)
     if name == "train_f32":   # the ViT-B/16 layer shape at batch 8, fp32 (the reference's training kernels are f32 only)
         return TrainWorkload(dev, 8, 12, 197, 64, False, cfg=8)
+    if name == "train_f32_causal":   # a decoder layer's shape, fp32, causal: forward with lse + backward
+        return TrainWorkload(dev, 2, 16, 2048, 128, True, cfg=9)
     if name == "ref_bf16":
         return FlashWorkload(dev, 8, 6, 789, 64, False, BF16, cfg=7)
     if name == "ref_f32":
@@ -434,7 +436,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="sage",
                     choices=["sage", "sage_causal_long", "vit", "decoder", "vit_f32", "flash_long", "ref_bf16",
-                             "ref_f32", "ref_sage", "train_f32", "sage_fp8"])
+                             "ref_f32", "ref_sage", "train_f32", "train_f32_causal", "sage_fp8"])
     ap.add_argument("--no-secondary", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="one step of the workload plus one plain 1 GiB copy kernel and nothing else: "
@@ -486,7 +488,7 @@ def main():
     secondary = []
     if not args.no_secondary:
         for name in ("vit", "decoder", "flash_long", "vit_f32", "sage", "sage_causal_long", "ref_bf16", "ref_f32",
-                     "ref_sage", "train_f32", "sage_fp8"):
+                     "ref_sage", "train_f32", "train_f32_causal", "sage_fp8"):
             if name == args.workload:
                 continue
             sw = build_workload(dev, name)
