@@ -37,6 +37,8 @@ struct FlashBwdParams {
     float scale;
 };
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
 constexpr float BWD_LSE_FLOOR = -5e29f;  // lse at or below: the row saw no key (cuda_flash_train.rs:206)
 constexpr float BWD_LOG2E = 1.44269504088896340736f;
 
@@ -324,33 +326,22 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
     const int qtiles = (N + F32_BK - 1) / F32_BK;
     const int steps = group * (qtiles - qt0);  // (head of the group, query tile) pairs, head-major
 
-    float4 qx[PER_THREAD], dx[PER_THREAD];
+    f32x4_t qx[PER_THREAD], dx[PER_THREAD];
     float st_l = 0.f, st_d = 0.f;
     auto fetch = [&](int step) __attribute__((always_inline)) {
         const int g = step / (qtiles - qt0);
         const int q0 = (qt0 + step - g * (qtiles - qt0)) * F32_BK;
         const size_t bh = (size_t)b * p.Hq + (size_t)kvh * group + g;
-        if (q0 + F32_BK <= N) {  // a full tile: no row tests, no zero fill
+        // Rows past the last query repeat it: whatever they hold is multiplied by P = dS = 0 (finite values, not
+        // zeros, are all that takes).  One path without a branch, and native vectors (typed loads and stores): both
+        // keep the staged tile in registers at D = 128.
 #pragma unroll
-            for (int j = 0; j < PER_THREAD; ++j) {
-                const int c = stid + j * T;
-                const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-                const size_t off = (bh * N + q0 + row) * D + col;
-                qx[j] = *(const float4 *)(p.q + off);
-                dx[j] = *(const float4 *)(p.dout + off);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < PER_THREAD; ++j) {
-                const int c = stid + j * T;
-                const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-                const int gr = q0 + row;
-                qx[j] = dx[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (gr < N) {
-                    qx[j] = *(const float4 *)(p.q + (bh * N + gr) * D + col);
-                    dx[j] = *(const float4 *)(p.dout + (bh * N + gr) * D + col);
-                }
-            }
+        for (int j = 0; j < PER_THREAD; ++j) {
+            const int c = stid + j * T;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            const size_t off = (bh * N + min(q0 + row, N - 1)) * D + col;
+            qx[j] = *(const f32x4_t *)(p.q + off);
+            dx[j] = *(const f32x4_t *)(p.dout + off);
         }
         if (stid < F32_BK) {
             const int gr = q0 + stid;
@@ -368,8 +359,8 @@ __device__ __forceinline__ void bwd_dkv_body(const FlashBwdParams &p, float *lds
         for (int j = 0; j < PER_THREAD; ++j) {
             const int c = stid + j * T;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-            *(float4 *)&qs[row * ROW + col] = qx[j];
-            *(float4 *)&dos[row * ROW + col] = dx[j];
+            *(f32x4_t *)&qs[row * ROW + col] = qx[j];
+            *(f32x4_t *)&dos[row * ROW + col] = dx[j];
         }
         if (stid < F32_BK) {
             stat[stid] = st_l * BWD_LOG2E;   // base-2 units: P = 2^(x log2(e) - lse log2(e))
