@@ -105,7 +105,7 @@ __device__ __forceinline__ void flash_f32_entry(float *lds, const float *Q, cons
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nq = (int)gridDim.x;
     p.total = (int)(gridDim.x * gridDim.y);
-    p.lpt_heads = (p.total <= 16 * 256) ? (int)gridDim.y : 0;  // few workgroups per compute unit: longest first over all heads
+    p.lpt_heads = (int)gridDim.y;  // causal: longest query tile first over all heads
     dense(p.qs, hq, N, head_dim);
     dense(p.ks, hkv, N, head_dim);
     dense(p.os, hq, N, head_dim);
@@ -149,7 +149,7 @@ extern "C" __global__ void __launch_bounds__(256) ar_fl_fwd(const float *Q, cons
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nq = (int)gridDim.x;
     p.total = (int)(gridDim.x * gridDim.y);
-    p.lpt_heads = (p.total <= 16 * 256) ? (int)gridDim.y : 0;  // few workgroups per compute unit: longest first over all heads
+    p.lpt_heads = (int)gridDim.y;  // causal: longest query tile first over all heads
     dense(p.qs, hq, N, head_dim);
     dense(p.ks, hkv, N, head_dim);
     dense(p.os, hq, N, head_dim);
@@ -178,7 +178,7 @@ __device__ __forceinline__ void flash_f32_short(const float *Q, const float *K, 
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nq = (int)gridDim.x;
     p.total = (int)(gridDim.x * gridDim.y);
-    p.lpt_heads = (p.total <= 16 * 256) ? (int)gridDim.y : 0;  // few workgroups per compute unit: longest first over all heads
+    p.lpt_heads = (int)gridDim.y;  // causal: longest query tile first over all heads
     dense(p.qs, hq, N, 64);
     dense(p.ks, hkv, N, 64);
     dense(p.os, hq, N, 64);
@@ -227,7 +227,7 @@ __device__ __forceinline__ FlashBwdParams bwd_params(const float *Q, const float
     p.Hq = hq; p.Hkv = hkv; p.N = N;
     p.nt = (int)gridDim.x;
     p.total_q = p.total_kv = (int)(gridDim.x * gridDim.y);
-    p.lpt_q = p.lpt_kv = (p.total_q <= 16 * 256) ? (int)gridDim.y : 0;  // few workgroups per compute unit: longest first over all heads
+    p.lpt_q = p.lpt_kv = (int)gridDim.y;  // causal: longest tile first over all heads
     p.scale = 1.0f / __builtin_sqrtf((float)head_dim);
     return p;
 }

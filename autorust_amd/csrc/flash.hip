@@ -187,7 +187,7 @@ extern "C" int arhip_flash_fwd_lse(arhip_device *dev, const void *q, const void 
         fp.scale = scale;
         const int64_t wgs = fp.nq * B * Hq;
         fp.total = (int)wgs;
-        fp.lpt_heads = (causal && wgs <= 16 * (int64_t)dev->cus) ? (int)(B * Hq) : 0;
+        fp.lpt_heads = causal ? (int)(B * Hq) : 0;  // causal: longest query tile first over all heads
         const bool two = splitk && D == 64 && wgs > 2 * (int64_t)dev->cus && wgs <= 4 * (int64_t)dev->cus;
         if (int rc = t.begin()) return rc;
         const dim3 grid((unsigned)wgs), block(two ? 128 : 256);
@@ -523,11 +523,11 @@ extern "C" int arhip_flash_bwd(arhip_device *dev, const float *q, const float *k
     const dim3 block(256), grid_prep((unsigned)((rows + 3) / 4)), grid_q((unsigned)(nt * B * Hq)),
         grid_kv((unsigned)(nt * B * Hkv));
     p.nt = nt;
-    // causal, few workgroups per compute unit: longest tile first over all heads, so that no head's long tiles are left for the end
+    // causal: longest tile first over all heads, so that no head's long tiles are left for the end
     p.total_q = (int)(nt * B * Hq);
     p.total_kv = (int)(nt * B * Hkv);
-    p.lpt_q = (causal && (int64_t)nt * B * Hq <= 16 * (int64_t)dev->cus) ? (int)(B * Hq) : 0;
-    p.lpt_kv = (causal && (int64_t)nt * B * Hkv <= 16 * (int64_t)dev->cus) ? (int)(B * Hkv) : 0;
+    p.lpt_q = causal ? (int)(B * Hq) : 0;
+    p.lpt_kv = causal ? (int)(B * Hkv) : 0;
 #define BWD_LAUNCH(DD, SP)                                                                              \
     do {                                                                                                \
         hipLaunchKernelGGL((bwd_prep_kernel<DD>), grid_prep, dim3(256), 0, dev->stream, o, dout, delta, rows); \

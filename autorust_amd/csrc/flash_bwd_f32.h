@@ -33,7 +33,7 @@ struct FlashBwdParams {
     int Hq, Hkv, N;
     int nt;  // tiles per head: query tiles (dQ kernel) or key tiles (dK/dV kernel)
     int total_q, total_kv;  // workgroups in the dQ grid (nt * B * Hq) and in the dK/dV grid (nt * B * Hkv)
-    int lpt_q, lpt_kv;  // causal, few workgroups per compute unit: B * Hq / B * Hkv, and the grids run longest tile first over all heads; else 0
+    int lpt_q, lpt_kv;  // causal: B * Hq / B * Hkv, and the grids run longest tile first over all heads; else 0
     float scale;
 };
 

@@ -35,7 +35,7 @@ struct FlashF32Params {
     const int32_t *kv_len;  // [B] or null
     float *lse;             // optional [B,Hq,N]: m + log(l), src/runtime/cuda_flash_train.rs:141
     int Hq, Hkv, N, nq;
-    int lpt_heads;  // causal, few workgroups per compute unit: B * Hq, and the grid runs longest query tile first over all heads; else 0
+    int lpt_heads;  // causal: B * Hq, and the grid runs longest query tile first over all heads; else 0
     int total;      // workgroups in the grid (nq * B * Hq)
     long qs[3], ks[3], os[3];  // element strides [batch, head, token] of q / k,v / o (channel stride 1)
     float scale;
@@ -75,8 +75,8 @@ __device__ __forceinline__ void flash_f32_body(const FlashF32Params &p, float *l
     float *vs = ks + F32_BK * KROW;                // [F32_BK][D]
     const int stid = SPLITK ? lane : tid;          // index among the threads staging a tile
     const int i32 = lane & 31, h = lane >> 5;
-    // causal: the longest query tiles first, within a head or (few, very unequal workgroups per compute unit) over
-    // the whole grid, so that no head's long tiles are left for the end
+    // causal: the longest query tiles first over the whole grid, so that no head's long tiles are left for the end
+    // (these kernels are bound by the matrix pipe at any grid size: every workgroup may stream its own K/V)
     // Consecutive workgroups go to different XCDs (8, each with its own L2): every XCD gets a contiguous range of
     // heads, so that the query tiles sharing a head's K/V meet in one L2 and, under the causal mask, every XCD gets
     // tiles of every length.

@@ -107,10 +107,10 @@ def test_backward_rejects_what_it_does_not_cover(dev):
 
 @pytest.mark.parametrize("causal", [False, True])
 def test_forward_and_backward_on_a_grid_of_many_workgroups(dev, causal):
-    """More than 16 workgroups per compute unit (5120 in the query grids, 2560 in the dK/dV grid with two query heads
-    per K/V head): the grids then run head by head with every eighth of them (one XCD's share) a contiguous range of
-    heads, instead of longest tile first over all heads.  Heads are independent, so a sample of them is checked
-    against the float64 oracle on their own slices."""
+    """Large grids (5120 workgroups in the query grids, 2560 in the dK/dV grid with two query heads per K/V head) in
+    both orders the fp32 kernels use: head by head with every eighth of the grid (one XCD's share) a contiguous range
+    of heads, and, under the causal mask, longest tile first over all heads.  Heads are independent, so a sample of
+    them is checked against the float64 oracle on their own slices."""
     B, Hq, Hkv, N, D = 8, 80, 40, 1024, 64
     q, k, v, do = (synth.normal(s, (B, H, N, D)) for s, H in ((81, Hq), (82, Hkv), (83, Hkv), (84, Hq)))
     kv_len = np.array([N, 1000, 513, N, 77, N, 900, 1], np.int32)
