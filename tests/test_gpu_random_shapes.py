@@ -97,3 +97,38 @@ def _sage_random_shapes(dev):
             # seeds: 8e-3
             bound = 2.0 ** -8 * float(np.abs(v).max())
             assert np.isfinite(r["out"]).all() and err < bound, (B, Hq, Hkv, N, D, causal, bq, bk, err, bound)
+
+
+@pytest.mark.parametrize("waves", [None, "8", "40"])
+def test_in_kernel_q_quantiser_random_shapes(dev, waves, monkeypatch):
+    """The attention entries that quantise their queries in the prologue (bf16 blocks of 128, int8 and FP8; f32 rows)
+    on the random shapes, with the 8- and the 4-wave form forced: scales, codes and output bit for bit those of the
+    quantiser launch followed by the plain entry."""
+    from gpu_util import Bufs
+    with _device_with_waves(dev, waves, monkeypatch) as d:
+        for (B, Hq, Hkv, N, D, causal, kv_len, seed) in _cases(9876, 10):
+            q, k, v = (synth.normal(seed + i, s) for i, s in enumerate(((B, Hq, N, D), (B, Hkv, N, D), (B, Hkv, N, D))))
+            qb, kb = oracle.bf16_round(q), oracle.bf16_round(k)
+            case = (B, Hq, Hkv, N, D, causal, None if kv_len is None else kv_len.tolist())
+            # bf16 queries, blocks of 128: int8
+            r = run_sage(d, qb, kb, v, 128, 64, smooth=True, in_dtype=BF16, out_dtype=BF16, kv_len=kv_len, causal=causal)
+            # f32 queries, a scale per query and per key
+            rr = run_sage(d, q, k, v, 1, 1, smooth=False, kv_len=kv_len, causal=causal)
+            with Bufs(d) as bufs:
+                dl = bufs.put(kv_len) if kv_len is not None else None
+                dv = bufs.put(synth.to_bf16_bits(v))
+                nqb = (N + 127) // 128
+                dq = bufs.put(synth.to_bf16_bits(qb))
+                k8, sk = bufs.put(r["k8"]), bufs.put(r["sk"])
+                do, sq_out, q8_out = bufs.new(q.size * 2), bufs.new(B * Hq * nqb * 4), bufs.new(q.size)
+                d.sage_fwd_qfused(dq, k8, sk, dv, do, B, Hq, Hkv, N, D, 64, out_dtype=BF16, sq_out=sq_out, q8_out=q8_out,
+                                  kv_len=dl, causal=causal)
+                assert np.array_equal(sq_out.copyout(np.float32, (B, Hq, nqb)), r["sq"]), case
+                assert np.array_equal(q8_out.copyout(np.int8, q.shape), r["q8"]), case
+                assert np.array_equal(synth.from_bf16_bits(do.copyout(np.uint16, q.shape)), r["out"]), case
+                dqf = bufs.put(q)
+                k8r, skr = bufs.put(rr["k8"]), bufs.put(rr["sk"])
+                dor, sqr = bufs.new(q.size * 4), bufs.new(B * Hq * N * 4)
+                d.sage_fwd_qfused_rows(dqf, k8r, skr, dv, dor, B, Hq, Hkv, N, D, 1, sq_out=sqr, kv_len=dl, causal=causal)
+                assert np.array_equal(sqr.copyout(np.float32, (B, Hq, N)), rr["sq"]), case
+                assert np.array_equal(dor.copyout(np.float32, q.shape), rr["out"]), case
