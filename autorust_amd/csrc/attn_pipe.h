@@ -692,11 +692,12 @@ __device__ __forceinline__ void attn_pipe_impl(const AttnParams &p, unsigned cha
     };
 
     // ---- prologue: tiles 0..2 on their way, tiles 0 and 1 visible ----
-    // Tiles [0, nfull) have no masked key for ANY wave of the workgroup (all full tiles; under the
-    // causal mask those before the workgroup's first query); the remaining ones (at most 4 on the
-    // causal diagonal, or the last partial one) run the same pipeline with the mask applied inside
-    // the softmax.  Every wave runs every tile, so all waves execute the same code between barriers.
-    const int nfull = CAUSAL ? min(kend / BK, qblk / BK) : kend / BK;
+    // Tiles [0, nfull) have no masked key for this wave (all full tiles; under the causal mask those
+    // before the wave's first query); the remaining ones (the one on the wave's causal diagonal, or the
+    // last partial one) run the same pipeline with the mask applied inside the softmax.  Every wave
+    // passes one barrier per tile and requests its share of every tile's transfers, whichever form of
+    // the tile it runs.
+    const int nfull = CAUSAL ? min(kend / BK, wq0 / BK) : kend / BK;
     static_for<0, AHEAD>([&](auto ti) __attribute__((always_inline)) { issue_tile(decltype(ti)::value); });
     // Q operand, resident in registers.  Everything in flight is awaited here once, Q included, so
     // that no wait for a global load is left inside the loops.
